@@ -1,0 +1,58 @@
+// Shared definitions for the gfx950 quantized-MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#define DMQ_GS 128            // quantization group: 128 consecutive input features
+#define DMQ_WAVE 64
+
+// status codes, precision modes and epilogue kinds come from the public C header
+#include "dartmoq_hip.h"
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+typedef int int8_t8 __attribute__((ext_vector_type(8)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+static inline int dmq_check_launch() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? DMQ_OK : DMQ_ERR_HIP;
+}
+
+static inline bool dmq_valid_bit(int bit) { return bit == 1 || bit == 2 || bit == 4; }
+
+// ---------------------------------------------------------------- device helpers
+__device__ __forceinline__ float dmq_silu(float x) { return x / (1.0f + __expf(-x)); }
+
+// OCP e4m3fn encode of a finite fp32 already clamped to [-448, 448]; round to nearest even.
+__device__ __forceinline__ uint32_t dmq_f32_to_e4m3(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t sign = (u >> 24) & 0x80u;
+  uint32_t a = u & 0x7fffffffu;
+  float af = __uint_as_float(a);
+  uint32_t r;
+  if (af >= 0.015625f) {                       // normal e4m3 range: 2^-6 ..
+    // keep 3 mantissa bits: add half-ulp with tie-to-even on bit 20
+    uint32_t lsb = (a >> 20) & 1u;
+    a += 0x7ffffu + lsb;
+    uint32_t e = (a >> 23) - 127u + 7u;        // rebias 127 -> 7
+    r = (e << 3) | ((a >> 20) & 7u);
+    if (r > 0x7eu) r = 0x7eu;                  // 448 is the largest finite code
+  } else {
+    // subnormals: multiples of 2^-9; rintf rounds half to even
+    r = (uint32_t)rintf(af * 512.0f);          // 0..8 (8 == smallest normal 0x08)
+  }
+  return sign | r;
+}
+
+// e2m1 magnitude index of |y| (y already clamped to [0, 6]); ties go to the smaller magnitude.
+__device__ __forceinline__ uint32_t dmq_e2m1_mag(float ay) {
+  return (uint32_t)(ay > 0.25f) + (uint32_t)(ay > 0.75f) + (uint32_t)(ay > 1.25f) +
+         (uint32_t)(ay > 1.75f) + (uint32_t)(ay > 2.5f) + (uint32_t)(ay > 3.5f) +
+         (uint32_t)(ay > 5.0f);
+}

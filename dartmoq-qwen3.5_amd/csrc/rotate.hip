@@ -1,0 +1,266 @@
+// Block-QR rotation of activations, optionally fused with per-token quantization.
+//
+//   y[r, g*128 + j] = sum_k x[r, g*128 + k] * P_g[j, k]          (fp32 accumulation on MFMA)
+//
+// followed, in registers, by one of
+//   fp16 store                                    (WxA16)
+//   per-(row, group) symmetric int8 + fp16 scale  (WxA8)
+//   per-(row, group) e4m3 + fp16 scale            (WxFP8)
+//   per-32 e2m1 + e8m0 scale byte                 (WxFP4)
+// so the rotated activation never reaches HBM in fp32/fp16 form for the quantized modes.
+//
+// One wave handles one (tile of 16*TT rows, group): the rotation matrix rows are the MFMA
+// "A" operand, activation rows the "B" operand, so lane (t = lane % 16, q = lane / 16) ends
+// up with the 32 rotated values j = 16*jt + 4q + r (jt < 8, r < 4) of row t; the row maximum
+// is a 32-value in-lane reduction plus two cross-lane steps.
+#include "params.h"
+
+
+__device__ __forceinline__ float wave_max16x4(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  v = fmaxf(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+template <int MODE, int TT>
+__global__ __launch_bounds__(256)
+void dmq_rotate_kernel(RotParams p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int l16 = lane & 15;
+  const int q = lane >> 4;
+  constexpr int ROWS_PER_ITEM = 16 * TT;
+
+  long item = (long)blockIdx.x * 4 + wave;
+  const int g = (int)(item % p.groups);
+  const long rt = item / p.groups;
+
+  int r_first, r_end, rot_g;
+  if (p.tiles) {
+    const int sub = p.tile_rows / ROWS_PER_ITEM;          // items per tile entry
+    const long tile = rt / sub;
+    if (tile >= p.n_tiles[0]) return;
+    const int eidx = p.tiles[2 * tile];
+    const int ttile = p.tiles[2 * tile + 1];
+    const int ts = p.expert_info[4 * eidx + 0];
+    const int tc = p.expert_info[4 * eidx + 1];
+    r_first = ts + ttile * p.tile_rows + (int)(rt % sub) * ROWS_PER_ITEM;
+    r_end = ts + tc;
+    rot_g = (p.rot_use_slice ? p.expert_info[4 * eidx + 2] : 0) + g;
+  } else {
+    r_first = (int)rt * ROWS_PER_ITEM;
+    r_end = p.rows;
+    rot_g = g;
+  }
+  if (r_first >= r_end) return;
+
+  int rlog[TT];
+  bool valid[TT];
+  const __half* xrow[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    rlog[t] = r_first + t * 16 + l16;
+    valid[t] = rlog[t] < r_end;
+    int phys = valid[t] ? (p.row_index ? p.row_index[rlog[t]] : rlog[t]) : 0;
+    xrow[t] = p.x + (long)phys * p.x_stride + g * DMQ_GS + 8 * q;
+  }
+  const __half* prow = p.rot + (long)rot_g * (DMQ_GS * DMQ_GS) + (long)l16 * DMQ_GS + 8 * q;
+
+  float4_t acc[8][TT];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int t = 0; t < TT; ++t) acc[j][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    half8_t b[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      uint4_t raw = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
+      b[t] = __builtin_bit_cast(half8_t, raw);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      half8_t a = __builtin_bit_cast(half8_t, *(const uint4_t*)(prow + (long)j * 16 * DMQ_GS + 32 * s));
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+        acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[j][t], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    uint8_t* orow = p.out + (long)rlog[t] * p.out_row_bytes;
+    if (MODE == DMQ_MODE_A16) {
+      if (!valid[t]) continue;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        half4_t h = {(_Float16)acc[j][t][0], (_Float16)acc[j][t][1], (_Float16)acc[j][t][2],
+                     (_Float16)acc[j][t][3]};
+        *(half4_t*)(orow + (g * DMQ_GS + j * 16 + 4 * q) * 2) = h;
+      }
+    } else if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
+      float amax = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) amax = fmaxf(amax, fabsf(acc[j][t][r]));
+      amax = wave_max16x4(amax);
+      const float qmax = (MODE == DMQ_MODE_A8) ? 127.0f : 448.0f;
+      const float sc = fmaxf(__fdiv_rn(amax, qmax), 1e-8f);
+      if (!valid[t]) continue;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float y = __fdiv_rn(acc[j][t][r], sc);
+          uint32_t code;
+          if (MODE == DMQ_MODE_A8) {
+            y = fminf(fmaxf(rintf(y), -127.f), 127.f);
+            code = (uint32_t)(int)y & 0xffu;
+          } else {
+            y = fminf(fmaxf(y, -448.f), 448.f);
+            code = dmq_f32_to_e4m3(y);
+          }
+          word |= code << (8 * r);
+        }
+        *(uint32_t*)(orow + g * DMQ_GS + j * 16 + 4 * q) = word;
+      }
+      if (q == 0) {
+        const float stored = sc * p.extra_scale;
+        if (p.scale_fp32) ((float*)p.scale)[(long)rlog[t] * p.scale_stride + g] = stored;
+        else ((__half*)p.scale)[(long)rlog[t] * p.scale_stride + g] = __float2half_rn(stored);
+      }
+    } else {   // FP4: four MX blocks of 32 per group
+      uint32_t sbytes = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        float amax = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) amax = fmaxf(amax, fabsf(acc[2 * b + jj][t][r]));
+        amax = fmaxf(wave_max16x4(amax), 1e-30f);
+        const float z = __fdiv_rn(amax, 6.0f);
+        float e = ceilf((float)log2((double)z));
+        const float s = fmaxf(exp2f(e), 1e-30f);
+        float eb = fminf(fmaxf(e + 127.0f, 0.f), 254.f);
+        sbytes |= ((uint32_t)eb & 0xffu) << (8 * b);
+        if (valid[t]) {
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            uint32_t half_word = 0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float y = fminf(fmaxf(__fdiv_rn(acc[2 * b + jj][t][r], s), -6.f), 6.f);
+              uint32_t nib = dmq_e2m1_mag(fabsf(y)) | ((y < 0.f) ? 8u : 0u);
+              half_word |= nib << (4 * r);
+            }
+            *(uint16_t*)(orow + (g * DMQ_GS + (2 * b + jj) * 16 + 4 * q) / 2) = (uint16_t)half_word;
+          }
+        }
+      }
+      if (valid[t] && q == 0)
+        *(uint32_t*)((uint8_t*)p.scale + (long)rlog[t] * p.scale_stride + g * 4) = sbytes;
+    }
+  }
+}
+
+// --------------------------------------------------------------------------------------------
+// Quantization of activations that are already rotated (no matrix product): one wave per
+// (row, group), two consecutive features per lane.
+
+template <int MODE>
+__global__ __launch_bounds__(256)
+void dmq_quantize_kernel(QuantParams p) {
+  const int lane = threadIdx.x & 63;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long)p.rows * p.groups) return;
+  const int g = (int)(item % p.groups);
+  const long r = item / p.groups;
+  const long col = (long)g * DMQ_GS + 2 * lane;
+  float v0, v1;
+  if (p.x_fp32) {
+    const float* xr = (const float*)p.x + r * p.x_stride + col;
+    v0 = xr[0]; v1 = xr[1];
+  } else {
+    const __half* xr = (const __half*)p.x + r * p.x_stride + col;
+    v0 = __half2float(xr[0]); v1 = __half2float(xr[1]);
+  }
+  float amax = fmaxf(fabsf(v0), fabsf(v1));
+  uint8_t* orow = p.out + r * p.out_row_bytes;
+  if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    const float qmax = (MODE == DMQ_MODE_A8) ? 127.0f : 448.0f;
+    const float sc = fmaxf(__fdiv_rn(amax, qmax), 1e-8f);
+    float y0 = __fdiv_rn(v0, sc), y1 = __fdiv_rn(v1, sc);
+    uint32_t c0, c1;
+    if (MODE == DMQ_MODE_A8) {
+      c0 = (uint32_t)(int)fminf(fmaxf(rintf(y0), -127.f), 127.f) & 0xffu;
+      c1 = (uint32_t)(int)fminf(fmaxf(rintf(y1), -127.f), 127.f) & 0xffu;
+    } else {
+      c0 = dmq_f32_to_e4m3(fminf(fmaxf(y0, -448.f), 448.f));
+      c1 = dmq_f32_to_e4m3(fminf(fmaxf(y1, -448.f), 448.f));
+    }
+    *(uint16_t*)(orow + col) = (uint16_t)(c0 | (c1 << 8));
+    if (lane == 0) {
+      const float stored = sc * p.extra_scale;
+      if (p.scale_fp32) ((float*)p.scale)[r * p.scale_stride + g] = stored;
+      else ((__half*)p.scale)[r * p.scale_stride + g] = __float2half_rn(stored);
+    }
+  } else {   // FP4: a block of 32 features is 16 consecutive lanes
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    amax = fmaxf(amax, 1e-30f);
+    const float z = __fdiv_rn(amax, 6.0f);
+    const float e = ceilf((float)log2((double)z));
+    const float s = fmaxf(exp2f(e), 1e-30f);
+    float y0 = fminf(fmaxf(__fdiv_rn(v0, s), -6.f), 6.f);
+    float y1 = fminf(fmaxf(__fdiv_rn(v1, s), -6.f), 6.f);
+    uint32_t n0 = dmq_e2m1_mag(fabsf(y0)) | ((y0 < 0.f) ? 8u : 0u);
+    uint32_t n1 = dmq_e2m1_mag(fabsf(y1)) | ((y1 < 0.f) ? 8u : 0u);
+    orow[col / 2] = (uint8_t)(n0 | (n1 << 4));
+    if ((lane & 15) == 0)
+      ((uint8_t*)p.scale)[r * p.scale_stride + g * 4 + (lane >> 4)] =
+          (uint8_t)fminf(fmaxf(e + 127.0f, 0.f), 254.f);
+  }
+}
+
+// --------------------------------------------------------------------------------------------
+template <int MODE>
+static int launch_rotate(const RotParams& p, long items, int tt, hipStream_t stream) {
+  const int grid = (int)((items + 3) / 4);
+  if (grid <= 0) return DMQ_OK;
+  if (tt == 4) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 4>), dim3(grid), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 1>), dim3(grid), dim3(256), 0, stream, p);
+  return dmq_check_launch();
+}
+
+int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream) {
+  switch (mode) {
+    case DMQ_MODE_A16: return launch_rotate<DMQ_MODE_A16>(p, items, tt, stream);
+    case DMQ_MODE_A8: return launch_rotate<DMQ_MODE_A8>(p, items, tt, stream);
+    case DMQ_MODE_FP8: return launch_rotate<DMQ_MODE_FP8>(p, items, tt, stream);
+    case DMQ_MODE_FP4: return launch_rotate<DMQ_MODE_FP4>(p, items, tt, stream);
+  }
+  return DMQ_ERR_MODE;
+}
+
+int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream) {
+  const long items = (long)p.rows * p.groups;
+  const int grid = (int)((items + 3) / 4);
+  if (grid <= 0) return DMQ_OK;
+  switch (mode) {
+    case DMQ_MODE_A8:
+      hipLaunchKernelGGL((dmq_quantize_kernel<DMQ_MODE_A8>), dim3(grid), dim3(256), 0, stream, p); break;
+    case DMQ_MODE_FP8:
+      hipLaunchKernelGGL((dmq_quantize_kernel<DMQ_MODE_FP8>), dim3(grid), dim3(256), 0, stream, p); break;
+    case DMQ_MODE_FP4:
+      hipLaunchKernelGGL((dmq_quantize_kernel<DMQ_MODE_FP4>), dim3(grid), dim3(256), 0, stream, p); break;
+    default: return DMQ_ERR_MODE;
+  }
+  return dmq_check_launch();
+}

@@ -1,0 +1,280 @@
+"""Bit-partitioned quantized MoE FFN layer on MI355X.
+
+Host-side mirror of WxA16BitPartitionedGroupMoE and its WxA8 / WxFP8 / WxFP4 subclasses
+(quantization/{wxa16,wxa8,wxfp8,wxfp4}/bit_partitioned_moe.py of the reference).  The module
+keeps the checkpoint tensors of the reference format (per bit pool: packed indices, fp16
+norms, fp16 codebook for gate_up [2*I*E_pool, H] and down [H, I*E_pool] plus cumulative
+``expert_offsets``), derives the runtime layout once (group-first indices, norms divided by
+sqrt(128), resident rotation matrices, per-mode look-up tables) and runs the whole routed
+forward through one C call that allocates nothing and never synchronizes with the host.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import hostprep, ops
+from ._lib import (MODE_A16, MODE_A8, MODE_BY_NAME, MODE_FP4, MODE_FP8, LayerDesc, PoolDesc, check,
+                   load)
+
+GROUP_SIZE = 128
+
+
+class BitPoolWeights:
+    """Runtime form of one bit pool (the reference's WxA16Weights, :32-265, after
+    _build_group_first :177-233 and the subclasses' _get_bit_context)."""
+
+    def __init__(self, bit: int, gate_up: dict, down: dict, expert_offsets, device):
+        self.bit = int(bit)
+        self.expert_offsets = [int(v) for v in expert_offsets]
+        self.gate_up_meta = {k: v for k, v in gate_up.items() if not torch.is_tensor(v)}
+        self.down_meta = {k: v for k, v in down.items() if not torch.is_tensor(v)}
+        gs = int(gate_up["group_size"])
+        if gs != GROUP_SIZE or int(down["group_size"]) != GROUP_SIZE:
+            raise ValueError(f"group_size must be {GROUP_SIZE}")
+        self.gu_codebook = gate_up["codebook"].to(device, torch.float16).contiguous()
+        self.dn_codebook = down["codebook"].to(device, torch.float16).contiguous()
+        # group-first relayout + norms / sqrt(gs) on the GPU; row-major originals are not kept
+        self.gu_idx, self.gu_norms = ops.convert_to_group_first(
+            gate_up["indices_packed"].to(device), gate_up["norms"].to(device), gs, bit, prescale=True)
+        self.dn_idx, self.dn_norms = ops.convert_to_group_first(
+            down["indices_packed"].to(device), down["norms"].to(device), gs, bit, prescale=True)
+        self.n_gate_up, self.hidden = gate_up["shape"]
+        self.down_in = down["shape"][1]
+        # resident rotations: gate_up [H/gs, gs, gs]; down one matrix per global group,
+        # seed = down_seed + j*gs  (== seed + original_start + g*gs, triton_kernels.py:1310)
+        self.gu_rot = hostprep.generate_batch_rotation_matrices(
+            gs, int(gate_up["seed"]), self.hidden // gs, gs, device)
+        self.dn_rot = hostprep.generate_batch_rotation_matrices(
+            gs, int(down["seed"]), self.down_in // gs, gs, device)
+        self._mode_ctx: dict[int, dict] = {}
+
+    def context(self, mode: int) -> dict:
+        """Per-mode look-up tables and scale constants, built on first use."""
+        ctx = self._mode_ctx.get(mode)
+        if ctx is not None:
+            return ctx
+        dev = self.gu_idx.device
+        ctx = {"gu_w": self.gu_idx, "dn_w": self.dn_idx, "gu_norms": self.gu_norms,
+               "dn_norms": self.dn_norms, "gu_extra": 1.0, "dn_extra": 1.0, "gu_wsb": 127,
+               "dn_wsb": 127}
+        if mode == MODE_A16:
+            ctx["gu_lut"], ctx["dn_lut"] = self.gu_codebook, self.dn_codebook
+        elif mode == MODE_A8:
+            gq, gstep = hostprep.build_int8_codebook(self.gu_codebook)
+            dq, dstep = hostprep.build_int8_codebook(self.dn_codebook)
+            ctx.update(gu_lut=gq.to(dev), dn_lut=dq.to(dev), gu_extra=gstep, dn_extra=dstep)
+        elif mode == MODE_FP8:
+            gq, gs_ = hostprep.build_fp8_codebook(self.gu_codebook)
+            dq, ds_ = hostprep.build_fp8_codebook(self.dn_codebook)
+            ctx.update(gu_lut=gq.to(dev), dn_lut=dq.to(dev), gu_extra=gs_, dn_extra=ds_)
+        elif mode == MODE_FP4:
+            # cb ~= e2m1(nib) * 2^E0 * residual: 2^E0 rides the weight e8m0 byte, the residual is
+            # folded into a copy of the norms (wxfp4/bit_partitioned_moe.py:94-100), indices are
+            # folded to packed e2m1 once (fold_indices_to_e2m1, triton_kernels_fp4.py:80-122)
+            gn, ge0, gres, _ = hostprep.build_e2m1_codebook(self.gu_codebook)
+            dn, de0, dres, _ = hostprep.build_e2m1_codebook(self.dn_codebook)
+            ctx.update(
+                gu_lut=None, dn_lut=None, gu_nib=gn.to(dev), dn_nib=dn.to(dev),
+                gu_wsb=127 + ge0, dn_wsb=127 + de0,
+                gu_norms=(self.gu_norms.float() * gres).half().contiguous(),
+                dn_norms=(self.dn_norms.float() * dres).half().contiguous(),
+                gu_w=ops.fold_indices_to_e2m1(self.gu_idx, gn, self.bit),
+                dn_w=ops.fold_indices_to_e2m1(self.dn_idx, dn, self.bit))
+        else:
+            raise ValueError(f"unknown mode {mode}")
+        self._mode_ctx[mode] = ctx
+        return ctx
+
+
+class WxA16BitPartitionedGroupMoE:
+    """Quantized MoE layer; ``forward(hidden_states)`` returns the routed-expert sum.
+
+    Mirrors the constructor fields and ``forward`` contract of the reference class
+    (quantization/wxa16/bit_partitioned_moe.py:268-318, :1059-1224).
+    """
+
+    MODE = "wxa16"
+    rotation_hoist_threshold = 1.5
+
+    def __init__(self, num_experts: int, hidden_size: int, intermediate_size: int, top_k: int,
+                 gate_weight: torch.Tensor | None = None, renormalize: bool = False, device="cuda"):
+        self.num_experts = num_experts
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.top_k = top_k
+        self.device = torch.device(device)
+        self.gate_weight = None if gate_weight is None else gate_weight.to(self.device)
+        self.renormalize = renormalize
+        self.bit_weights: dict[str, BitPoolWeights] = {}
+        self.expert_offsets: dict[str, list] = {}
+        self.bit_list: list[int] = []
+        self._desc = None
+        self._workspace = None
+        self.tt_override = 0
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_packed(cls, pools: dict, num_experts: int, hidden_size: int, intermediate_size: int,
+                    top_k: int, gate_weight=None, renormalize=False, device="cuda"):
+        """pools: {bit_str: {"gate_up": packed, "down": packed, "expert_offsets": [E+1]}} in
+        processing order (the ModuleDict order of the reference)."""
+        moe = cls(num_experts, hidden_size, intermediate_size, top_k, gate_weight, renormalize, device)
+        for bit_str, p in pools.items():
+            bit = int(bit_str)
+            if bit not in (1, 2, 4):
+                raise ValueError(f"bit_width must be 1/2/4, got {bit}")
+            offs = [int(v) for v in p["expert_offsets"]]
+            if len(offs) != num_experts + 1:
+                raise ValueError("expert_offsets must have num_experts + 1 entries")
+            widths = {b - a for a, b in zip(offs[:-1], offs[1:]) if b > a}
+            if widths and widths != {intermediate_size}:
+                raise ValueError(f"every member of a pool must own {intermediate_size} neurons, "
+                                 f"got widths {sorted(widths)}")
+            moe.bit_weights[bit_str] = BitPoolWeights(bit, p["gate_up"], p["down"], offs, moe.device)
+            moe.expert_offsets[bit_str] = offs
+            moe.bit_list.append(bit)
+        return moe
+
+    @classmethod
+    def from_wxa16(cls, moe: "WxA16BitPartitionedGroupMoE"):
+        """Switch an already loaded layer to this precision mode in place (no tensor copies),
+        like WxA8BitPartitionedGroupMoE.from_wxa16 (wxa8/bit_partitioned_moe.py:47-61)."""
+        if not isinstance(moe, WxA16BitPartitionedGroupMoE):
+            raise TypeError(f"expected WxA16BitPartitionedGroupMoE, got {type(moe)}")
+        moe.__class__ = cls
+        moe._desc = None
+        return moe
+
+    # ------------------------------------------------------------------ descriptors
+    def pool_mode(self, bit: int) -> int:
+        mode = MODE_BY_NAME[self.MODE]
+        if mode == MODE_FP4 and bit not in hostprep.FP4_BITS:
+            return MODE_A8                      # wxfp4/bit_partitioned_moe.py:50,296-299
+        return mode
+
+    def _descriptor(self):
+        if self._desc is not None:
+            return self._desc
+        e = self.num_experts
+        n_pools = len(self.bit_weights)
+        start = torch.full((n_pools, e), -1, dtype=torch.int32)
+        count = torch.zeros((n_pools, e), dtype=torch.int32)
+        pool_arr = (PoolDesc * n_pools)()
+        keep = []
+        for pi, (bit_str, bw) in enumerate(self.bit_weights.items()):
+            members = 0
+            for ex in range(e):
+                s, t = bw.expert_offsets[ex], bw.expert_offsets[ex + 1]
+                if t > s:
+                    start[pi, ex] = 2 * s
+                    count[pi, ex] = 2 * (t - s)
+                    members += 1
+            mode = self.pool_mode(bw.bit)
+            ctx = bw.context(mode)
+            keep.append(ctx)
+            d = pool_arr[pi]
+            d.bit, d.mode = bw.bit, mode
+            # expected routed rows of the pool exceed threshold * T  <=>  share * top_k > threshold
+            d.major = int(members * self.top_k > self.rotation_hoist_threshold * e)
+            d.n_gate_up, d.down_groups = bw.n_gate_up, bw.down_in // GROUP_SIZE
+            d.gu_w, d.gu_norms = ctx["gu_w"].data_ptr(), ctx["gu_norms"].data_ptr()
+            d.gu_lut = ctx["gu_lut"].data_ptr() if ctx["gu_lut"] is not None else None
+            d.gu_rot = bw.gu_rot.data_ptr()
+            d.gu_extra_scale, d.gu_w_scale_byte = ctx["gu_extra"], ctx["gu_wsb"]
+            d.dn_w, d.dn_norms = ctx["dn_w"].data_ptr(), ctx["dn_norms"].data_ptr()
+            d.dn_lut = ctx["dn_lut"].data_ptr() if ctx["dn_lut"] is not None else None
+            d.dn_rot = bw.dn_rot.data_ptr()
+            d.dn_extra_scale, d.dn_w_scale_byte = ctx["dn_extra"], ctx["dn_wsb"]
+        slice_start = start.to(self.device)
+        slice_count = count.to(self.device)
+        desc = LayerDesc()
+        desc.hidden, desc.inter = self.hidden_size, self.intermediate_size
+        desc.experts, desc.top_k, desc.pools = e, self.top_k, n_pools
+        desc.pool = ctypes.cast(pool_arr, ctypes.POINTER(PoolDesc))
+        desc.slice_start, desc.slice_count = slice_start.data_ptr(), slice_count.data_ptr()
+        self._desc = (desc, pool_arr, slice_start, slice_count, keep)
+        return self._desc
+
+    def _get_workspace(self, tokens: int) -> torch.Tensor:
+        desc = self._descriptor()[0]
+        need = load().dmq_moe_workspace_bytes(ctypes.byref(desc), tokens)
+        if self._workspace is None or self._workspace.numel() < need:
+            self._workspace = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self._workspace
+
+    # ------------------------------------------------------------------ forward
+    def route(self, x: torch.Tensor, router_logits: torch.Tensor | None = None):
+        """softmax -> top-k (bit_partitioned_moe.py:1112-1120); logits default to x @ W_g^T."""
+        if router_logits is None:
+            if self.gate_weight is None:
+                raise ValueError("no gate weight: pass router_logits or topk_idx/topk_w")
+            router_logits = torch.matmul(x, self.gate_weight.t().to(x.dtype))
+        return ops.route_topk(router_logits, self.top_k, self.renormalize)
+
+    @torch.no_grad()
+    def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None,
+                topk_idx: torch.Tensor | None = None, topk_w: torch.Tensor | None = None,
+                residual: torch.Tensor | None = None) -> torch.Tensor:
+        shape = hidden_states.shape
+        x = hidden_states.reshape(-1, shape[-1])
+        if not x.is_cuda:
+            raise RuntimeError("dartmoq_hip layers run on the GPU only (no CPU fallback)")
+        orig_dtype = x.dtype
+        if x.dtype != torch.float16:
+            x = x.half()
+        x = x.contiguous()
+        tokens = x.shape[0]
+        if topk_idx is None:
+            topk_w, topk_idx = self.route(x, router_logits)
+        topk_idx = topk_idx.to(torch.int32).contiguous()
+        topk_w = topk_w.float().contiguous()
+        desc = self._descriptor()[0]
+        ws = self._get_workspace(tokens)
+        out = torch.empty_like(x)
+        add = None if residual is None else residual.reshape(-1, shape[-1]).half().contiguous()
+        stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+        check(load().dmq_moe_ffn_forward(
+            ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens,
+            None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
+            int(self.tt_override), stream), "moe_ffn_forward")
+        if orig_dtype != torch.float16:
+            out = out.to(orig_dtype)
+        return out.reshape(shape)
+
+    __call__ = forward
+
+    # ------------------------------------------------------------------ accounting
+    def weight_bytes_per_expert(self, bit: int) -> int:
+        """Algorithmic packed-weight bytes of one expert: indices + fp16 norms."""
+        h, i = self.hidden_size, self.intermediate_size
+        return 3 * h * i * bit // 8 + 6 * h * i // GROUP_SIZE
+
+    def flops_per_token(self) -> int:
+        return self.top_k * 6 * self.hidden_size * self.intermediate_size
+
+
+class WxA8BitPartitionedGroupMoE(WxA16BitPartitionedGroupMoE):
+    MODE = "wxa8"
+
+
+class WxFP8BitPartitionedGroupMoE(WxA16BitPartitionedGroupMoE):
+    MODE = "wxfp8"
+
+
+class WxFP4BitPartitionedGroupMoE(WxA8BitPartitionedGroupMoE):
+    MODE = "wxfp4"
+
+
+MOE_CLASS_BY_MODE = {
+    "wxa16": WxA16BitPartitionedGroupMoE, "wxa8": WxA8BitPartitionedGroupMoE,
+    "wxfp8": WxFP8BitPartitionedGroupMoE, "wxfp4": WxFP4BitPartitionedGroupMoE,
+}
+
+
+def convert_moe(moe: WxA16BitPartitionedGroupMoE, mode: str) -> WxA16BitPartitionedGroupMoE:
+    """convert_model_to_wxa8 / wxfp8 / wxfp4 for one layer (qwen35_quant_io.py:416-532)."""
+    return MOE_CLASS_BY_MODE[mode].from_wxa16(moe)

@@ -1,0 +1,285 @@
+"""Thin torch-tensor front end of the C ABI: pointer extraction, output allocation, checks.
+
+torch is used for device memory and streams only; every computation below happens in
+libdartmoq_hip.so.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import (EPI_SCATTER, EPI_SILU, EPI_STORE, MODE_A16, MODE_A8, MODE_FP4, MODE_FP8, GemmArgs,
+                   check, load)
+
+GROUP_SIZE = 128
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(device=None):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("dartmoq_hip operates on GPU tensors only (no CPU fallback)")
+
+
+def _check_bit(bit, allowed=(1, 2, 4)):
+    if bit not in allowed:
+        raise ValueError(f"bit_width must be one of {allowed}, got {bit}")
+
+
+def act_bytes_per_group(mode: int) -> int:
+    return {MODE_A16: 256, MODE_A8: 128, MODE_FP8: 128, MODE_FP4: 64}[mode]
+
+
+# ----------------------------------------------------------------------------- packed format
+
+def unpack_nbit(packed: torch.Tensor, bit_width: int, n: int | None = None) -> torch.Tensor:
+    """uint8 (..., P) -> uint8 (..., P*8/bit) [:n]."""
+    _check_bit(bit_width, (1, 2, 4, 8))
+    _need_cuda(packed)
+    packed = packed.contiguous()
+    epb = 8 // bit_width
+    out = torch.empty(packed.shape[:-1] + (packed.shape[-1] * epb,), dtype=torch.uint8,
+                      device=packed.device)
+    check(load().dmq_unpack_nbit(_ptr(packed), packed.numel(), bit_width, _ptr(out),
+                                 _stream(packed.device)), "unpack_nbit")
+    return out if n is None else out[..., :n]
+
+
+def convert_to_group_first(indices_packed, norms, group_size, bit_width, prescale: bool = False):
+    _check_bit(bit_width, (1, 2, 4, 8))
+    if group_size != GROUP_SIZE:
+        raise ValueError(f"group_size must be {GROUP_SIZE}, got {group_size}")
+    _need_cuda(indices_packed, norms)
+    indices_packed = indices_packed.contiguous()
+    norms = norms.contiguous().to(torch.float16)
+    ppg = group_size * bit_width // 8
+    n_rows, packed_k = indices_packed.shape
+    if packed_k % ppg:
+        raise ValueError(f"packed row length {packed_k} is not a multiple of {ppg}")
+    groups = packed_k // ppg
+    idx_gf = torch.empty((groups, n_rows, ppg), dtype=torch.uint8, device=indices_packed.device)
+    norms_gf = torch.empty((groups, n_rows), dtype=torch.float16, device=indices_packed.device)
+    check(load().dmq_convert_to_group_first(_ptr(indices_packed), _ptr(norms), n_rows, groups,
+                                            bit_width, int(prescale), _ptr(idx_gf), _ptr(norms_gf),
+                                            _stream(idx_gf.device)), "convert_to_group_first")
+    return idx_gf, norms_gf
+
+
+def dequant_tile(idx_gf, codebook, norms_gf, g0, g_cnt, n0, n_cnt, bit_width):
+    _check_bit(bit_width)
+    _need_cuda(idx_gf, codebook)
+    out = torch.empty((g_cnt, n_cnt, GROUP_SIZE), dtype=torch.float16, device=idx_gf.device)
+    check(load().dmq_dequant_tile(_ptr(idx_gf), _ptr(codebook.contiguous()), _ptr(norms_gf),
+                                  idx_gf.shape[1], g0, g_cnt, n0, n_cnt, bit_width, _ptr(out),
+                                  _stream(out.device)), "dequant_tile")
+    return out
+
+
+def fold_indices_to_e2m1(indices_gf, nib, bit_width, group_size=GROUP_SIZE):
+    if bit_width not in (1, 2, 4):
+        raise ValueError(f"fold supports bit 1/2/4, got {bit_width}")
+    _need_cuda(indices_gf)
+    g, n, _ = indices_gf.shape
+    out = torch.empty((g, n, group_size // 2), dtype=torch.uint8, device=indices_gf.device)
+    nib = nib.to(indices_gf.device, torch.uint8).contiguous()
+    check(load().dmq_fold_indices_to_e2m1(_ptr(indices_gf.contiguous()), _ptr(nib), g * n, bit_width,
+                                          _ptr(out), _stream(out.device)), "fold_indices_to_e2m1")
+    return out
+
+
+# ----------------------------------------------------------------------------- routing
+
+def route_topk(logits: torch.Tensor, top_k: int, renormalize: bool = False):
+    _need_cuda(logits)
+    if logits.dtype not in (torch.float32, torch.float16):
+        logits = logits.float()
+    logits = logits.contiguous()
+    t, e = logits.shape
+    w = torch.empty((t, top_k), dtype=torch.float32, device=logits.device)
+    idx = torch.empty((t, top_k), dtype=torch.int32, device=logits.device)
+    check(load().dmq_route_topk(_ptr(logits), int(logits.dtype == torch.float16), t, e, top_k,
+                                int(renormalize), _ptr(w), _ptr(idx), _stream(logits.device)),
+          "route_topk")
+    return w, idx
+
+
+def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_rows=16):
+    """Device-side sort + pool partition.  Returns a dict of int32/fp32 device tensors."""
+    _need_cuda(topk_idx, topk_w, slice_start, slice_count)
+    t, k = topk_idx.shape
+    dev = topk_idx.device
+    pools = slice_start.shape[0]
+    rows = t * k
+    max_tiles = rows // tile_rows + num_experts
+    i32 = dict(dtype=torch.int32, device=dev)
+    res = {
+        "counts": torch.empty(num_experts, **i32),
+        "offsets": torch.empty(num_experts + 1, **i32),
+        "sorted_tokens": torch.empty(rows, **i32),
+        "sorted_weights": torch.empty(rows, dtype=torch.float32, device=dev),
+        "sorted_slots": torch.empty(rows, **i32),
+        "gu_info": torch.empty((pools, num_experts, 4), **i32),
+        "dn_info": torch.empty((pools, num_experts, 4), **i32),
+        "n_tiles": torch.zeros((pools, 4), **i32),
+        "tiles": torch.zeros((pools, max_tiles, 2), **i32),
+        "max_tiles": max_tiles, "tile_rows": tile_rows,
+    }
+    check(load().dmq_route_permute(
+        _ptr(topk_idx.to(torch.int32).contiguous()), _ptr(topk_w.float().contiguous()), t, k,
+        num_experts, pools, _ptr(slice_start.contiguous()), _ptr(slice_count.contiguous()), tile_rows,
+        max_tiles, _ptr(res["counts"]), _ptr(res["offsets"]), _ptr(res["sorted_tokens"]),
+        _ptr(res["sorted_weights"]), _ptr(res["sorted_slots"]), _ptr(res["gu_info"]),
+        _ptr(res["dn_info"]), _ptr(res["n_tiles"]), _ptr(res["tiles"]), _stream(dev)), "route_permute")
+    return res
+
+
+def build_tiles(expert_info: torch.Tensor, rows_total: int, tile_rows: int):
+    """(n_tiles int32[1], tiles int32[max_tiles, 2], max_tiles) for a device expert_info [E, 4]."""
+    _need_cuda(expert_info)
+    n_exp = expert_info.shape[0]
+    max_tiles = rows_total // tile_rows + n_exp
+    n_tiles = torch.zeros(4, dtype=torch.int32, device=expert_info.device)
+    tiles = torch.zeros((max_tiles, 2), dtype=torch.int32, device=expert_info.device)
+    check(load().dmq_build_tiles(_ptr(expert_info), n_exp, tile_rows, max_tiles, _ptr(n_tiles),
+                                 _ptr(tiles), _stream(expert_info.device)), "build_tiles")
+    return n_tiles, tiles, max_tiles
+
+
+# ----------------------------------------------------------------------------- activations
+
+def _alloc_codes(mode, rows, k, device, scale_fp32):
+    groups = k // GROUP_SIZE
+    if mode == MODE_A16:
+        return torch.empty((rows, k), dtype=torch.float16, device=device), None, 0
+    if mode == MODE_A8:
+        codes = torch.empty((rows, k), dtype=torch.int8, device=device)
+    elif mode == MODE_FP8:
+        codes = torch.empty((rows, k), dtype=torch.float8_e4m3fn, device=device)
+    else:
+        codes = torch.empty((rows, k // 2), dtype=torch.uint8, device=device)
+        return codes, torch.empty((rows, k // 32), dtype=torch.uint8, device=device), k // 32
+    sdt = torch.float32 if scale_fp32 else torch.float16
+    return codes, torch.empty((rows, groups), dtype=sdt, device=device), groups
+
+
+def rotate(mode: int, x: torch.Tensor, rot: torch.Tensor, extra_scale: float = 1.0,
+           scale_fp32: bool = False, row_index: torch.Tensor | None = None, tt: int | None = None):
+    """Rotate (and quantize for mode != A16) x[B, K] with rot[G, 128, 128]."""
+    _need_cuda(x, rot)
+    if x.dtype != torch.float16:
+        x = x.half()
+    x = x.contiguous()
+    rot = rot.contiguous()
+    k = x.shape[1]
+    rows = x.shape[0] if row_index is None else row_index.numel()
+    groups = k // GROUP_SIZE
+    if k != groups * GROUP_SIZE:
+        raise ValueError(f"K ({k}) must be a multiple of {GROUP_SIZE}")
+    if tuple(rot.shape) != (groups, GROUP_SIZE, GROUP_SIZE) or rot.dtype != torch.float16:
+        raise ValueError(f"rot must be fp16 {(groups, GROUP_SIZE, GROUP_SIZE)}, got {tuple(rot.shape)}")
+    codes, scale, sstride = _alloc_codes(mode, rows, k, x.device, scale_fp32)
+    if tt is None:
+        tt = 4 if rows >= 1024 else 1
+    check(load().dmq_rotate(mode, _ptr(x), x.stride(0), _ptr(row_index), _ptr(rot), rows, groups,
+                            _ptr(codes), codes.stride(0) * codes.element_size(), _ptr(scale), sstride,
+                            int(scale_fp32), float(extra_scale), tt, _stream(x.device)), "rotate")
+    return codes, scale
+
+
+def rotate_tiled(mode, x, rot, expert_info, n_tiles, tiles, tile_rows, max_tiles, rows_out,
+                 rot_per_expert=True, extra_scale=1.0, row_index=None, tt=1):
+    """Per-expert rotation: rows of expert e use rot[slice_start_e + g]."""
+    _need_cuda(x, rot, expert_info)
+    x = x.contiguous()
+    k = x.shape[1]
+    groups = k // GROUP_SIZE
+    codes, scale, sstride = _alloc_codes(mode, rows_out, k, x.device, False)
+    check(load().dmq_rotate_tiled(mode, _ptr(x), x.stride(0), _ptr(row_index), _ptr(rot.contiguous()),
+                                  int(rot_per_expert), groups, _ptr(expert_info), _ptr(tiles),
+                                  _ptr(n_tiles), tile_rows, max_tiles, _ptr(codes),
+                                  codes.stride(0) * codes.element_size(), _ptr(scale), sstride, 0,
+                                  float(extra_scale), tt, _stream(x.device)), "rotate_tiled")
+    return codes, scale
+
+
+def quantize_act(mode: int, x_rot: torch.Tensor, extra_scale: float = 1.0, scale_fp32: bool = True):
+    """Quantize already rotated activations (fp16 or fp32)."""
+    _need_cuda(x_rot)
+    if x_rot.dtype not in (torch.float16, torch.float32):
+        x_rot = x_rot.float()
+    x_rot = x_rot.contiguous()
+    rows, k = x_rot.shape
+    if k % GROUP_SIZE:
+        raise ValueError(f"K ({k}) must be a multiple of group_size ({GROUP_SIZE})")
+    codes, scale, sstride = _alloc_codes(mode, rows, k, x_rot.device, scale_fp32)
+    check(load().dmq_quantize_act(mode, _ptr(x_rot), int(x_rot.dtype == torch.float32), x_rot.stride(0),
+                                  rows, k // GROUP_SIZE, _ptr(codes),
+                                  codes.stride(0) * codes.element_size(), _ptr(scale), sstride,
+                                  int(scale_fp32), float(extra_scale), _stream(x_rot.device)),
+          "quantize_act")
+    return codes, scale
+
+
+# ----------------------------------------------------------------------------- GEMM
+
+def pick_tt(rows_total: int, n_experts: int) -> int:
+    avg = rows_total / max(n_experts, 1)
+    return 1 if avg <= 8 else (2 if avg <= 48 else 4)
+
+
+def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *, groups, n_out,
+                  slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
+                  row_index=None, w_scale_byte=127, row_weight=None, row_token=None, tt=None,
+                  tiling=None, dbg_acc=None):
+    """One merged dequant-GEMM launch.  ``expert_info`` is an int32 device tensor [E, 4]."""
+    _need_cuda(act, w, norms, expert_info)
+    dev = act.device
+    n_exp = expert_info.shape[0]
+    if tt is None:
+        tt = pick_tt(rows_total, n_exp)
+    if tiling is None:
+        tiling = build_tiles(expert_info, rows_total, 16 * tt)
+    n_tiles, tiles, max_tiles = tiling
+    if out is None:
+        if epi == EPI_SCATTER:
+            raise ValueError("scatter epilogue needs a caller-provided fp32 accumulator")
+        out = torch.empty((rows_total, n_out), dtype=torch.float16, device=dev)
+        out_stride = n_out
+    a = GemmArgs()
+    a.mode, a.bit, a.epi, a.tt = mode, bit, epi, tt
+    a.act = act.data_ptr()
+    a.act_row_bytes = act.stride(0) * act.element_size()
+    a.act_scale = act_scale.data_ptr() if act_scale is not None else None
+    a.act_scale_stride = act_scale.stride(0) if act_scale is not None else 0
+    a.row_index = row_index.data_ptr() if row_index is not None else None
+    a.w, a.norms = w.data_ptr(), norms.data_ptr()
+    a.lut = lut.data_ptr() if lut is not None else None
+    a.n_total = w.shape[1]
+    a.groups, a.n_out, a.half_width = groups, n_out, half_width
+    a.slice_is_groups, a.w_scale_byte = int(slice_is_groups), int(w_scale_byte)
+    a.expert_info, a.n_experts = expert_info.data_ptr(), n_exp
+    a.tiles, a.n_tiles, a.max_tiles = tiles.data_ptr(), n_tiles.data_ptr(), max_tiles
+    a.out, a.out_stride = out.data_ptr(), out_stride if out_stride is not None else out.stride(0)
+    a.row_weight = row_weight.data_ptr() if row_weight is not None else None
+    a.row_token = row_token.data_ptr() if row_token is not None else None
+    a.dbg_acc = dbg_acc.data_ptr() if dbg_acc is not None else None
+    check(load().dmq_matmul_merged_gf(ctypes.byref(a), _stream(dev)), "matmul_merged_gf")
+    return out
+
+
+def finalize_f16(acc32: torch.Tensor, add: torch.Tensor | None = None) -> torch.Tensor:
+    _need_cuda(acc32)
+    out = torch.empty(acc32.shape, dtype=torch.float16, device=acc32.device)
+    check(load().dmq_finalize_f16(_ptr(acc32), _ptr(add), acc32.numel(), _ptr(out),
+                                  _stream(acc32.device)), "finalize_f16")
+    return out

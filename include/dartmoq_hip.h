@@ -1,0 +1,219 @@
+/*
+ * dartmoq_hip -- C ABI of the MI355X (gfx950) quantized MoE FFN kernels.
+ *
+ * Every entry point takes raw device pointers, explicit sizes and a HIP stream
+ * (passed as void*; NULL = the default stream), launches asynchronously on that
+ * stream, never allocates or synchronizes, and returns a DMQ_* status code.
+ * Inputs are never modified; outputs and workspaces are caller-owned.
+ *
+ * The reference (zzningxp/DartMoQ-Qwen3.5) has no FFI for this path: its
+ * boundary is the set of Python callables in turboquant_utils/triton_kernels*.py
+ * that quantization/{wxa16,wxa8,wxfp8,wxfp4}/bit_partitioned_moe.py import.  Each
+ * declaration below names the callable(s) it stands in for (paths relative to
+ * the reference checkout).
+ *
+ * Conventions shared by all entry points
+ *   group size            128 input features per quantization group
+ *   bit                   1, 2 or 4 bits per codebook index (unpack also takes 8)
+ *   idx_gf                uint8 [G, N, 128*bit/8]  group-first packed indices
+ *   norms_gf              fp16  [G, N]             per-(group,row) norms / sqrt(128)
+ *   mode                  DMQ_MODE_A16 / A8 / FP8 / FP4
+ *   expert_info           int32 [n_experts, 4] = token_start, token_count,
+ *                         slice_start, slice_count   (device memory)
+ */
+#ifndef DARTMOQ_HIP_H
+#define DARTMOQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  DMQ_OK = 0, DMQ_ERR_BIT = 1, DMQ_ERR_ALIGN = 2, DMQ_ERR_SHAPE = 3, DMQ_ERR_EMPTY = 4,
+  DMQ_ERR_MODE = 5, DMQ_ERR_NULL = 6, DMQ_ERR_HIP = 7, DMQ_ERR_LIMIT = 8
+};
+enum { DMQ_MODE_A16 = 0, DMQ_MODE_A8 = 1, DMQ_MODE_FP8 = 2, DMQ_MODE_FP4 = 3 };
+enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
+
+/* Library / build identification: returns the ABI version (currently 1). */
+int dmq_abi_version(void);
+/* Human-readable text for a status code (static storage). */
+const char* dmq_status_string(int status);
+
+/* ------------------------------------------------------------------ packed format */
+
+/* unpack_nbit, turboquant_utils/quantize.py:74-100.  out holds one index per byte,
+ * n_bytes * 8/bit entries. */
+int dmq_unpack_nbit(const void* packed, long n_bytes, int bit, void* out_u8, void* stream);
+
+/* convert_to_group_first, turboquant_utils/triton_kernels.py:1042-1069, plus the optional
+ * pre-division of the norms by sqrt(128) that WxA16Weights._build_group_first performs
+ * (quantization/wxa16/bit_partitioned_moe.py:193-204).
+ * indices_packed [n_rows, groups*ppg] -> idx_gf [groups, n_rows, ppg];
+ * norms [n_rows, groups] -> norms_gf [groups, n_rows]. */
+int dmq_convert_to_group_first(const void* indices_packed, const void* norms, int n_rows,
+                               int groups, int bit, int prescale, void* idx_gf, void* norms_gf,
+                               void* stream);
+
+/* The dequantized weight tile the GEMM kernels consume: out fp16 [g_cnt, n_cnt, 128] =
+ * codebook[idx] (times norms_gf when given), produced through the same LDS byte table.
+ * Stands in for the in-kernel "w_quant" tile of
+ * turboquant_utils/triton_kernels.py:893-991. */
+int dmq_dequant_tile(const void* idx_gf, const void* codebook_f16, const void* norms_gf,
+                     int n_total, int g0, int g_cnt, int n0, int n_cnt, int bit, void* out_f16,
+                     void* stream);
+
+/* fold_indices_to_e2m1, turboquant_utils/triton_kernels_fp4.py:80-122.
+ * idx_gf [rows, 128*bit/8] -> out [rows, 64], rows = G*N. */
+int dmq_fold_indices_to_e2m1(const void* idx_gf, const void* nib_lut, long rows, int bit,
+                             void* out, void* stream);
+
+/* ------------------------------------------------------------------ routing */
+
+/* softmax + top-k of quantization/wxa16/bit_partitioned_moe.py:1112-1120 (lowest expert
+ * index wins ties; renorm != 0 divides by the kept mass like the HF TopKRouter).
+ * logits [tokens, experts] fp32 (logits_fp16 == 0) or fp16; out_w fp32 [tokens, k],
+ * out_idx int32 [tokens, k].  experts <= 1024, k <= 64. */
+int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts, int k,
+                   int renorm, void* out_w, void* out_idx, void* stream);
+
+/* Sort / bincount / pool partition of bit_partitioned_moe.py:1125-1138 and
+ * _merged_pools / _merged_expert_info_rows / _merged_expert_info_groups (:1014-1057) and
+ * _build_merged_block_info (turboquant_utils/triton_kernels_a8.py:938-956), without the
+ * host round trip.
+ *   slice_start [pools, experts] int32: 2*start of the expert in that pool, -1 = not a member
+ *   slice_count [pools, experts] int32: 2*I
+ * Outputs (device, int32 unless noted):
+ *   counts [experts], offsets [experts+1], sorted_tokens [tokens*k],
+ *   sorted_weights fp32 [tokens*k], sorted_slots [tokens*k] (may be NULL),
+ *   gu_info / dn_info [pools, experts, 4], n_tiles [pools, 4], tiles [pools, max_tiles, 2]. */
+int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
+                      int pools, const void* slice_start, const void* slice_count, int tile_rows,
+                      int max_tiles, void* counts, void* offsets, void* sorted_tokens,
+                      void* sorted_weights, void* sorted_slots, void* gu_info, void* dn_info,
+                      void* n_tiles, void* tiles, void* stream);
+
+/* Tile list for a caller-built expert_info: n_tiles int32[1], tiles int32 [max_tiles, 2]. */
+int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_tiles,
+                    void* n_tiles, void* tiles, void* stream);
+
+/* ------------------------------------------------------------------ activations */
+
+/* batch_rotate_input (turboquant_utils/rotation.py:176-212) for mode A16 and the fused
+ * rotate+quantize kernels rotate_quantize_fused (triton_kernels_a8.py:486-523),
+ * rotate_quantize_fused_fp8 (triton_kernels_fp8.py:188-226) and rotate_quantize_fused_fp4
+ * (triton_kernels_fp4.py:1111-1135) for A8 / FP8 / FP4.
+ *   x fp16 [*, x_stride]; row_index (optional) gathers input rows; rot fp16 [groups,128,128]
+ *   out: fp16 [rows, K] | int8 / e4m3 [rows, K] | packed e2m1 [rows, K/2] (row-major)
+ *   scale: fp16 (scale_fp32 == 0) or fp32 [rows, scale_stride] | FP4: u8 [rows, scale_stride]
+ * tt = 1 or 4 activation tiles of 16 rows per wave. */
+int dmq_rotate(int mode, const void* x, long x_stride, const void* row_index, const void* rot,
+               int rows, int groups, void* out, long out_row_bytes, void* scale,
+               int scale_stride, int scale_fp32, float extra_scale, int tt, void* stream);
+
+/* Same, for rows grouped by expert: tile entry (e, i) covers rows token_start + i*tile_rows ..
+ * With rot_per_expert != 0 group g of expert e uses rot[slice_start_e + g] (the per-expert
+ * down rotations, seed + original_start of triton_kernels.py:1310), otherwise rot[g].
+ * max_tiles bounds the tile list. */
+int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_index,
+                     const void* rot, int rot_per_expert, int groups, const void* expert_info, const void* tiles,
+                     const void* n_tiles, int tile_rows, int max_tiles, void* out,
+                     long out_row_bytes, void* scale, int scale_stride, int scale_fp32,
+                     float extra_scale, int tt, void* stream);
+
+/* quantize_act_per_token_group (triton_kernels_a8.py:384-421), ..._fp8
+ * (triton_kernels_fp8.py:94-124) and quantize_act_e2m1_per32 (triton_kernels_fp4.py:125-150):
+ * quantization of already rotated activations (fp16 or fp32 input). */
+int dmq_quantize_act(int mode, const void* x, int x_fp32, long x_stride, int rows, int groups,
+                     void* out, long out_row_bytes, void* scale, int scale_stride, int scale_fp32,
+                     float extra_scale, void* stream);
+
+/* ------------------------------------------------------------------ dequant GEMMs */
+
+typedef struct {
+  int mode;                 /* DMQ_MODE_* */
+  int bit;                  /* index width of idx_gf (FP4 reads folded e2m1: pass the pool bit) */
+  int epi;                  /* DMQ_EPI_* */
+  int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4 */
+  const void* act;          /* activation codes, row-major */
+  long act_row_bytes;
+  const void* act_scale;    /* fp16 [rows, act_scale_stride] (A8/FP8), u8 (FP4), NULL (A16) */
+  int act_scale_stride;
+  const void* row_index;    /* optional gather of activation rows (int32) */
+  const void* w;            /* idx_gf, or folded e2m1 [G, N, 64] for FP4 */
+  const void* norms;        /* norms_gf */
+  const void* lut;          /* fp16 / int8 / e4m3 codebook; unused for FP4 */
+  int n_total;              /* N of the shared weight */
+  int groups;               /* groups contracted per expert */
+  int n_out;                /* output features per row (SILU: I) */
+  int half_width;           /* SILU: I */
+  int slice_is_groups;      /* 0 gate_up (slice offsets rows), 1 down (slice offsets groups) */
+  int w_scale_byte;         /* FP4: 127 + E0 */
+  const void* expert_info;
+  int n_experts;
+  const void* tiles;        /* from dmq_build_tiles / dmq_route_permute, tile_rows == 16*tt */
+  const void* n_tiles;
+  int max_tiles;
+  void* out;                /* STORE/SILU: fp16 [rows, out_stride]; SCATTER: fp32 [tokens, out_stride] */
+  long out_stride;
+  const void* row_weight;   /* SCATTER: fp32 routing weight per row */
+  const void* row_token;    /* SCATTER: int32 destination token per row */
+  void* dbg_acc;            /* A8, tt == 1, STORE only: int32 [rows, groups, n_out] or NULL */
+} dmq_gemm_args;
+
+/* Merged (one launch per bit pool) dequant GEMM.  Stands in for
+ *   triton_fused_matmul_merged_rows_gf / _merged_in_features_gf   (triton_kernels.py:1482-1615)
+ *   wxa8_matmul_merged_rows_gf / _merged_in_features_gf           (triton_kernels_a8.py:959-1068)
+ *   wxfp8_matmul_merged_rows_gf / _merged_in_features_gf          (triton_kernels_fp8.py:641-750)
+ *   wxfp4_matmul_merged_rows_gf / _merged_in_features_gf          (triton_kernels_fp4.py:740-874)
+ * and, with a one-row expert_info, for the per-expert *_grouped_slice_rows_gf /
+ * *_grouped_slice_in_features_gf / *_grouped_gf wrappers.  DMQ_EPI_SILU fuses
+ * F.silu(gate) * up (bit_partitioned_moe.py:925-930), DMQ_EPI_SCATTER fuses the routing
+ * weight and index_add_ (:965-967) into fp32 atomics. */
+int dmq_matmul_merged_gf(const dmq_gemm_args* args, void* stream);
+
+/* fp16(out32 (+ add16)) over n elements (n % 4 == 0): final store of the scatter target. */
+int dmq_finalize_f16(const void* acc_f32, const void* add_f16, long n, void* out_f16, void* stream);
+/* Zero-fill n bytes (n % 4 == 0) with a kernel (usable under graph capture). */
+int dmq_fill_zero(void* ptr, long n_bytes, void* stream);
+
+/* ------------------------------------------------------------------ whole layer */
+
+typedef struct {
+  int bit;
+  int mode;                 /* mode of this pool (WxFP4 keeps bit-2 pools on DMQ_MODE_A8) */
+  int major;                /* 1: rotate all tokens once (hoisted); 0: rotate routed rows only */
+  int n_gate_up;            /* rows of the gate_up pool matrix (2*I*members) */
+  int down_groups;          /* groups of the down pool matrix (I*members/128) */
+  const void* gu_w;  const void* gu_norms;  const void* gu_lut;  const void* gu_rot;
+  float gu_extra_scale;  int gu_w_scale_byte;
+  const void* dn_w;  const void* dn_norms;  const void* dn_lut;  const void* dn_rot;
+  float dn_extra_scale;  int dn_w_scale_byte;
+} dmq_pool_desc;
+
+typedef struct {
+  int hidden, inter, experts, top_k, pools;
+  const dmq_pool_desc* pool;      /* host array [pools] */
+  const void* slice_start;        /* device int32 [pools, experts] (2*start or -1) */
+  const void* slice_count;        /* device int32 [pools, experts] (2*I) */
+} dmq_layer_desc;
+
+/* Bytes of workspace dmq_moe_ffn_forward needs for `tokens` tokens. */
+size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens);
+
+/* WxA16BitPartitionedGroupMoE.forward (quantization/wxa16/bit_partitioned_moe.py:1059-1224)
+ * and its WxA8 / WxFP8 / WxFP4 subclasses, routed experts only:
+ *   x fp16 [tokens, hidden]; topk_idx int32 / topk_w fp32 [tokens, top_k];
+ *   out fp16 [tokens, hidden] = sum_k w * down_e(silu(gate_e(x)) * up_e(x)) (+ add_f16).
+ * tt <= 0 picks the activation tile count from tokens. */
+int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
+                        const void* topk_w, int tokens, const void* add_f16, void* out,
+                        void* workspace, size_t workspace_bytes, int tt, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,189 @@
+"""GPU parity: activation quantizers and the fused rotate+quantize kernel.
+
+* The quantizer stage on already rotated input is bit-exact against the oracle
+  (int8 / e4m3 / e2m1 codes and scales).
+* The fused kernel is bit-exact whenever the rotation sums are exact in fp32
+  whatever the order of accumulation (signed permutations, +-1/2 block Hadamard
+  mixes on coarse-grained inputs); with Haar rotations the matrix-core
+  accumulation order differs from the CPU's, so codes may differ by one step on
+  rounding boundaries -- bounded below like the reference bounds its own fused
+  kernel against torch (int8 max code diff 1, a few e4m3 bytes per million).
+"""
+
+import pytest
+import torch
+
+from oracle import actquant, rotation
+
+pytestmark = pytest.mark.gpu
+
+A8, FP8, FP4 = 1, 2, 3
+
+
+def _inputs(rows, k, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(rows, k, generator=g) * scale).half()
+    x[0, :128] = 0                                    # an all-zero group hits the scale floor
+    if rows > 2:
+        x[2, 5] = 60000.0                             # large outlier
+    return x
+
+
+@pytest.mark.parametrize("rows,k", [(1, 128), (37, 512), (300, 2048)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_quantize_int8_bit_exact(rows, k, dtype):
+    from dartmoq_hip import ops
+    x = _inputs(rows, k, 1).to(dtype)
+    if dtype == torch.float32:
+        x = x * 1.00003 + 1e-4
+    q_ref, s_ref = actquant.quantize_act_int8(x, 128, 0.0118931)
+    q, s = ops.quantize_act(A8, x.cuda(), 0.0118931, scale_fp32=True)
+    assert torch.equal(q.cpu(), q_ref)
+    assert torch.equal(s.cpu(), s_ref)
+    _, s16 = ops.quantize_act(A8, x.cuda(), 0.0118931, scale_fp32=False)
+    assert torch.equal(s16.cpu().view(torch.int16), s_ref.half().view(torch.int16))
+
+
+@pytest.mark.parametrize("rows,k", [(1, 128), (37, 512), (300, 2048)])
+def test_quantize_fp8_bit_exact(rows, k):
+    from dartmoq_hip import ops
+    x = _inputs(rows, k, 2)
+    q_ref, s_ref = actquant.quantize_act_fp8(x, 128, 0.00472)
+    q, s = ops.quantize_act(FP8, x.cuda(), 0.00472, scale_fp32=True)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+    assert torch.equal(s.cpu(), s_ref)
+
+
+def test_fp8_encoder_all_codes():
+    """Every e4m3 value, every midpoint between neighbours and saturation."""
+    from dartmoq_hip import ops
+    codes = torch.arange(0, 127, dtype=torch.uint8).view(torch.float8_e4m3fn).float()   # 0 .. 448
+    mids = (codes[1:] + codes[:-1]) / 2
+    vals = torch.cat([codes, mids, mids * (1 + 2 ** -20), mids * (1 - 2 ** -20)])
+    vals = torch.cat([vals, -vals])
+    pad = (-vals.numel()) % 128
+    vals = torch.cat([vals, torch.zeros(pad)]).reshape(-1, 128)
+    vals[:, 0] = 448.0                                 # amax == 448 -> scale exactly 1
+    q_ref, _ = actquant.quantize_act_fp8(vals, 128)
+    q, _ = ops.quantize_act(FP8, vals.cuda(), 1.0, scale_fp32=True)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("rows,k", [(1, 128), (37, 512), (300, 2048)])
+def test_quantize_e2m1_bit_exact(rows, k):
+    from dartmoq_hip import ops
+    x = _inputs(rows, k, 3)
+    p_ref, sb_ref = actquant.quantize_act_e2m1(x)
+    p, sb = ops.quantize_act(FP4, x.cuda())
+    assert torch.equal(sb.cpu(), sb_ref)
+    assert torch.equal(p.cpu(), p_ref)
+
+
+def test_e2m1_power_of_two_edges_and_ties():
+    """amax = 6 * 2^k * (1 +- ulp) decides the block exponent; grid midpoints tie downwards."""
+    from dartmoq_hip import ops
+    rows = []
+    for kexp in range(-12, 6):
+        for delta in (0.0, 2.0 ** -11, -(2.0 ** -11)):          # fp16 ulp steps around 6 * 2^k
+            amax = 6.0 * 2.0 ** kexp * (1.0 + delta)
+            row = torch.tensor([0.0, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 0.5, 1.0, 3.0]
+                               ).repeat(11)[:128] * (2.0 ** kexp)
+            row[::2] *= -1
+            row[3] = amax
+            row[35] = amax
+            rows.append(row)
+    x = torch.stack(rows).float()
+    # one fp32 ulp either side of 6 * 2^k as well
+    edge = x[::3].clone()
+    up = torch.nextafter(edge[:, 3], torch.tensor(float("inf")))
+    dn = torch.nextafter(edge[:, 3], torch.tensor(0.0))
+    e_up, e_dn = edge.clone(), edge.clone()
+    e_up[:, 3], e_up[:, 35] = up, up
+    e_dn[:, 3], e_dn[:, 35] = dn, dn
+    x = torch.cat([x, e_up, e_dn])
+    p_ref, sb_ref = actquant.quantize_act_e2m1(x)
+    p, sb = ops.quantize_act(FP4, x.cuda())
+    assert torch.equal(sb.cpu(), sb_ref)
+    assert torch.equal(p.cpu(), p_ref)
+
+
+def _exact_rotations(groups, seed):
+    """Rotations whose products are exact in fp32 in any summation order: a signed permutation
+    composed with a block-diagonal 4x4 Hadamard / 2 (entries 0, +-1/2)."""
+    g = torch.Generator().manual_seed(seed)
+    h4 = torch.tensor([[1, 1, 1, 1], [1, -1, 1, -1], [1, 1, -1, -1], [1, -1, -1, 1]]).float() / 2
+    mats = []
+    for _ in range(groups):
+        perm = torch.randperm(128, generator=g)
+        sign = torch.randint(0, 2, (128,), generator=g).float() * 2 - 1
+        p = torch.zeros(128, 128)
+        p[torch.arange(128), perm] = sign
+        mats.append(torch.block_diag(*[h4] * 32) @ p)
+    return torch.stack(mats).half()
+
+
+@pytest.mark.parametrize("mode", [0, A8, FP8, FP4])
+@pytest.mark.parametrize("rows,tt", [(50, 1), (130, 4)])
+def test_fused_rotate_quantize_exact_rotations(mode, rows, tt):
+    from dartmoq_hip import ops
+    k = 512
+    g = torch.Generator().manual_seed(rows)
+    # multiples of 1/64 below 8: four-term sums with +-1/2 weights are exact in fp32 and fp16
+    x = (torch.randint(-512, 512, (rows, k), generator=g).float() / 64).half()
+    rot = _exact_rotations(k // 128, 7)
+    x_rot = rotation.rotate_with(x, rot, torch.float32)
+    codes, scale = ops.rotate(mode, x.cuda(), rot.cuda(), extra_scale=0.0215203, tt=tt)
+    if mode == 0:
+        assert torch.equal(codes.cpu().view(torch.int16), x_rot.half().view(torch.int16))
+    elif mode == A8:
+        q_ref, s_ref = actquant.quantize_act_int8(x_rot, 128, 0.0215203)
+        assert torch.equal(codes.cpu(), q_ref)
+        assert torch.equal(scale.cpu().view(torch.int16), s_ref.half().view(torch.int16))
+    elif mode == FP8:
+        q_ref, s_ref = actquant.quantize_act_fp8(x_rot, 128, 0.0215203)
+        assert torch.equal(codes.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+        assert torch.equal(scale.cpu().view(torch.int16), s_ref.half().view(torch.int16))
+    else:
+        p_ref, sb_ref = actquant.quantize_act_e2m1(x_rot)
+        assert torch.equal(scale.cpu(), sb_ref)
+        assert torch.equal(codes.cpu(), p_ref)
+
+
+@pytest.mark.parametrize("mode", [0, A8, FP8, FP4])
+def test_fused_rotate_quantize_haar(mode):
+    """Haar rotations: values agree to accumulation round-off, codes to one rounding step."""
+    from dartmoq_hip import ops
+    rows, k = 257, 2048
+    x = _inputs(rows, k, 11)
+    x[2, 5] = 3.0
+    rot = rotation.batch_rotation_matrices(128, 44, k // 128, 128)
+    x_rot = rotation.rotate_with(x, rot, torch.float32)
+    codes, scale = ops.rotate(mode, x.cuda(), rot.cuda(), extra_scale=0.0118931, tt=4)
+    if mode == 0:
+        torch.testing.assert_close(codes.cpu().float(), x_rot, rtol=2e-3, atol=2e-3)
+        return
+    if mode == A8:
+        q_ref, s_ref = actquant.quantize_act_int8(x_rot, 128, 0.0118931)
+        diff = (codes.cpu().int() - q_ref.int()).abs()
+        assert diff.max() <= 1
+        assert (diff != 0).float().mean() < 2e-3
+        torch.testing.assert_close(scale.cpu().float(), s_ref, rtol=2e-3, atol=1e-9)
+    elif mode == FP8:
+        q_ref, s_ref = actquant.quantize_act_fp8(x_rot, 128, 0.0118931)
+        same = codes.cpu().view(torch.uint8) == q_ref.view(torch.uint8)
+        assert (~same).float().mean() < 2e-3
+        torch.testing.assert_close(codes.cpu().float(), q_ref.float(), rtol=0.13, atol=2 ** -9)
+        torch.testing.assert_close(scale.cpu().float(), s_ref, rtol=2e-3, atol=1e-9)
+    else:
+        p_ref, sb_ref = actquant.quantize_act_e2m1(x_rot)
+        assert (scale.cpu() != sb_ref).float().mean() < 1e-3
+        assert (codes.cpu() != p_ref).float().mean() < 5e-3
+
+
+def test_rotate_rejects_bad_shapes():
+    from dartmoq_hip import ops
+    x = torch.zeros(4, 256, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.rotate(0, x, torch.zeros(3, 128, 128, dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.quantize_act(A8, torch.zeros(4, 100, dtype=torch.float16, device="cuda"))

@@ -1,0 +1,195 @@
+"""GPU parity: merged codebook-dequant GEMMs in all four precision modes.
+
+Each case feeds the kernel and the oracle the *same* activation codes / scales and the same
+packed pool, so the comparison isolates the GEMM: int32 accumulators are exact, fp16 outputs
+match fp32 maths to fp16 rounding.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import actquant, codebook, luts, moe, packing, routing
+
+pytestmark = pytest.mark.gpu
+
+A16, A8, FP8, FP4 = 0, 1, 2, 3
+STORE, SILU, SCATTER = 0, 1, 2
+
+
+def _pool(bit, n_rows, k, seed):
+    """Random packed pool in group-first layout (indices, prescaled fp16 norms, codebook)."""
+    g = torch.Generator().manual_seed(seed)
+    groups = k // 128
+    idx_gf = torch.randint(0, 256, (groups, n_rows, 128 * bit // 8), dtype=torch.uint8, generator=g)
+    norms_gf = ((torch.rand(groups, n_rows, generator=g) * 0.2 + 0.02) / math.sqrt(128)).half()
+    cb = codebook.get_codebook(bit)[0].half()
+    return idx_gf, norms_gf, cb
+
+
+def _expert_rows(counts):
+    info, cur = [], 0
+    for c in counts:
+        info.append(cur)
+        cur += c
+    return info, cur
+
+
+def _mode_inputs(mode, x_rot, cb):
+    """(act codes tensor for the GPU, scale tensor or None, oracle codes fp32, oracle scale fp32,
+    lut for the GPU, oracle lut values fp32, w block scale, norm factor, w_scale_byte)."""
+    b, k = x_rot.shape
+    if mode == A16:
+        xh = x_rot.half()
+        return xh, None, xh.float(), torch.ones(b, k // 128), cb, cb.float(), 1.0, 1.0, 127
+    if mode == A8:
+        q, step = luts.build_int8_codebook(cb)
+        codes, s = actquant.quantize_act_int8(x_rot, 128, step)
+        return codes, s.half(), codes.float(), s.half().float(), q, q.float(), 1.0, 1.0, 127
+    if mode == FP8:
+        q, scale = luts.build_fp8_codebook(cb)
+        codes, s = actquant.quantize_act_fp8(x_rot, 128, scale)
+        return codes, s.half(), codes.float(), s.half().float(), q, q.float(), 1.0, 1.0, 127
+    nib, e0, resid, _ = luts.build_e2m1_codebook(cb)
+    p, sb = actquant.quantize_act_e2m1(x_rot)
+    return (p, sb, actquant.dequant_act_e2m1(p, sb), torch.ones(b, k // 128), nib,
+            luts.e2m1_value(nib), 2.0 ** e0, resid, 127 + e0)
+
+
+def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed):
+    from dartmoq_hip import ops
+    n_exp = len(counts)
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(seed)
+    if slice_is_groups:                       # down: weight [G_total = n_exp * k/128, N = n_slice]
+        idx_gf, norms_gf, cb = _pool(bit, n_slice, k * n_exp, seed)
+        info = [(starts[e], counts[e], e * (k // 128), k // 128) for e in range(n_exp)]
+    else:                                     # gate_up: weight [G = k/128, N = n_exp * n_slice]
+        idx_gf, norms_gf, cb = _pool(bit, n_slice * n_exp, k, seed)
+        info = [(starts[e], counts[e], e * n_slice, n_slice) for e in range(n_exp)]
+    x_rot = torch.randn(rows_total, k, generator=g) * 0.7
+    act, scale, o_codes, o_scale, lut, o_lut, wbs, nfac, wsb = _mode_inputs(mode, x_rot, cb)
+    norms_used = (norms_gf.float() * nfac).half() if mode == FP4 else norms_gf
+    w_dev = idx_gf.cuda()
+    if mode == FP4:
+        w_dev = ops.fold_indices_to_e2m1(w_dev, lut, bit)
+    idx = packing.unpack_nbit(idx_gf, bit, 128).long()           # [G, N, 128]
+    w_vals = o_lut[idx]                                           # lut[idx] fp32
+
+    ref = torch.zeros(rows_total, n_slice)
+    for e, (ts, cnt, ss, sc) in enumerate(info):
+        if cnt == 0:
+            continue
+        if slice_is_groups:
+            wl = w_vals[ss:ss + sc].permute(1, 0, 2).reshape(n_slice, -1)
+            nl = norms_used[ss:ss + sc].float().t()
+        else:
+            wl = w_vals[:, ss:ss + sc].permute(1, 0, 2).reshape(n_slice, -1)
+            nl = norms_used[:, ss:ss + sc].float().t()
+        ref[ts:ts + cnt] = moe.lut_gemm(o_codes[ts:ts + cnt], o_scale[ts:ts + cnt], wl, nl, 128, wbs)
+
+    info_dev = torch.tensor(info, dtype=torch.int32).cuda()
+    out = ops.matmul_merged(
+        mode, bit, STORE, act.cuda(), None if scale is None else scale.cuda(), w_dev,
+        norms_used.cuda(), None if mode == FP4 else lut.cuda(), info_dev, groups=k // 128,
+        n_out=n_slice, slice_is_groups=slice_is_groups, rows_total=rows_total, w_scale_byte=wsb, tt=tt)
+    torch.cuda.synchronize()
+    return out.cpu().float(), ref
+
+
+@pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])
+@pytest.mark.parametrize("bit", [1, 2, 4])
+@pytest.mark.parametrize("tt", [1, 2, 4])
+def test_merged_rows_gate_up(mode, bit, tt):
+    counts = [3, 0, 17, 64, 1, 130]            # ragged, an empty expert, several tiles
+    out, ref = _run_case(mode, bit, tt, counts, k=512, n_slice=128, slice_is_groups=False,
+                         seed=100 + 10 * mode + bit)
+    # only the fp16 rounding of the output (and fp32 summation order) separates the two
+    torch.testing.assert_close(out, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])
+@pytest.mark.parametrize("bit", [1, 2, 4])
+def test_merged_in_features_down(mode, bit):
+    counts = [5, 33, 0, 16]
+    out, ref = _run_case(mode, bit, 1, counts, k=256, n_slice=256, slice_is_groups=True,
+                         seed=200 + 10 * mode + bit)
+    torch.testing.assert_close(out, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("bit", [1, 2, 4])
+def test_wxa8_int32_accumulators_exact(bit):
+    """Per-group int32 accumulators of the i8 matrix cores equal an int64 numpy matmul."""
+    from dartmoq_hip import ops
+    counts = [7, 20, 1]
+    k, n_slice = 384, 128
+    starts, rows_total = _expert_rows(counts)
+    idx_gf, norms_gf, cb = _pool(bit, n_slice * len(counts), k, 300 + bit)
+    q_lut, step = luts.build_int8_codebook(cb)
+    g = torch.Generator().manual_seed(bit)
+    codes, s = actquant.quantize_act_int8(torch.randn(rows_total, k, generator=g), 128, step)
+    info = [(starts[e], counts[e], e * n_slice, n_slice) for e in range(len(counts))]
+    dbg = torch.zeros(rows_total, k // 128, n_slice, dtype=torch.int32, device="cuda")
+    ops.matmul_merged(A8, bit, STORE, codes.cuda(), s.half().cuda(), idx_gf.cuda(), norms_gf.cuda(),
+                      q_lut.cuda(), torch.tensor(info, dtype=torch.int32).cuda(), groups=k // 128,
+                      n_out=n_slice, slice_is_groups=False, rows_total=rows_total, tt=1, dbg_acc=dbg)
+    torch.cuda.synchronize()
+    w = q_lut.long()[packing.unpack_nbit(idx_gf, bit, 128).long()]          # [G, N, 128]
+    for e, (ts, cnt, ss, sc) in enumerate(info):
+        a = codes[ts:ts + cnt].long().reshape(cnt, k // 128, 128)
+        ref = torch.einsum("bgk,gnk->bgn", a, w[:, ss:ss + sc])
+        assert torch.equal(dbg[ts:ts + cnt].cpu().long(), ref)
+
+
+def test_silu_and_scatter_epilogues():
+    """gate_up with fused SiLU*up and down with fused weight + scatter-add (WxA16, 2-bit)."""
+    from dartmoq_hip import ops
+    bit, k, inter, hidden = 2, 256, 128, 256
+    counts = [9, 40, 2]
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(5)
+    idx_gf, norms_gf, cb = _pool(bit, 2 * inter * len(counts), k, 41)
+    x = (torch.randn(rows_total, k, generator=g) * 0.5).half()
+    info = [(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(len(counts))]
+    info_dev = torch.tensor(info, dtype=torch.int32).cuda()
+    common = dict(groups=k // 128, slice_is_groups=False, rows_total=rows_total, tt=1)
+    gu = ops.matmul_merged(A16, bit, STORE, x.cuda(), None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(),
+                           info_dev, n_out=2 * inter, **common).float().cpu()
+    act = ops.matmul_merged(A16, bit, SILU, x.cuda(), None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(),
+                            info_dev, n_out=inter, half_width=inter, **common).float().cpu()
+    ref_act = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    torch.testing.assert_close(act, ref_act, rtol=4e-3, atol=4e-3 * ref_act.abs().max().item())
+
+    # scatter: rows map to 12 tokens with weights; compare against STORE + index_add
+    didx, dnorms, dcb = _pool(bit, hidden, inter * len(counts), 43)
+    a = (torch.randn(rows_total, inter, generator=g) * 0.5).half()
+    dinfo = [(starts[e], counts[e], e * (inter // 128), inter // 128) for e in range(len(counts))]
+    dinfo_dev = torch.tensor(dinfo, dtype=torch.int32).cuda()
+    tok = torch.randint(0, 12, (rows_total,), generator=g, dtype=torch.int32)
+    wts = torch.rand(rows_total, generator=g)
+    dcommon = dict(groups=inter // 128, n_out=hidden, slice_is_groups=True, rows_total=rows_total, tt=1)
+    dn = ops.matmul_merged(A16, bit, STORE, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(),
+                           dinfo_dev, **dcommon).float().cpu()
+    acc = torch.zeros(12, hidden, dtype=torch.float32, device="cuda")
+    ops.matmul_merged(A16, bit, SCATTER, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(),
+                      dinfo_dev, out=acc, out_stride=hidden, row_weight=wts.cuda(),
+                      row_token=tok.cuda(), **dcommon)
+    ref = torch.zeros(12, hidden).index_add_(0, tok.long(), dn * wts.unsqueeze(1))
+    torch.testing.assert_close(acc.cpu(), ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+def test_gemm_argument_errors():
+    from dartmoq_hip import ops
+    x = torch.zeros(16, 256, dtype=torch.float16, device="cuda")
+    idx_gf, norms_gf, cb = _pool(2, 128, 256, 1)
+    info = torch.tensor([[0, 16, 0, 128]], dtype=torch.int32).cuda()
+    with pytest.raises(ValueError):            # unsupported bit width
+        ops.matmul_merged(A16, 3, STORE, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info,
+                          groups=2, n_out=128, slice_is_groups=False, rows_total=16, tt=1)
+    with pytest.raises(ValueError):            # n_out not a multiple of the wave tile
+        ops.matmul_merged(A16, 2, STORE, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info,
+                          groups=2, n_out=100, slice_is_groups=False, rows_total=16, tt=1)
+    with pytest.raises(ValueError):            # activation rows shorter than groups * 128
+        ops.matmul_merged(A16, 2, STORE, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info,
+                          groups=4, n_out=128, slice_is_groups=False, rows_total=16, tt=1)

@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""MoE-layer throughput benchmark on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W [--tokens 2048] [--sweep 1,64] [--mode wxa16]
+
+A step is one pass of the hot path (device top-k routing, permutation, rotation, gate_up
+dequant-GEMM + SiLU*up, per-expert rotation, down dequant-GEMM + scatter-add, fp16 store) over
+one batch of synthetic tokens of BASELINE configs[1]: H=2048, 256 experts, top-8, I=512, WxA16
+with mixed bit pools at ~2 bpw and Zipf(1.1)-skewed routing.  Inputs are resident in HBM when
+the timed region starts.  The 2 bpw layer (~216 MB packed) fits in the 256 MB Infinity Cache, so
+the steps rotate through three independent copies of the layer.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the gate_up dequant-GEMM of the
+largest bit pool), timed live with events on the stream it runs on; `cpu_baseline` is the CPU
+oracle (dequantize-then-matmul, fp32) timed on the host cores on a bounded sample.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG_DIR = os.path.join(ROOT, "dartmoq-qwen3.5_amd")
+for _p in (ROOT, PKG_DIR):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK = 8.0e12          # B/s, MI355X HBM3E
+MFMA_PEAK = {"wxa16": 2.5e15, "wxa8": 5.0e15, "wxfp8": 5.0e15, "wxfp4": 10.1e15}
+DTYPE = {"wxa16": "f16", "wxa8": "i8", "wxfp8": "f8e4m3", "wxfp4": "f4e2m1"}
+N_COPIES = 3
+
+
+def layer_bytes(mod, counts):
+    """Algorithmic HBM bytes of one forward: packed weights (indices + fp16 norms) of the
+    distinct routed experts plus activations in and out."""
+    h, i = mod.hidden_size, mod.intermediate_size
+    total = 0
+    per_pool = {}
+    for bit_str, bw in mod.bit_weights.items():
+        distinct = sum(1 for e in range(mod.num_experts)
+                       if counts[e] > 0 and bw.expert_offsets[e + 1] > bw.expert_offsets[e])
+        rows = sum(int(counts[e]) for e in range(mod.num_experts)
+                   if bw.expert_offsets[e + 1] > bw.expert_offsets[e])
+        per_pool[bit_str] = (distinct, rows)
+        total += distinct * mod.weight_bytes_per_expert(bw.bit)
+    return total, per_pool
+
+
+def time_steps(mods, x, logits, steps, warmup):
+    import torch
+    n = len(mods)
+    for s in range(warmup):
+        mods[s % n].forward(x, router_logits=logits)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        mods[s % n].forward(x, router_logits=logits)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def measure(mods, tokens, steps, warmup, seed, zipf, mode):
+    """Throughput of the full layer plus the live timing of its dominant kernel."""
+    import torch
+    from dartmoq_hip import ops, synthetic
+    from dartmoq_hip.moe import HipStageProfiler, forward_staged
+    mod = mods[0]
+    h, i, k = mod.hidden_size, mod.intermediate_size, mod.top_k
+    x = torch.randn(tokens, h, generator=torch.Generator().manual_seed(seed)).half().cuda()
+    logits = synthetic.zipf_logits(tokens, mod.num_experts, seed, skew=zipf).cuda()
+    sec = time_steps(mods, x, logits, steps, warmup)
+
+    # stage timing (events on the launch stream), rotating the copies like the timed loop
+    topk_w, topk_idx = ops.route_topk(logits, k)
+    reps = max(3, min(steps, 20))
+    acc = {}
+    aux = None
+    for r in range(reps + 1):
+        _out, stats, aux = forward_staged(mods[r % len(mods)], x, topk_idx, topk_w,
+                                          profiler=HipStageProfiler(True))
+        if r == 0:
+            continue                                   # first pass warms the allocator
+        for name, s in stats.items():
+            acc[name] = acc.get(name, 0.0) + s["ms"]
+    stage_ms = {n: v / reps for n, v in acc.items()}
+    counts = aux["counts"].cpu().tolist()
+    bytes_total, per_pool = layer_bytes(mod, counts)
+    bytes_total += 2 * tokens * h * 2                  # x in, y out (fp16)
+    flops = tokens * mod.flops_per_token()
+
+    # dominant kernel: gate_up GEMM of the pool with the most routed rows
+    dom = max(per_pool, key=lambda b: per_pool[b][1])
+    bit = int(dom)
+    distinct, rows = per_pool[dom]
+    gu_bytes = distinct * (2 * h * i * bit // 8 + 4 * h * i // 128) + tokens * h * 2 + rows * i * 2
+    gu_flops = 2.0 * rows * h * 2 * i
+    gu_ms = stage_ms[f"merged_gate_up.{dom}"]
+    t_hbm, t_mfma = gu_bytes / HBM_PEAK, gu_flops / MFMA_PEAK[mode]
+    if t_hbm >= t_mfma:
+        roof = {"bound": "hbm", "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
+                "unit": "GB/s"}
+    else:
+        roof = {"bound": "mfma", "achieved": gu_flops / (gu_ms * 1e-3) / 1e12,
+                "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof.update(kernel=f"dmq_gemm_gf_kernel gate_up+SiLU bit{bit}", launch_ms=gu_ms,
+                algorithmic_bytes=gu_bytes, algorithmic_flops=gu_flops,
+                distinct_experts=distinct, routed_rows=rows)
+    return {
+        "tokens": tokens, "ms_per_step": sec * 1e3, "tokens_per_s": tokens / sec,
+        "eff_tflops": flops / sec / 1e12,
+        "layer_hbm_frac": bytes_total / HBM_PEAK / sec,
+        "layer_mfma_frac": flops / MFMA_PEAK[mode] / sec,
+        "layer_algorithmic_bytes": bytes_total,
+        "gpu_stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
+        "gpu_stage_sum_ms": round(sum(stage_ms.values()), 4),
+        "tt": aux["tt"],
+    }, roof
+
+
+def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf):
+    """The CPU oracle (dequantize per call, fp32 matmuls) on a bounded sample of the workload."""
+    import torch
+    from oracle import moe as omoe, routing
+    layer = omoe.MoELayer(spec["hidden"], spec["inter"], spec["experts"], spec["top_k"], 128,
+                          expert_bit=expert_bit)
+    for b, p in pools_cpu.items():
+        layer.pools[b] = omoe.BitPool(int(b), p["gate_up"], p["down"], p["expert_offsets"])
+    torch.set_num_threads(os.cpu_count() or 1)
+    x = torch.randn(tokens, spec["hidden"], generator=torch.Generator().manual_seed(seed)).half()
+    w, idx = routing.route_topk(routing.zipf_logits(tokens, spec["experts"], seed, skew=zipf),
+                                spec["top_k"])
+    t0 = time.perf_counter()
+    omoe.reference_forward(layer, x, idx, w)
+    sec = time.perf_counter() - t0
+    return {"value": tokens / sec, "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port", "seconds": sec,
+            "sample": f"one forward of {tokens} tokens of the same layer, dequantize-per-call "
+                      f"fp32 oracle (reference_forward), {torch.get_num_threads()} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--tokens", type=int, default=2048)
+    ap.add_argument("--sweep", type=str, default="1,64")
+    ap.add_argument("--config", type=int, default=1)
+    ap.add_argument("--mode", type=str, default="wxa16", choices=list(MFMA_PEAK))
+    ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--cpu-tokens", type=int, default=16)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import dartmoq_hip
+    from dartmoq_hip import synthetic
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(3)
+    spec = synthetic.CONFIGS[args.config]
+    expert_bit = synthetic.assign_bits(spec["experts"], spec["fractions"], args.seed)
+    pools = synthetic.build_pools(spec["hidden"], spec["inter"], spec["experts"], expert_bit,
+                                  seed=args.seed, device="cuda")
+    mods = []
+    for _ in range(N_COPIES):
+        m = dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
+            pools, spec["experts"], spec["hidden"], spec["inter"], spec["top_k"], device="cuda")
+        mods.append(dartmoq_hip.convert_moe(m, args.mode))
+
+    main_res, roof = measure(mods, args.tokens, args.steps, args.warmup, args.seed, spec["zipf"],
+                             args.mode)
+    sweep = []
+    for t in [int(v) for v in args.sweep.split(",") if v]:
+        if t == args.tokens:
+            continue
+        res, r = measure(mods, t, args.steps, args.warmup, args.seed, spec["zipf"], args.mode)
+        res["roofline"] = r
+        sweep.append(res)
+
+    cpu = None
+    if not args.no_cpu:
+        pools_cpu = {b: {"gate_up": {k: (v.cpu() if torch.is_tensor(v) else v)
+                                     for k, v in p["gate_up"].items()},
+                         "down": {k: (v.cpu() if torch.is_tensor(v) else v)
+                                  for k, v in p["down"].items()},
+                         "expert_offsets": p["expert_offsets"]} for b, p in pools.items()}
+        cpu = cpu_baseline(pools_cpu, spec, expert_bit, args.cpu_tokens, args.seed, spec["zipf"])
+
+    bits = {b: sum(1 for e in expert_bit if e == int(b)) for b in pools}
+    line = {
+        "metric": "moe_layer_tokens_per_s", "value": main_res["tokens_per_s"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": DTYPE[args.mode], "data": "synthetic",
+        "config": {
+            "workload": f"configs[{args.config}]: single MoE FFN layer, {args.mode}, H={spec['hidden']} "
+                        f"E={spec['experts']} top-{spec['top_k']} I={spec['inter']} SwiGLU, "
+                        f"experts per bit {bits}, group 128, T={args.tokens} tokens, "
+                        f"{'Zipf(1.1)-skewed' if spec['zipf'] else 'uniform'} randn router logits",
+            "tokens": args.tokens, "mode": args.mode, "weight_copies_rotated": N_COPIES,
+        },
+        "eff_tflops": main_res["eff_tflops"],
+        "layer": main_res,
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "sweep": sweep,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -278,3 +278,110 @@ MOE_CLASS_BY_MODE = {
 def convert_moe(moe: WxA16BitPartitionedGroupMoE, mode: str) -> WxA16BitPartitionedGroupMoE:
     """convert_model_to_wxa8 / wxfp8 / wxfp4 for one layer (qwen35_quant_io.py:416-532)."""
     return MOE_CLASS_BY_MODE[mode].from_wxa16(moe)
+
+
+class HipStageProfiler:
+    """Event-pair stage timer on the current stream (the role of the reference's
+    CudaStageProfiler, turboquant_utils/cuda_profiler.py:51-174): ``begin_round()``,
+    ``with stage(name)``, ``end_round() -> {stage: {"ms": total, "calls": n}}``."""
+
+    def __init__(self, enabled: bool = True):
+        self.enabled = enabled
+        self._pairs = []
+
+    def begin_round(self):
+        self._pairs = []
+        if self.enabled:
+            torch.cuda.synchronize()
+
+    class _Stage:
+        def __init__(self, prof, name):
+            self.prof, self.name = prof, name
+
+        def __enter__(self):
+            if self.prof.enabled:
+                self.start = torch.cuda.Event(enable_timing=True)
+                self.stop = torch.cuda.Event(enable_timing=True)
+                self.start.record()
+            return self
+
+        def __exit__(self, *exc):
+            if self.prof.enabled:
+                self.stop.record()
+                self.prof._pairs.append((self.name, self.start, self.stop))
+            return False
+
+    def stage(self, name: str):
+        return HipStageProfiler._Stage(self, name)
+
+    def end_round(self) -> dict:
+        if not self.enabled:
+            return {}
+        torch.cuda.synchronize()
+        stats: dict[str, dict] = {}
+        for name, a, b in self._pairs:
+            s = stats.setdefault(name, {"ms": 0.0, "calls": 0})
+            s["ms"] += a.elapsed_time(b)
+            s["calls"] += 1
+        return stats
+
+
+@torch.no_grad()
+def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: torch.Tensor,
+                   topk_w: torch.Tensor, tt: int | None = None, profiler: HipStageProfiler | None = None):
+    """The same launches as dmq_moe_ffn_forward, issued stage by stage from Python so that each
+    one can be timed with events on the stream it runs on.  Returns (out fp16 [T, H], stats,
+    aux) where aux carries the routing plan (counts per expert) for byte accounting.  Stage
+    names follow the reference: sort_prep, rotation_hoisted, merged_gate_up, act_quant_down,
+    merged_down, scatter (fused into merged_down here), finalize."""
+    from ._lib import EPI_SCATTER, EPI_SILU
+    prof = profiler or HipStageProfiler(enabled=False)
+    x = x.half().contiguous()
+    tokens, hidden = x.shape
+    inter, e, k = moe.intermediate_size, moe.num_experts, moe.top_k
+    rows = tokens * k
+    if tt is None or tt <= 0:
+        tt = ops.pick_tt(rows, e)
+    rot_tt = 4 if tt == 4 else 1
+    desc, pool_arr, slice_start, slice_count, _keep = moe._descriptor()
+    prof.begin_round()
+    with prof.stage("sort_prep"):
+        plan = ops.route_permute(topk_idx.int().contiguous(), topk_w.float().contiguous(), e,
+                                 slice_start, slice_count, 16 * tt)
+    out32 = torch.zeros((tokens, hidden), dtype=torch.float32, device=x.device)
+    for pi, (bit_str, bw) in enumerate(moe.bit_weights.items()):
+        mode = moe.pool_mode(bw.bit)
+        ctx = bw.context(mode)
+        major = bool(pool_arr[pi].major)
+        gu_info, dn_info = plan["gu_info"][pi], plan["dn_info"][pi]
+        tiling = (plan["n_tiles"][pi], plan["tiles"][pi], plan["max_tiles"])
+        with prof.stage(f"rotation_hoisted.{bit_str}"):
+            if major:
+                xq, xs = ops.rotate(mode, x, bw.gu_rot, ctx["gu_extra"], tt=rot_tt)
+                row_index = plan["sorted_tokens"]
+            else:
+                xq, xs = ops.rotate_tiled(mode, x, bw.gu_rot, gu_info, tiling[0], tiling[1], 16 * tt,
+                                          tiling[2], rows, rot_per_expert=False,
+                                          extra_scale=ctx["gu_extra"],
+                                          row_index=plan["sorted_tokens"], tt=rot_tt)
+                row_index = None
+        with prof.stage(f"merged_gate_up.{bit_str}"):
+            act = ops.matmul_merged(mode, bw.bit, EPI_SILU, xq, xs, ctx["gu_w"], ctx["gu_norms"],
+                                    ctx["gu_lut"], gu_info, groups=hidden // GROUP_SIZE, n_out=inter,
+                                    half_width=inter, slice_is_groups=False, rows_total=rows,
+                                    row_index=row_index, w_scale_byte=ctx["gu_wsb"], tt=tt,
+                                    tiling=tiling)
+        with prof.stage(f"act_quant_down.{bit_str}"):
+            aq, as_ = ops.rotate_tiled(mode, act, bw.dn_rot, dn_info, tiling[0], tiling[1], 16 * tt,
+                                       tiling[2], rows, rot_per_expert=True,
+                                       extra_scale=ctx["dn_extra"], tt=rot_tt)
+        with prof.stage(f"merged_down.{bit_str}"):
+            ops.matmul_merged(mode, bw.bit, EPI_SCATTER, aq, as_, ctx["dn_w"], ctx["dn_norms"],
+                              ctx["dn_lut"], dn_info, groups=inter // GROUP_SIZE, n_out=hidden,
+                              slice_is_groups=True, rows_total=rows, out=out32, out_stride=hidden,
+                              w_scale_byte=ctx["dn_wsb"], row_weight=plan["sorted_weights"],
+                              row_token=plan["sorted_tokens"], tt=tt, tiling=tiling)
+    with prof.stage("finalize"):
+        out = ops.finalize_f16(out32)
+    stats = prof.end_round()
+    return out, stats, {"counts": plan["counts"], "tt": tt}

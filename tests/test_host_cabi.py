@@ -1,0 +1,143 @@
+"""CPU checks of the host side: the C-ABI library loads and exports every declared symbol,
+argument validation returns the documented status codes without touching a GPU, and the
+load-time host helpers agree with the oracle and the golden vectors."""
+
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import codebook as ocodebook, luts as oluts, moe as omoe, rotation as orotation
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "dartmoq_hip.h")
+GOLDEN = os.path.join(ROOT, "tests", "golden", "lut_fixtures.json")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dmq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from dartmoq_hip import _lib
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 17
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/dartmoq_hip.h but not exported"
+    assert set(declared) == set(_lib.PROTOTYPES), "ctypes prototypes and header disagree"
+    assert lib.dmq_abi_version() == 1
+    assert lib.dmq_status_string(0) == b"ok"
+    assert b"bit width" in lib.dmq_status_string(1)
+
+
+def test_argument_validation_without_gpu():
+    """Entry points reject bad arguments before any launch (status codes, no compute)."""
+    from dartmoq_hip import _lib
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.dmq_convert_to_group_first(p, p, 4, 4, 3, 0, p, p, None) == 1           # bad bit
+    assert lib.dmq_dequant_tile(p, p, None, 16, 0, 1, 8, 16, 2, p, None) == 3          # n0+n_cnt > N
+    assert lib.dmq_fold_indices_to_e2m1(p, p, 4, 8, p, None) == 1
+    assert lib.dmq_route_topk(None, 0, 1, 8, 2, 0, p, p, None) == 6                   # null logits
+    assert lib.dmq_build_tiles(p, 4, 24, 8, p, p, None) == 2                          # tile not /16
+    assert lib.dmq_finalize_f16(p, None, 7, p, None) == 2
+    assert lib.dmq_fill_zero(p, 6, None) == 2
+    a = _lib.GemmArgs()
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 1                       # bit 0
+    a.bit, a.mode, a.tt = 2, 9, 1
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # bad mode
+    a.mode = 0
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 6                       # null pointers
+    with pytest.raises(ValueError):
+        _lib.check(2, "demo")
+    with pytest.raises(TypeError):
+        _lib.check(6, "demo")
+    assert lib.dmq_moe_workspace_bytes(None, 4) == 0
+
+
+def test_workspace_size_formula():
+    from dartmoq_hip import _lib
+    lib = _lib.load()
+    d = _lib.LayerDesc()
+    d.hidden, d.inter, d.experts, d.top_k, d.pools = 2048, 512, 256, 8, 3
+    small = lib.dmq_moe_workspace_bytes(ctypes.byref(d), 64)
+    big = lib.dmq_moe_workspace_bytes(ctypes.byref(d), 4096)
+    r = 4096 * 8
+    # dominated by x codes [R, H] fp16 + act/actq [R, I] fp16 + fp32 output [T, H]
+    assert big >= r * 2048 * 2 + 2 * r * 512 * 2 + 4096 * 2048 * 4
+    assert big < 1.3 * (r * 2048 * 2 + 2 * r * 512 * 2 + 4096 * 2048 * 4) + (1 << 22)
+    assert small < big
+
+
+def test_cpu_tensors_are_rejected():
+    from dartmoq_hip import ops
+    with pytest.raises(RuntimeError):
+        ops.unpack_nbit(torch.zeros(2, 2, dtype=torch.uint8), 2)
+    with pytest.raises(RuntimeError):
+        ops.quantize_act(1, torch.zeros(2, 128, dtype=torch.float16))
+    with pytest.raises(ValueError):
+        ops.unpack_nbit(torch.zeros(2, 2, dtype=torch.uint8), 3)
+
+
+def test_host_helpers_match_oracle_and_golden():
+    from dartmoq_hip import hostprep, synthetic
+    golden = json.load(open(GOLDEN))
+    for bit in (1, 2, 4):
+        cents, bounds = hostprep.get_codebook(bit)
+        o_cents, o_bounds = ocodebook.get_codebook(bit)
+        assert torch.equal(cents, o_cents) and torch.equal(bounds, o_bounds)
+        cb = cents.half()
+        g = golden[str(bit)]
+        q, step = hostprep.build_int8_codebook(cb)
+        assert q.tolist() == g["int8"] and step == g["int8_step"]
+        f8, s8 = hostprep.build_fp8_codebook(cb)
+        assert f8.view(torch.uint8).tolist() == g["e4m3_bytes"] and s8 == g["e4m3_scale"]
+        nib, e0, resid, _ = hostprep.build_e2m1_codebook(cb)
+        assert nib.tolist() == g["e2m1_nib"] and e0 == g["e2m1_e0"] and resid == g["e2m1_residual"]
+    assert torch.equal(hostprep.generate_rotation_matrix(128, 1046), orotation.rotation_matrix(128, 1046))
+    mats = hostprep.generate_batch_rotation_matrices(128, 44, 3, 128)
+    assert torch.equal(mats, orotation.batch_rotation_matrices(128, 44, 3, 128))
+    assert synthetic.assign_bits(256, {2: 0.979, 1: 0.010, 4: 0.011}, 42) == \
+        omoe.assign_bits(256, {2: 0.979, 1: 0.010, 4: 0.011}, 42)
+
+
+def test_synthetic_quantizer_matches_oracle_on_cpu():
+    """The benchmark's layer builder produces the same packed checkpoint tensors as the oracle."""
+    from dartmoq_hip import synthetic
+    from oracle import turboquant
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(96, 256, generator=g) * 0.02).half()
+    for bit in (1, 2, 4):
+        a = synthetic.quantize_packed(w, bit, 42 + bit)
+        b = turboquant.quantize_packed(w, bit, 128, seed=42 + bit)
+        assert torch.equal(a["indices_packed"], b["indices_packed"])
+        assert torch.equal(a["norms"], b["norms"]) and torch.equal(a["codebook"], b["codebook"])
+        assert a["shape"] == b["shape"] and a["seed"] == b["seed"]
+
+
+def test_module_construction_errors():
+    import dartmoq_hip
+    with pytest.raises(TypeError):
+        dartmoq_hip.WxA8BitPartitionedGroupMoE.from_wxa16(object())
+    with pytest.raises(ValueError):
+        dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
+            {"3": {"gate_up": {}, "down": {}, "expert_offsets": [0, 1]}}, 1, 128, 128, 1, device="cpu")
+    with pytest.raises(ValueError):
+        dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
+            {"2": {"gate_up": {}, "down": {}, "expert_offsets": [0, 128, 384]}}, 2, 128, 128, 1,
+            device="cpu")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr

@@ -66,7 +66,7 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     """Throughput of the full layer plus the live timing of its dominant kernel."""
     import torch
     from dartmoq_hip import ops, synthetic
-    from dartmoq_hip.moe import HipStageProfiler, forward_staged
+    from dartmoq_hip.moe import forward_staged
     mod = mods[0]
     h, i, k = mod.hidden_size, mod.intermediate_size, mod.top_k
     x = torch.randn(tokens, h, generator=torch.Generator().manual_seed(seed)).half().cuda()
@@ -79,25 +79,30 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     acc = {}
     aux = None
     for r in range(reps + 1):
-        _out, stats, aux = forward_staged(mods[r % len(mods)], x, topk_idx, topk_w,
-                                          profiler=HipStageProfiler(True))
+        _out, stats, aux = forward_staged(mods[r % len(mods)], x, topk_idx, topk_w)
         if r == 0:
             continue                                   # first pass warms the allocator
-        for name, s in stats.items():
-            acc[name] = acc.get(name, 0.0) + s["ms"]
+        for name, ms in stats.items():
+            acc[name] = acc.get(name, 0.0) + ms
     stage_ms = {n: v / reps for n, v in acc.items()}
     counts = aux["counts"].cpu().tolist()
     bytes_total, per_pool = layer_bytes(mod, counts)
     bytes_total += 2 * tokens * h * 2                  # x in, y out (fp16)
     flops = tokens * mod.flops_per_token()
 
-    # dominant kernel: gate_up GEMM of the pool with the most routed rows
-    dom = max(per_pool, key=lambda b: per_pool[b][1])
-    bit = int(dom)
-    distinct, rows = per_pool[dom]
-    gu_bytes = distinct * (2 * h * i * bit // 8 + 4 * h * i // 128) + tokens * h * 2 + rows * i * 2
+    # dominant kernel: the merged gate_up dequant-GEMM (one launch over all bit pools).
+    # algorithmic bytes = packed gate_up indices + fp16 norms of the distinct routed experts,
+    # the rotated activations read once per token and pool, and the SiLU*up rows written
+    gu_bytes = 0
+    rows = 0
+    distinct = 0
+    for b, (d_b, r_b) in per_pool.items():
+        gu_bytes += d_b * (2 * h * i * int(b) // 8 + 4 * h * i // 128)
+        gu_bytes += (tokens if r_b else 0) * h * 2 + r_b * i * 2
+        rows += r_b
+        distinct += d_b
     gu_flops = 2.0 * rows * h * 2 * i
-    gu_ms = stage_ms[f"merged_gate_up.{dom}"]
+    gu_ms = stage_ms["merged_gate_up"]
     t_hbm, t_mfma = gu_bytes / HBM_PEAK, gu_flops / MFMA_PEAK[mode]
     if t_hbm >= t_mfma:
         roof = {"bound": "hbm", "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
@@ -107,7 +112,8 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
                 "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
-    roof.update(kernel=f"dmq_gemm_gf_kernel gate_up+SiLU bit{bit}", launch_ms=gu_ms,
+    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={aux['ks']},SILU> merged gate_up",
+                launch_ms=gu_ms,
                 algorithmic_bytes=gu_bytes, algorithmic_flops=gu_flops,
                 distinct_experts=distinct, routed_rows=rows)
     return {
@@ -118,7 +124,7 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
         "layer_algorithmic_bytes": bytes_total,
         "gpu_stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
         "gpu_stage_sum_ms": round(sum(stage_ms.values()), 4),
-        "tt": aux["tt"],
+        "tt": aux["tt"], "ks": aux["ks"], "work_items": aux["n_items"],
     }, roof
 
 

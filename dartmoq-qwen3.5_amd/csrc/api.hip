@@ -12,9 +12,22 @@ static inline int act_bytes_per_group(int mode) {
   return mode == DMQ_MODE_A16 ? 256 : (mode == DMQ_MODE_FP4 ? 64 : 128);
 }
 
+// Inside the layer workspace every code row spans K*2 bytes and every scale row 4 bytes per
+// group whatever the precision mode, so pools of different modes can share one buffer
+// without their rows overlapping.  The stride is counted in scale elements (fp16 or byte).
+static inline int scale_stride_for(int mode, int k) {
+  return mode == DMQ_MODE_FP4 ? k / 32 : k / 64;
+}
+
+static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE_FP4; }
+
+// K split across the four waves of a workgroup: small row tiles want parallelism along K,
+// large ones keep the waves on different output features
+static inline int pick_ks(int tt) { return tt == 1 ? 4 : (tt == 2 ? 2 : 1); }
+
 extern "C" {
 
-int dmq_abi_version(void) { return 1; }
+int dmq_abi_version(void) { return 2; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -73,65 +86,78 @@ int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts,
 
 int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
                       int pools, const void* slice_start, const void* slice_count, int tile_rows,
-                      int max_tiles, void* counts, void* offsets, void* sorted_tokens,
-                      void* sorted_weights, void* sorted_slots, void* gu_info, void* dn_info,
-                      void* n_tiles, void* tiles, void* stream) {
+                      int max_items, void* counts, void* offsets, void* sorted_tokens,
+                      void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
+                      void* n_items, void* items, void* stream) {
   if (!topk_idx || !topk_w || !slice_start || !slice_count || !counts || !offsets ||
-      !sorted_tokens || !sorted_weights || !gu_info || !dn_info || !n_tiles || !tiles)
+      !sorted_tokens || !sorted_weights || !sorted_rows || !gu_info || !dn_info || !n_items || !items)
     return DMQ_ERR_NULL;
   if (tokens <= 0 || k <= 0 || experts <= 0 || pools <= 0) return DMQ_ERR_SHAPE;
+  if (pools > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
   if (tile_rows <= 0 || tile_rows % 16) return DMQ_ERR_ALIGN;
-  PlanParams plan{(const int*)counts, experts, pools, tile_rows, max_tiles,
+  PlanParams plan{(const int*)counts, experts, pools, tile_rows, max_items,
                   (const int*)slice_start, (const int*)slice_count, (int*)offsets, (int*)gu_info,
-                  (int*)dn_info, (int*)n_tiles, (int*)tiles};
+                  (int*)dn_info, (int*)n_items, (int*)items};
   return dmq_route_permute_launch((const int*)topk_idx, (const float*)topk_w, tokens, k, (int*)counts,
                                   plan, (int*)sorted_tokens, (float*)sorted_weights,
-                                  (int*)sorted_slots, (hipStream_t)stream);
+                                  (int*)sorted_rows, (hipStream_t)stream);
 }
 
-int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_tiles,
-                    void* n_tiles, void* tiles, void* stream) {
-  if (!expert_info || !n_tiles || !tiles) return DMQ_ERR_NULL;
-  if (n_experts <= 0 || max_tiles <= 0) return DMQ_ERR_EMPTY;
+int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_items, int pool,
+                    void* n_items, void* items, void* stream) {
+  if (!expert_info || !n_items || !items) return DMQ_ERR_NULL;
+  if (n_experts <= 0 || max_items <= 0) return DMQ_ERR_EMPTY;
   if (tile_rows <= 0 || tile_rows % 16) return DMQ_ERR_ALIGN;
-  return dmq_tiles_from_info_launch((const int*)expert_info, n_experts, tile_rows, max_tiles,
-                                    (int*)n_tiles, (int*)tiles, (hipStream_t)stream);
-}
-
-static int rotate_common(int mode, RotParams& p, long items, int tt, void* stream) {
-  if (mode < DMQ_MODE_A16 || mode > DMQ_MODE_FP4) return DMQ_ERR_MODE;
-  if (tt != 1 && tt != 4) return DMQ_ERR_MODE;
-  if (!p.x || !p.rot || !p.out) return DMQ_ERR_NULL;
-  if (mode != DMQ_MODE_A16 && !p.scale) return DMQ_ERR_NULL;
-  if (p.groups <= 0) return DMQ_ERR_SHAPE;
-  return dmq_rotate_dispatch(mode, p, items, tt, (hipStream_t)stream);
+  if (pool < 0 || pool >= DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
+  return dmq_items_from_info_launch((const int*)expert_info, n_experts, tile_rows, max_items, pool,
+                                    (int*)n_items, (int*)items, (hipStream_t)stream);
 }
 
 int dmq_rotate(int mode, const void* x, long x_stride, const void* row_index, const void* rot,
                int rows, int groups, void* out, long out_row_bytes, void* scale, int scale_stride,
                int scale_fp32, float extra_scale, int tt, void* stream) {
   if (rows <= 0) return DMQ_OK;
-  RotParams p{(const __half*)x, x_stride, (const int*)row_index, (const __half*)rot, rows, groups, 1,
-              nullptr, nullptr, nullptr, 0, (uint8_t*)out, out_row_bytes, scale, scale_stride,
-              scale_fp32, extra_scale};
+  if (!valid_mode(mode)) return DMQ_ERR_MODE;
   if (tt != 1 && tt != 4) return DMQ_ERR_MODE;
+  if (row_index) return DMQ_ERR_MODE;    // gathered rows go through dmq_rotate_tiled
+  if (!x || !rot || !out) return DMQ_ERR_NULL;
+  if (mode != DMQ_MODE_A16 && !scale) return DMQ_ERR_NULL;
+  if (groups <= 0) return DMQ_ERR_SHAPE;
+  RotParams p{};
+  p.pool[0] = RotPool{(const __half*)rot, (uint8_t*)out, out_row_bytes, scale, scale_stride, nullptr,
+                      extra_scale, mode, 1, 0};
+  p.x = (const __half*)x; p.x_stride = x_stride; p.row_index = nullptr;
+  p.rows = rows; p.groups = groups;
+  p.n_hoisted = 1; p.hoisted_pool[0] = 0;
   const long row_tiles = (rows + 16 * tt - 1) / (16 * tt);
-  return rotate_common(mode, p, row_tiles * groups, tt, stream);
+  p.hoisted_items_per_pool = (int)(row_tiles * groups);
+  p.items = nullptr; p.n_items = nullptr; p.tile_rows = 16 * tt; p.scale_fp32 = scale_fp32;
+  return dmq_rotate_dispatch(mode, p, row_tiles * groups, tt, (hipStream_t)stream);
 }
 
 int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_index, const void* rot,
-                     int rot_per_expert, int groups, const void* expert_info, const void* tiles, const void* n_tiles,
-                     int tile_rows, int max_tiles, void* out, long out_row_bytes, void* scale,
-                     int scale_stride, int scale_fp32, float extra_scale, int tt, void* stream) {
-  if (!expert_info || !tiles || !n_tiles) return DMQ_ERR_NULL;
-  if (max_tiles <= 0) return DMQ_OK;
+                     int rot_per_expert, int groups, const void* expert_info, const void* items,
+                     const void* n_items, int tile_rows, int max_items, void* out,
+                     long out_row_bytes, void* scale, int scale_stride, int scale_fp32,
+                     float extra_scale, int tt, void* stream) {
+  if (!expert_info || !items || !n_items) return DMQ_ERR_NULL;
+  if (max_items <= 0) return DMQ_OK;
+  if (!valid_mode(mode)) return DMQ_ERR_MODE;
   if (tt != 1 && tt != 4) return DMQ_ERR_MODE;
   if (tile_rows <= 0 || tile_rows % (16 * tt)) return DMQ_ERR_ALIGN;
-  RotParams p{(const __half*)x, x_stride, (const int*)row_index, (const __half*)rot, 0, groups,
-              rot_per_expert ? 1 : 0, (const int*)expert_info, (const int*)tiles, (const int*)n_tiles, tile_rows,
-              (uint8_t*)out, out_row_bytes, scale, scale_stride, scale_fp32, extra_scale};
-  const long items = (long)max_tiles * (tile_rows / (16 * tt)) * groups;
-  return rotate_common(mode, p, items, tt, stream);
+  if (!x || !rot || !out) return DMQ_ERR_NULL;
+  if (mode != DMQ_MODE_A16 && !scale) return DMQ_ERR_NULL;
+  if (groups <= 0) return DMQ_ERR_SHAPE;
+  RotParams p{};
+  const RotPool rp{(const __half*)rot, (uint8_t*)out, out_row_bytes, scale, scale_stride,
+                   (const int*)expert_info, extra_scale, mode, 0, rot_per_expert ? 1 : 0};
+  for (int i = 0; i < DMQ_MAX_POOLS; ++i) p.pool[i] = rp;     // items may carry any pool id
+  p.x = (const __half*)x; p.x_stride = x_stride; p.row_index = (const int*)row_index;
+  p.rows = 0; p.groups = groups; p.n_hoisted = 0; p.hoisted_items_per_pool = 1;
+  p.items = (const int*)items; p.n_items = (const int*)n_items; p.tile_rows = tile_rows;
+  p.scale_fp32 = scale_fp32;
+  const long n = (long)max_items * (tile_rows / (16 * tt)) * groups;
+  return dmq_rotate_dispatch(mode, p, n, tt, (hipStream_t)stream);
 }
 
 int dmq_quantize_act(int mode, const void* x, int x_fp32, long x_stride, int rows, int groups,
@@ -147,58 +173,61 @@ int dmq_quantize_act(int mode, const void* x, int x_fp32, long x_stride, int row
 
 int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (!a) return DMQ_ERR_NULL;
-  if (a->mode < DMQ_MODE_A16 || a->mode > DMQ_MODE_FP4) return DMQ_ERR_MODE;
-  if (!dmq_valid_bit(a->bit)) return DMQ_ERR_BIT;
+  if (a->n_pools <= 0 || a->n_pools > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
+  for (int i = 0; i < a->n_pools; ++i)
+    if (!dmq_valid_bit(a->pool[i].bit)) return DMQ_ERR_BIT;
+  if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
   if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SCATTER) return DMQ_ERR_MODE;
-  if (a->tt != 1 && a->tt != 2 && a->tt != 4) return DMQ_ERR_MODE;
-  if (!a->act || !a->w || !a->norms || !a->expert_info || !a->tiles || !a->n_tiles || !a->out)
-    return DMQ_ERR_NULL;
-  if (a->mode != DMQ_MODE_FP4 && !a->lut) return DMQ_ERR_NULL;
-  if (a->mode != DMQ_MODE_A16 && !a->act_scale) return DMQ_ERR_NULL;
-  if (a->epi == DMQ_EPI_SCATTER && (!a->row_weight || !a->row_token)) return DMQ_ERR_NULL;
-  if (a->n_experts <= 0 || a->max_tiles <= 0) return DMQ_ERR_EMPTY;
-  if (a->groups <= 0 || a->n_out <= 0 || a->n_total <= 0) return DMQ_ERR_SHAPE;
+  const int ks = a->ks > 0 ? a->ks : pick_ks(a->tt);
+  if (!dmq_gemm_config_ok(a->tt, ks)) return DMQ_ERR_MODE;
+  if (!a->items || !a->n_items || !a->out) return DMQ_ERR_NULL;
+  for (int i = 0; i < a->n_pools; ++i) {
+    const dmq_gemm_pool& q = a->pool[i];
+    if (!q.act || !q.w || !q.norms || !q.expert_info) return DMQ_ERR_NULL;
+    if (q.mode == a->mode && a->mode != DMQ_MODE_FP4 && !q.lut) return DMQ_ERR_NULL;
+    if (q.mode == a->mode && a->mode != DMQ_MODE_A16 && !q.act_scale) return DMQ_ERR_NULL;
+    if (q.n_total <= 0 || q.n_total % 16) return DMQ_ERR_ALIGN;
+  }
+  if (a->epi == DMQ_EPI_SCATTER && (!a->row_weight || !a->row_slot)) return DMQ_ERR_NULL;
+  if (a->max_items <= 0) return DMQ_ERR_EMPTY;
+  if (a->groups <= 0 || a->n_out <= 0) return DMQ_ERR_SHAPE;
   const int feat_per_wave = (a->epi == DMQ_EPI_SILU) ? 32 : 64;
   if (a->n_out % feat_per_wave) return DMQ_ERR_ALIGN;
   if (a->epi == DMQ_EPI_SILU && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
-  if (a->n_total % 16) return DMQ_ERR_ALIGN;
   if (a->act_row_bytes < (long)a->groups * act_bytes_per_group(a->mode)) return DMQ_ERR_SHAPE;
 
   GemmLaunch L;
   GemmParams& p = L.p;
-  p.act = (const uint8_t*)a->act;
+  for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
+    const dmq_gemm_pool& q = a->pool[i < a->n_pools ? i : 0];
+    p.pool[i] = PoolW{(const uint8_t*)q.w, (const __half*)q.norms, q.lut, (const int*)q.expert_info,
+                      (const uint8_t*)q.act, q.act_scale, (const int*)q.row_index, q.n_total, q.bit,
+                      q.mode, q.w_scale_byte};
+  }
   p.act_row_bytes = a->act_row_bytes;
-  p.act_scale = a->act_scale;
   p.act_scale_stride = a->act_scale_stride;
-  p.row_index = (const int*)a->row_index;
-  p.w = (const uint8_t*)a->w;
-  p.norms = (const __half*)a->norms;
-  p.lut = a->lut;
-  p.n_total = a->n_total;
   p.groups = a->groups;
   p.n_out = a->n_out;
   p.half_width = a->half_width;
   p.slice_is_groups = a->slice_is_groups;
-  p.w_scale_byte = a->w_scale_byte;
-  p.expert_info = (const int*)a->expert_info;
-  p.tiles = (const int*)a->tiles;
-  p.n_tiles = (const int*)a->n_tiles;
-  const int feat_per_block = 4 * feat_per_wave;
+  p.items = (const int*)a->items;
+  p.n_items = (const int*)a->n_items;
+  const int feat_per_block = (4 / ks) * feat_per_wave;
   p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
   p.out = (__half*)a->out;
   p.out_stride = a->out_stride;
-  p.out_accum = (float*)a->out;
+  p.out_slots = (float*)a->out;
   p.row_weight = (const float*)a->row_weight;
-  p.row_token = (const int*)a->row_token;
+  p.row_slot = (const int*)a->row_slot;
   p.dbg_acc = (int*)a->dbg_acc;
-  L.bit = a->bit;
   L.epi = a->epi;
   L.tt = a->tt;
+  L.ks = ks;
   L.dbg = a->dbg_acc != nullptr;
   L.stream = (hipStream_t)stream;
-  const long max_work = (long)a->max_tiles * p.n_blocks;
-  const int resident = 256 * (a->tt == 1 ? 4 : (a->tt == 2 ? 2 : 1));
-  L.grid = (int)(max_work < resident ? max_work : resident);
+  const long work = (long)a->max_items * p.n_blocks;
+  if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
+  L.grid = (int)work;
   switch (a->mode) {
     case DMQ_MODE_A16: return dmq_gemm_launch_a16(L);
     case DMQ_MODE_A8: return dmq_gemm_launch_a8(L);
@@ -206,6 +235,15 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     case DMQ_MODE_FP4: return dmq_gemm_launch_fp4(L);
   }
   return DMQ_ERR_MODE;
+}
+
+int dmq_combine_slots(const void* slots_f32, int k, const void* add_f16, long tokens, int hidden,
+                      void* out_f16, void* stream) {
+  if (!slots_f32 || !out_f16) return DMQ_ERR_NULL;
+  if (k <= 0 || hidden <= 0) return DMQ_ERR_SHAPE;
+  if (hidden % 4) return DMQ_ERR_ALIGN;
+  return dmq_combine_launch((const float*)slots_f32, k, (const __half*)add_f16, tokens, hidden,
+                            (__half*)out_f16, (hipStream_t)stream);
 }
 
 int dmq_finalize_f16(const void* acc_f32, const void* add_f16, long n, void* out_f16, void* stream) {
@@ -229,10 +267,12 @@ int dmq_fill_zero(void* ptr, long n_bytes, void* stream) {
 
 // ------------------------------------------------------------------------------- whole layer
 struct MoeWorkspace {
-  int *counts, *offsets, *sorted_tokens, *gu_info, *dn_info, *n_tiles, *tiles;
-  float *sorted_weights, *out32;
-  uint8_t *xq, *xq_scale, *act, *actq, *actq_scale;
-  int max_tiles, tile_rows;
+  int *counts, *offsets, *sorted_tokens, *sorted_rows, *gu_info, *dn_info, *n_items, *items;
+  float *sorted_weights, *slots;
+  uint8_t* xq[DMQ_MAX_POOLS];        // hoisted pools: codes by token; others share xq_rows
+  uint8_t* xq_scale[DMQ_MAX_POOLS];
+  uint8_t *xq_rows, *xq_rows_scale, *act, *actq, *actq_scale;
+  int max_items, tile_rows;
   size_t bytes;
 };
 
@@ -248,20 +288,26 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   const size_t R = (size_t)tokens * L->top_k;
   const size_t E = L->experts, P = L->pools, H = L->hidden, I = L->inter;
   w.tile_rows = 16 * tt;
-  w.max_tiles = (int)(R / w.tile_rows + E);
+  w.max_items = (int)(R / w.tile_rows + E);
   size_t off = 0;
   auto take = [&](size_t n) { uint8_t* p = base + off; off += align_up(n); return p; };
   w.counts = (int*)take(E * 4);
   w.offsets = (int*)take((E + 1) * 4);
   w.sorted_tokens = (int*)take(R * 4);
+  w.sorted_rows = (int*)take(R * 4);
   w.sorted_weights = (float*)take(R * 4);
   w.gu_info = (int*)take(P * E * 16);
   w.dn_info = (int*)take(P * E * 16);
-  w.n_tiles = (int*)take(P * 16);
-  w.tiles = (int*)take(P * (size_t)w.max_tiles * 8);
-  w.out32 = (float*)take((size_t)tokens * H * 4);
-  w.xq = take(R * H * 2);
-  w.xq_scale = take(R * (H / DMQ_GS) * 4);
+  w.n_items = (int*)take(16);
+  w.items = (int*)take((size_t)w.max_items * 16);
+  w.slots = (float*)take(R * H * 4);
+  for (size_t i = 0; i < DMQ_MAX_POOLS; ++i) {
+    // every pool gets a by-token buffer so the size does not depend on which pools are hoisted
+    w.xq[i] = i < P ? take((size_t)tokens * H * 2) : nullptr;
+    w.xq_scale[i] = i < P ? take((size_t)tokens * (H / DMQ_GS) * 4) : nullptr;
+  }
+  w.xq_rows = take(R * H * 2);
+  w.xq_rows_scale = take(R * (H / DMQ_GS) * 4);
   w.act = take(R * I * 2);
   w.actq = take(R * I * 2);
   w.actq_scale = take(R * (I / DMQ_GS) * 4);
@@ -271,98 +317,173 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
 
 size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens) {
   if (!layer || tokens <= 0) return 0;
-  // tile size 16 gives the largest tile list; everything else is independent of tt
+  // tile size 16 gives the largest item list; everything else is independent of tt
   return carve(layer, tokens, 1, nullptr).bytes;
 }
 
 int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                         const void* topk_w, int tokens, const void* add_f16, void* out,
-                        void* workspace, size_t workspace_bytes, int tt, void* stream) {
+                        void* workspace, size_t workspace_bytes, int tt, int ks, void* stream) {
+  return dmq_moe_ffn_forward_staged(layer, x, topk_idx, topk_w, tokens, add_f16, out, workspace,
+                                    workspace_bytes, tt, ks, nullptr, nullptr, stream);
+}
+
+int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
+                               const void* topk_w, int tokens, const void* add_f16, void* out,
+                               void* workspace, size_t workspace_bytes, int tt, int ks,
+                               void* const* stage_events, void* aux_out, void* stream) {
   if (!layer || !x || !topk_idx || !topk_w || !out || !workspace || !layer->pool) return DMQ_ERR_NULL;
+  auto mark = [&](int i) {
+    if (stage_events && stage_events[i]) (void)hipEventRecord((hipEvent_t)stage_events[i], (hipStream_t)stream);
+  };
   if (tokens <= 0) return DMQ_ERR_EMPTY;
   const int H = layer->hidden, I = layer->inter, E = layer->experts, K = layer->top_k;
+  const int P = layer->pools;
   if (H % DMQ_GS || I % DMQ_GS || H / DMQ_GS < 1 || I / DMQ_GS < 1) return DMQ_ERR_ALIGN;
-  if (layer->pools <= 0 || E <= 0 || K <= 0) return DMQ_ERR_SHAPE;
+  if (P <= 0 || E <= 0 || K <= 0) return DMQ_ERR_SHAPE;
+  if (P > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
   if (tt <= 0) tt = pick_tt(tokens, K, E);
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
+  if (ks <= 0) ks = pick_ks(tt);
+  if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   const int rot_tt = (tt == 4) ? 4 : 1;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
   if (w.bytes > workspace_bytes) return DMQ_ERR_LIMIT;
-  const int R = tokens * K;
+  hipStream_t st = (hipStream_t)stream;
   int rc;
+  if (aux_out) {
+    long* aux = (long*)aux_out;
+    aux[0] = tt; aux[1] = ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
+    aux[3] = w.max_items; aux[4] = (long)((uint8_t*)w.n_items - (uint8_t*)workspace);
+  }
+  mark(0);
 
-  rc = dmq_route_permute(topk_idx, topk_w, tokens, K, E, layer->pools, layer->slice_start,
-                         layer->slice_count, w.tile_rows, w.max_tiles, w.counts, w.offsets,
-                         w.sorted_tokens, w.sorted_weights, nullptr, w.gu_info, w.dn_info,
-                         w.n_tiles, w.tiles, stream);
+  // distinct precision modes of the pools (one launch per mode and stage)
+  int modes[DMQ_MAX_POOLS], n_modes = 0;
+  for (int i = 0; i < P; ++i) {
+    const int m = layer->pool[i].mode;
+    if (!valid_mode(m)) return DMQ_ERR_MODE;
+    if (!dmq_valid_bit(layer->pool[i].bit)) return DMQ_ERR_BIT;
+    bool seen = false;
+    for (int j = 0; j < n_modes; ++j) seen |= (modes[j] == m);
+    if (!seen) modes[n_modes++] = m;
+  }
+
+  // 1. sort by expert, per-pool expert_info, work items
+  rc = dmq_route_permute(topk_idx, topk_w, tokens, K, E, P, layer->slice_start, layer->slice_count,
+                         w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
+                         w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items, w.items,
+                         stream);
   if (rc) return rc;
-  rc = dmq_fill_zero(w.out32, (long)tokens * H * 4, stream);
-  if (rc) return rc;
+  mark(1);
 
-  for (int pi = 0; pi < layer->pools; ++pi) {
-    const dmq_pool_desc& pd = layer->pool[pi];
-    const int mode = pd.mode;
-    if (mode < DMQ_MODE_A16 || mode > DMQ_MODE_FP4) return DMQ_ERR_MODE;
-    const int* gu_info = w.gu_info + (size_t)pi * E * 4;
-    const int* dn_info = w.dn_info + (size_t)pi * E * 4;
-    const int* n_tiles = w.n_tiles + pi * 4;
-    const int* tiles = w.tiles + (size_t)pi * w.max_tiles * 2;
-    const long code_row_bytes_h = (long)(H / DMQ_GS) * act_bytes_per_group(mode);
-    const long code_row_bytes_i = (long)(I / DMQ_GS) * act_bytes_per_group(mode);
-    const int sstride_h = (mode == DMQ_MODE_FP4) ? H / 32 : H / DMQ_GS;
-    const int sstride_i = (mode == DMQ_MODE_FP4) ? I / 32 : I / DMQ_GS;
-
-    // 1. gate_up input: rotate (+quantize) once per token (major pool) or per routed row
-    if (pd.major) {
-      rc = dmq_rotate(mode, x, H, nullptr, pd.gu_rot, tokens, H / DMQ_GS, w.xq, code_row_bytes_h,
-                      w.xq_scale, sstride_h, 0, pd.gu_extra_scale, rot_tt, stream);
-    } else {
-      // gate_up rotation matrices do not depend on the expert
-      rc = dmq_rotate_tiled(mode, x, H, w.sorted_tokens, pd.gu_rot, 0, H / DMQ_GS, gu_info, tiles,
-                            n_tiles, w.tile_rows, w.max_tiles, w.xq, code_row_bytes_h, w.xq_scale,
-                            sstride_h, 0, pd.gu_extra_scale, rot_tt, stream);
+  // 2. gate_up input: rotate (+quantize) once per token (hoisted pools) or per routed row
+  for (int mi = 0; mi < n_modes; ++mi) {
+    const int mode = modes[mi];
+    RotParams rp{};
+    rp.x = (const __half*)x; rp.x_stride = H; rp.row_index = w.sorted_tokens;
+    rp.rows = tokens; rp.groups = H / DMQ_GS;
+    rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0;
+    const long row_tiles = (tokens + 16 * rot_tt - 1) / (16 * rot_tt);
+    rp.hoisted_items_per_pool = (int)(row_tiles * rp.groups);
+    bool any_tiled = false;
+    for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
+      const int pi = i < P ? i : 0;
+      const dmq_pool_desc& pd = layer->pool[pi];
+      const bool live = i < P && pd.mode == mode;
+      const bool hoisted = pd.major != 0;
+      const long row_bytes = (long)H * 2;
+      rp.pool[i] = RotPool{(const __half*)pd.gu_rot, hoisted ? w.xq[pi] : w.xq_rows, row_bytes,
+                           hoisted ? (void*)w.xq_scale[pi] : (void*)w.xq_rows_scale,
+                           scale_stride_for(pd.mode, H), w.gu_info + (size_t)pi * E * 4,
+                           pd.gu_extra_scale, live ? pd.mode : -1, hoisted ? 1 : 0, 0};
+      if (live && hoisted) rp.hoisted_pool[rp.n_hoisted++] = i;
+      if (live && !hoisted) any_tiled = true;
     }
+    long n = (long)rp.n_hoisted * rp.hoisted_items_per_pool;
+    if (any_tiled) n += (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
+    else rp.items = nullptr;
+    rc = dmq_rotate_dispatch(mode, rp, n, rot_tt, st);
     if (rc) return rc;
+  }
 
-    // 2. gate_up GEMM with fused SiLU * up -> act[R, I]
+  mark(2);
+
+  // 3. gate_up GEMM with fused SiLU * up -> act[R, I]
+  for (int mi = 0; mi < n_modes; ++mi) {
+    const int mode = modes[mi];
     dmq_gemm_args g{};
-    g.mode = mode; g.bit = pd.bit; g.epi = DMQ_EPI_SILU; g.tt = tt;
-    g.act = w.xq; g.act_row_bytes = code_row_bytes_h;
-    g.act_scale = (mode == DMQ_MODE_A16) ? nullptr : w.xq_scale; g.act_scale_stride = sstride_h;
-    g.row_index = pd.major ? w.sorted_tokens : nullptr;
-    g.w = pd.gu_w; g.norms = pd.gu_norms; g.lut = pd.gu_lut;
-    g.n_total = pd.n_gate_up; g.groups = H / DMQ_GS; g.n_out = I; g.half_width = I;
-    g.slice_is_groups = 0; g.w_scale_byte = pd.gu_w_scale_byte;
-    g.expert_info = gu_info; g.n_experts = E; g.tiles = tiles; g.n_tiles = n_tiles;
-    g.max_tiles = w.max_tiles;
+    g.mode = mode; g.epi = DMQ_EPI_SILU; g.tt = tt; g.ks = ks; g.n_pools = P;
+    for (int i = 0; i < P; ++i) {
+      const dmq_pool_desc& pd = layer->pool[i];
+      const bool hoisted = pd.major != 0;
+      g.pool[i] = dmq_gemm_pool{pd.gu_w, pd.gu_norms, pd.gu_lut, w.gu_info + (size_t)i * E * 4,
+                                hoisted ? w.xq[i] : w.xq_rows,
+                                hoisted ? w.xq_scale[i] : w.xq_rows_scale,
+                                hoisted ? w.sorted_tokens : nullptr, pd.n_gate_up, pd.bit, pd.mode,
+                                pd.gu_w_scale_byte};
+    }
+    g.act_row_bytes = (long)H * 2;
+    g.act_scale_stride = scale_stride_for(mode, H);
+    g.groups = H / DMQ_GS; g.n_out = I; g.half_width = I; g.slice_is_groups = 0;
+    g.items = w.items; g.n_items = w.n_items; g.max_items = w.max_items;
     g.out = w.act; g.out_stride = I;
     rc = dmq_matmul_merged_gf(&g, stream);
     if (rc) return rc;
+  }
 
-    // 3. down input: per-expert rotation (+quantize) of act
-    rc = dmq_rotate_tiled(mode, w.act, I, nullptr, pd.dn_rot, 1, I / DMQ_GS, dn_info, tiles, n_tiles,
-                          w.tile_rows, w.max_tiles, w.actq, code_row_bytes_i, w.actq_scale,
-                          sstride_i, 0, pd.dn_extra_scale, rot_tt, stream);
+  mark(3);
+
+  // 4. down input: per-expert rotation (+quantize) of act
+  for (int mi = 0; mi < n_modes; ++mi) {
+    const int mode = modes[mi];
+    RotParams rp{};
+    rp.x = (const __half*)w.act; rp.x_stride = I; rp.row_index = nullptr;
+    rp.rows = 0; rp.groups = I / DMQ_GS; rp.n_hoisted = 0; rp.hoisted_items_per_pool = 1;
+    rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0;
+    for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
+      const int pi = i < P ? i : 0;
+      const dmq_pool_desc& pd = layer->pool[pi];
+      const bool live = i < P && pd.mode == mode;
+      rp.pool[i] = RotPool{(const __half*)pd.dn_rot, w.actq,
+                           (long)I * 2, w.actq_scale,
+                           scale_stride_for(pd.mode, I), w.dn_info + (size_t)pi * E * 4,
+                           pd.dn_extra_scale, live ? pd.mode : -1, 0, 1};
+    }
+    const long n = (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
+    rc = dmq_rotate_dispatch(mode, rp, n, rot_tt, st);
     if (rc) return rc;
+  }
 
-    // 4. down GEMM with fused routing weight + scatter-add into out32
+  mark(4);
+
+  // 5. down GEMM with fused routing weight, rows scattered to their (token, slot) rows
+  for (int mi = 0; mi < n_modes; ++mi) {
+    const int mode = modes[mi];
     dmq_gemm_args d{};
-    d.mode = mode; d.bit = pd.bit; d.epi = DMQ_EPI_SCATTER; d.tt = tt;
-    d.act = w.actq; d.act_row_bytes = code_row_bytes_i;
-    d.act_scale = (mode == DMQ_MODE_A16) ? nullptr : w.actq_scale; d.act_scale_stride = sstride_i;
-    d.row_index = nullptr;
-    d.w = pd.dn_w; d.norms = pd.dn_norms; d.lut = pd.dn_lut;
-    d.n_total = H; d.groups = I / DMQ_GS; d.n_out = H; d.half_width = 0;
-    d.slice_is_groups = 1; d.w_scale_byte = pd.dn_w_scale_byte;
-    d.expert_info = dn_info; d.n_experts = E; d.tiles = tiles; d.n_tiles = n_tiles;
-    d.max_tiles = w.max_tiles;
-    d.out = w.out32; d.out_stride = H;
-    d.row_weight = w.sorted_weights; d.row_token = w.sorted_tokens;
+    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt; d.ks = ks; d.n_pools = P;
+    for (int i = 0; i < P; ++i) {
+      const dmq_pool_desc& pd = layer->pool[i];
+      d.pool[i] = dmq_gemm_pool{pd.dn_w, pd.dn_norms, pd.dn_lut, w.dn_info + (size_t)i * E * 4,
+                                w.actq, w.actq_scale, nullptr, H, pd.bit, pd.mode,
+                                pd.dn_w_scale_byte};
+    }
+    d.act_row_bytes = (long)I * 2;
+    d.act_scale_stride = scale_stride_for(mode, I);
+    d.groups = I / DMQ_GS; d.n_out = H; d.half_width = 0; d.slice_is_groups = 1;
+    d.items = w.items; d.n_items = w.n_items; d.max_items = w.max_items;
+    d.out = w.slots; d.out_stride = H;
+    d.row_weight = w.sorted_weights; d.row_slot = w.sorted_rows;
     rc = dmq_matmul_merged_gf(&d, stream);
     if (rc) return rc;
   }
-  (void)R;
-  return dmq_finalize_f16(w.out32, add_f16, (long)tokens * H, out, stream);
+
+  mark(5);
+
+  // 6. out[t] = sum of the k slot rows of token t
+  rc = dmq_combine_slots(w.slots, K, add_f16, tokens, H, out, stream);
+  mark(6);
+  return rc;
 }
 
 }  // extern "C"

@@ -5,53 +5,52 @@
 
 struct GemmLaunch {
   GemmParams p;
-  int bit;
   int epi;
-  int tt;          // token tiles per wave: 1, 2 or 4
+  int tt;          // activation tiles of 16 rows per wave: 1, 2 or 4
+  int ks;          // waves splitting K: 1, 2 or 4
   int dbg;
   int grid;
   hipStream_t stream;
 };
 
-template <int MODE, int BIT, int TT, int EPI, bool DBG>
+// instantiated (tt, ks) pairs: decode (1,4) (1,1); mid (2,2) (2,1); prefill (4,1) (4,2)
+static inline bool dmq_gemm_config_ok(int tt, int ks) {
+  return (tt == 1 && (ks == 4 || ks == 1)) || (tt == 2 && (ks == 2 || ks == 1)) ||
+         (tt == 4 && (ks == 1 || ks == 2));
+}
+
+template <int MODE, int TT, int KS, int EPI, bool DBG>
 static int dmq_gemm_launch_one(const GemmLaunch& L) {
-  hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, BIT, 4, TT, EPI, DBG>), dim3(L.grid), dim3(256), 0,
+  hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG>), dim3(L.grid), dim3(256), 0,
                      L.stream, L.p);
   return dmq_check_launch();
 }
 
-template <int MODE, int BIT, int TT>
+template <int MODE, int TT, int KS>
 static int dmq_gemm_launch_epi(const GemmLaunch& L) {
   switch (L.epi) {
     case DMQ_EPI_STORE:
-      if (MODE == DMQ_MODE_A8 && TT == 1 && L.dbg)
-        return dmq_gemm_launch_one<MODE, BIT, TT, DMQ_EPI_STORE, (MODE == DMQ_MODE_A8 && TT == 1)>(L);
-      return dmq_gemm_launch_one<MODE, BIT, TT, DMQ_EPI_STORE, false>(L);
-    case DMQ_EPI_SILU: return dmq_gemm_launch_one<MODE, BIT, TT, DMQ_EPI_SILU, false>(L);
-    case DMQ_EPI_SCATTER: return dmq_gemm_launch_one<MODE, BIT, TT, DMQ_EPI_SCATTER, false>(L);
-  }
-  return DMQ_ERR_MODE;
-}
-
-template <int MODE, int BIT>
-static int dmq_gemm_launch_tt(const GemmLaunch& L) {
-  if (L.dbg && !(MODE == DMQ_MODE_A8 && L.tt == 1 && L.epi == DMQ_EPI_STORE)) return DMQ_ERR_MODE;
-  switch (L.tt) {
-    case 1: return dmq_gemm_launch_epi<MODE, BIT, 1>(L);
-    case 2: return dmq_gemm_launch_epi<MODE, BIT, 2>(L);
-    case 4: return dmq_gemm_launch_epi<MODE, BIT, 4>(L);
+      if constexpr (MODE == DMQ_MODE_A8 && TT == 1 && KS == 1) {
+        if (L.dbg) return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_STORE, true>(L);
+      }
+      return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_STORE, false>(L);
+    case DMQ_EPI_SILU: return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_SILU, false>(L);
+    case DMQ_EPI_SCATTER: return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_SCATTER, false>(L);
   }
   return DMQ_ERR_MODE;
 }
 
 template <int MODE>
-static int dmq_gemm_launch_bits(const GemmLaunch& L) {
-  switch (L.bit) {
-    case 1: return dmq_gemm_launch_tt<MODE, 1>(L);
-    case 2: return dmq_gemm_launch_tt<MODE, 2>(L);
-    case 4: return dmq_gemm_launch_tt<MODE, 4>(L);
-  }
-  return DMQ_ERR_BIT;
+static int dmq_gemm_launch_mode(const GemmLaunch& L) {
+  if (L.dbg && !(MODE == DMQ_MODE_A8 && L.tt == 1 && L.ks == 1 && L.epi == DMQ_EPI_STORE))
+    return DMQ_ERR_MODE;
+  if (L.tt == 1 && L.ks == 4) return dmq_gemm_launch_epi<MODE, 1, 4>(L);
+  if (L.tt == 1 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 1, 1>(L);
+  if (L.tt == 2 && L.ks == 2) return dmq_gemm_launch_epi<MODE, 2, 2>(L);
+  if (L.tt == 2 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 2, 1>(L);
+  if (L.tt == 4 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 4, 1>(L);
+  if (L.tt == 4 && L.ks == 2) return dmq_gemm_launch_epi<MODE, 4, 2>(L);
+  return DMQ_ERR_MODE;
 }
 
 // one definition per mode translation unit

@@ -2,8 +2,12 @@
 //
 //   out[r, n] = sum_g  s_a[r, g] * norm[g, n] * sum_{k<128} a[r, g, k] * LUT[idx[g, n, k]]
 //
-// One wave owns NT tiles of 16 weight rows and TT tiles of 16 activation rows and walks
-// the K dimension one quantization group (128 features) at a time:
+// One launch covers every bit pool of a layer: a work item is (pool, expert, tile of 16*TT
+// activation rows) and a workgroup of four waves handles one item for one block of output
+// features.  Inside the workgroup the waves split the output features (ROWPARTS) and / or the
+// quantization groups (KS way split of K, reduced through LDS at the end); each wave owns NT
+// tiles of 16 weight rows and TT tiles of 16 activation rows and walks its share of K one
+// group (128 features) at a time:
 //
 //   * weights are the MFMA "A" operand: lane (n = lane % 16, q = lane / 16) owns the 32
 //     features [32q, 32q+32) of row n inside the group, i.e. 4*BIT consecutive packed
@@ -20,34 +24,40 @@
 #include "common.h"
 #include "lut.h"
 
-struct GemmParams {
-  // activations
-  const uint8_t* act;          // row-major codes; row stride in bytes below
-  long act_row_bytes;
-  const void* act_scale;       // A8/FP8: fp16 [rows, act_scale_stride]; FP4: u8 [rows, act_scale_stride]
-  int act_scale_stride;
-  const int* row_index;        // optional gather: physical activation row of logical row r
-  // weights (one bit pool)
+#define DMQ_MAX_POOLS 4
+
+struct PoolW {
   const uint8_t* w;            // [G_total, n_total, ppg] packed indices (FP4: folded e2m1, ppg = 64)
   const __half* norms;         // [G_total, n_total] fp16, already divided by sqrt(128)
   const void* lut;             // fp16 / int8 / e4m3 codebook (unused for FP4)
+  const int* expert_info;      // [n_experts, 4] token_start, token_count, slice_start, slice_count
+  const uint8_t* act;          // activation codes of this pool, row-major
+  const void* act_scale;       // A8/FP8: fp16 [rows, stride]; FP4: u8 [rows, stride]
+  const int* row_index;        // optional gather: physical activation row of logical row r
   int n_total;
+  int bit;
+  int mode;                    // items of pools whose mode differs from the kernel's are skipped
+  int w_scale_byte;            // FP4: constant e8m0 byte of the weight blocks
+};
+
+struct GemmParams {
+  PoolW pool[DMQ_MAX_POOLS];
+  long act_row_bytes;
+  int act_scale_stride;
   int groups;                  // groups contracted per expert (K / 128)
   int n_out;                   // output features per activation row
   int half_width;              // SiLU epilogue: I (gate rows [0,I), up rows [I,2I) of the slice)
   int slice_is_groups;         // 0: slice_start offsets weight rows; 1: offsets groups (down)
-  int w_scale_byte;            // FP4: constant e8m0 byte of the weight blocks
   // work list
-  const int* expert_info;      // [n_experts, 4] token_start, token_count, slice_start, slice_count
-  const int* tiles;            // [*, 2] expert index, token tile index inside the expert
-  const int* n_tiles;          // device scalar
+  const int* items;            // [*, 4] pool, expert index, token tile inside the expert, unused
+  const int* n_items;          // device scalar
   int n_blocks;                // workgroups along the output features
   // outputs
   __half* out;                 // STORE / SILU: fp16 [rows, out_stride]
   long out_stride;
-  float* out_accum;            // SCATTER: fp32 [tokens, out_stride]
-  const float* row_weight;     // SCATTER: routing weight of logical row r
-  const int* row_token;        // SCATTER: destination token of logical row r
+  float* out_slots;            // SLOT: fp32 [rows, out_stride] addressed by row_slot[r]
+  const float* row_weight;     // SLOT: routing weight of logical row r
+  const int* row_slot;         // SLOT: destination row (token * top_k + slot) of logical row r
   int* dbg_acc;                // optional int32 [rows, groups, n_out] per-group accumulators (A8)
 };
 
@@ -99,84 +109,83 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
   }
 }
 
-template <int MODE, int BIT, int NT, int TT, int EPI, bool DBG>
-__global__ __launch_bounds__(256)
-void dmq_gemm_gf_kernel(GemmParams p) {
+// LDS needed by the K-split reduction: every wave parks NT*TT tiles of 64 lanes x 4 floats
+template <int NT, int TT, int KS> struct RedGeom {
+  static constexpr int FLOATS = (KS > 1) ? 4 * NT * TT * 256 : 4; };
+
+template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
+__device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
+                                              float* red, int eidx, int ttile, int nb) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   constexpr int WW = WeightWords<MODE, BIT>::N;
   constexpr int AW = T::ACT_WORDS;
-  constexpr int WAVES = 4;
-  constexpr int FEAT_TILES = (EPI == DMQ_EPI_SILU) ? NT / 2 : NT;   // output tiles per wave
+  constexpr int ROWPARTS = 4 / KS;                                   // waves along the features
+  constexpr int UNIT = (EPI == DMQ_EPI_SILU) ? 2 : 1;                // tiles finalized together
+  constexpr int UNITS = NT / UNIT;
+  constexpr int FEAT_TILES = NT / UNIT;                              // output tiles per wave
   constexpr int PPG = (MODE == DMQ_MODE_FP4) ? 64 : (DMQ_GS * BIT / 8);
-  static_assert(EPI != DMQ_EPI_SILU || (NT % 2 == 0), "SiLU epilogue pairs gate/up tiles");
+  static_assert(NT % UNIT == 0, "SiLU epilogue pairs gate/up tiles");
 
-  __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
-  if (MODE != DMQ_MODE_FP4) {
-    dmq_lut_build<BIT, T::ES>(tbl, p.lut);
-    __syncthreads();
-  }
+  if (MODE != DMQ_MODE_FP4) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
+  __syncthreads();
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int l16 = lane & 15;
   const int q = lane >> 4;
+  const int kpart = wave % KS;
+  const int rowpart = wave / KS;
   const uint32_t lane_base = (MODE == DMQ_MODE_FP4) ? 0u : dmq_lut_lane_base<BIT, T::ES>(lane);
 
-  const int total = p.n_tiles[0] * p.n_blocks;
-  for (int work = blockIdx.x; work < total; work += gridDim.x) {
-    const int tile = work / p.n_blocks;
-    const int nb = work - tile * p.n_blocks;
-    const int eidx = p.tiles[2 * tile];
-    const int ttile = p.tiles[2 * tile + 1];
-    const int token_start = p.expert_info[4 * eidx + 0];
-    const int token_count = p.expert_info[4 * eidx + 1];
-    const int slice_start = p.expert_info[4 * eidx + 2];
+  const int token_start = pw.expert_info[4 * eidx + 0];
+  const int token_count = pw.expert_info[4 * eidx + 1];
+  const int slice_start = pw.expert_info[4 * eidx + 2];
 
-    const int feat0 = (nb * WAVES + wave) * (FEAT_TILES * 16);     // first output feature of the wave
-    if (feat0 >= p.n_out) continue;
+  const int feat0 = (nb * ROWPARTS + rowpart) * (FEAT_TILES * 16);   // first output feature of the wave
+  const bool wave_active = feat0 < p.n_out;                          // wave-uniform
 
-    // weight row of each n-tile and its first group
-    int wrow[NT];
+  // weight row of each n-tile
+  int wrow[NT];
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      if (EPI == DMQ_EPI_SILU) {
-        wrow[j] = slice_start + ((j & 1) ? p.half_width : 0) + feat0 + (j >> 1) * 16;
-      } else {
-        wrow[j] = (p.slice_is_groups ? 0 : slice_start) + feat0 + j * 16;
-      }
-    }
-    const int g_base = p.slice_is_groups ? slice_start : 0;
+  for (int j = 0; j < NT; ++j) {
+    if (EPI == DMQ_EPI_SILU) wrow[j] = slice_start + ((j & 1) ? p.half_width : 0) + feat0 + (j >> 1) * 16;
+    else wrow[j] = (p.slice_is_groups ? 0 : slice_start) + feat0 + j * 16;
+  }
+  const int g_base = p.slice_is_groups ? slice_start : 0;
+  const int g_lo = (p.groups * kpart) / KS;
+  const int g_hi = (p.groups * (kpart + 1)) / KS;
 
-    // activation rows of each token tile
-    const int r_first = token_start + ttile * (16 * TT);
-    const int r_end = token_start + token_count;
-    const uint8_t* arow[TT];
-    bool avalid[TT];
-    int rlog[TT];
-    int rphys[TT];
+  // activation rows of each token tile
+  const int r_first = token_start + ttile * (16 * TT);
+  const int r_end = token_start + token_count;
+  const uint8_t* arow[TT];
+  bool avalid[TT];
+  int rlog[TT];
+  int rphys[TT];
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-      rlog[t] = r_first + t * 16 + l16;
-      avalid[t] = rlog[t] < r_end;
-      rphys[t] = avalid[t] ? (p.row_index ? p.row_index[rlog[t]] : rlog[t]) : 0;
-      arow[t] = p.act + (long)rphys[t] * p.act_row_bytes + q * (AW * 4);
-    }
+  for (int t = 0; t < TT; ++t) {
+    rlog[t] = r_first + t * 16 + l16;
+    avalid[t] = rlog[t] < r_end;
+    rphys[t] = avalid[t] ? (pw.row_index ? pw.row_index[rlog[t]] : rlog[t]) : 0;
+    arow[t] = pw.act + (long)rphys[t] * p.act_row_bytes + q * (AW * 4);
+  }
 
-    float4_t total_acc[NT][TT];
+  float4_t total_acc[NT][TT];
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int t = 0; t < TT; ++t) total_acc[j][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < TT; ++t) total_acc[j][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
+  if (wave_active && g_lo < g_hi) {
     uint32_t pk_n[NT][WW];
     uint32_t xa_n[TT][AW];
 
     auto fetch = [&](int g) {
-      const long gg = (long)(g_base + g) * p.n_total;
+      const long gg = (long)(g_base + g) * pw.n_total;
 #pragma unroll
       for (int j = 0; j < NT; ++j)
-        dmq_load_words<WW>(p.w + (gg + wrow[j] + l16) * PPG + q * (WW * 4), pk_n[j]);
+        dmq_load_words<WW>(pw.w + (gg + wrow[j] + l16) * PPG + q * (WW * 4), pk_n[j]);
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
         if (avalid[t]) {
@@ -188,8 +197,8 @@ void dmq_gemm_gf_kernel(GemmParams p) {
       }
     };
 
-    fetch(0);
-    for (int g = 0; g < p.groups; ++g) {
+    fetch(g_lo);
+    for (int g = g_lo; g < g_hi; ++g) {
       uint32_t pk[NT][WW];
       uint32_t xa[TT][AW];
 #pragma unroll
@@ -202,11 +211,11 @@ void dmq_gemm_gf_kernel(GemmParams p) {
         for (int i = 0; i < AW; ++i) xa[t][i] = xa_n[t][i];
 
       // per-group scales: 4 consecutive norms per n-tile, one activation scale per token tile
-      const long gg = (long)(g_base + g) * p.n_total;
+      const long gg = (long)(g_base + g) * pw.n_total;
       float nrm[NT][4];
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        half4_t h = *(const half4_t*)(p.norms + gg + wrow[j] + 4 * q);
+        half4_t h = *(const half4_t*)(pw.norms + gg + wrow[j] + 4 * q);
         nrm[j][0] = (float)h[0]; nrm[j][1] = (float)h[1];
         nrm[j][2] = (float)h[2]; nrm[j][3] = (float)h[3];
       }
@@ -216,15 +225,15 @@ void dmq_gemm_gf_kernel(GemmParams p) {
       for (int t = 0; t < TT; ++t) {
         xs[t] = 1.0f; xsb[t] = 127;
         if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
-          xs[t] = avalid[t] ? (float)((const __half*)p.act_scale)[(long)rphys[t] * p.act_scale_stride + g]
+          xs[t] = avalid[t] ? (float)((const __half*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g]
                             : 0.f;
         } else if (MODE == DMQ_MODE_FP4) {
           if (avalid[t])
-            xsb[t] = ((const uint8_t*)p.act_scale)[(long)rphys[t] * p.act_scale_stride + g * 4 + q];
+            xsb[t] = ((const uint8_t*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g * 4 + q];
         }
       }
 
-      if (g + 1 < p.groups) fetch(g + 1);
+      if (g + 1 < g_hi) fetch(g + 1);
 
       acc_t acc[NT][TT];
 #pragma unroll
@@ -236,7 +245,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
       for (int s = 0; s < T::STEPS; ++s) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          if (MODE == DMQ_MODE_A16) {
+          if constexpr (MODE == DMQ_MODE_A16) {
             uint32_t wq[4];
             dmq_dequant_step<MODE, BIT>(tbl, lane_base, pk[j], s, wq);
             half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[0], wq[1], wq[2], wq[3]});
@@ -246,7 +255,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
                                                                 xa[t][4 * s + 2], xa[t][4 * s + 3]});
               acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j][t], 0, 0, 0);
             }
-          } else if (MODE == DMQ_MODE_A8) {
+          } else if constexpr (MODE == DMQ_MODE_A8) {
             uint32_t wq[4];
             dmq_dequant_step<MODE, BIT>(tbl, lane_base, pk[j], s, wq);
             int4_t a = {(int)wq[0], (int)wq[1], (int)wq[2], (int)wq[3]};
@@ -256,7 +265,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
                           (int)xa[t][4 * s + 3]};
               acc[j][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[j][t], 0, 0, 0);
             }
-          } else if (MODE == DMQ_MODE_FP8) {
+          } else if constexpr (MODE == DMQ_MODE_FP8) {
             uint32_t wq[2];
             dmq_dequant_step<MODE, BIT>(tbl, lane_base, pk[j], s, wq);
             long a = (long)(((uint64_t)wq[1] << 32) | wq[0]);
@@ -271,7 +280,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
             for (int t = 0; t < TT; ++t) {
               int8_t8 b = {(int)xa[t][0], (int)xa[t][1], (int)xa[t][2], (int)xa[t][3], 0, 0, 0, 0};
               acc[j][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                  a, b, acc[j][t], 4, 4, 0, p.w_scale_byte, 0, xsb[t]);
+                  a, b, acc[j][t], 4, 4, 0, pw.w_scale_byte, 0, xsb[t]);
             }
           }
         }
@@ -294,36 +303,90 @@ void dmq_gemm_gf_kernel(GemmParams p) {
           }
         }
     }
+  }
 
-    // ------------------------------------------------------------------ epilogue
+  // ------------------------------------------------------------------ K-split reduction
+  // unit u (a tile, or a gate/up pair) is finalized by the wave with kpart == owner(u); the
+  // other waves of the K group park their partial sums in LDS.
+  if (KS > 1) {
+    float4_t* red4 = (float4_t*)red;
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-      if (!avalid[t]) continue;
-      if (EPI == DMQ_EPI_STORE) {
+    for (int j = 0; j < NT; ++j) {
+      const int owner = ((j / UNIT) * KS) / UNITS;
+      if (kpart != owner) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          half4_t h = {(_Float16)total_acc[j][t][0], (_Float16)total_acc[j][t][1],
-                       (_Float16)total_acc[j][t][2], (_Float16)total_acc[j][t][3]};
-          *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + j * 16 + 4 * q) = h;
-        }
-      } else if (EPI == DMQ_EPI_SILU) {
-#pragma unroll
-        for (int j = 0; j < NT; j += 2) {
-          half4_t h;
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
-          *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + (j >> 1) * 16 + 4 * q) = h;
-        }
-      } else {
-        const float rw = p.row_weight[rlog[t]];
-        float* dst = p.out_accum + (long)p.row_token[rlog[t]] * p.out_stride;
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            atomicAdd(dst + feat0 + j * 16 + 4 * q + r, total_acc[j][t][r] * rw);
+        for (int t = 0; t < TT; ++t)
+          red4[((wave * NT + j) * TT + t) * 64 + lane] = total_acc[j][t];
       }
     }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int owner = ((j / UNIT) * KS) / UNITS;
+      if (kpart == owner) {
+#pragma unroll
+        for (int o = 0; o < KS; ++o) {
+          if (o == owner) continue;
+          const int src = rowpart * KS + o;
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            float4_t v = red4[((src * NT + j) * TT + t) * 64 + lane];
+            total_acc[j][t] += v;
+          }
+        }
+      }
+    }
+  }
+  if (!wave_active) return;
+
+  // ------------------------------------------------------------------ epilogue
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    if (!avalid[t]) continue;
+#pragma unroll
+    for (int j = 0; j < NT; j += UNIT) {
+      if (KS > 1 && kpart != ((j / UNIT) * KS) / UNITS) continue;
+      if (EPI == DMQ_EPI_STORE) {
+        half4_t h = {(_Float16)total_acc[j][t][0], (_Float16)total_acc[j][t][1],
+                     (_Float16)total_acc[j][t][2], (_Float16)total_acc[j][t][3]};
+        *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + j * 16 + 4 * q) = h;
+      } else if (EPI == DMQ_EPI_SILU) {
+        half4_t h;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
+        *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + (j >> 1) * 16 + 4 * q) = h;
+      } else {
+        const float rw = p.row_weight[rlog[t]];
+        float4_t v = total_acc[j][t] * rw;
+        *(float4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat0 + j * 16 + 4 * q) = v;
+      }
+    }
+  }
+}
+
+template <int MODE, int TT, int EPI, int KS, bool DBG>
+__global__ __launch_bounds__(256)
+void dmq_gemm_gf_kernel(GemmParams p) {
+  constexpr int NT = 4;
+  __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
+  __shared__ __attribute__((aligned(16))) float red[RedGeom<NT, TT, KS>::FLOATS];
+
+  const int item = blockIdx.x / p.n_blocks;
+  if (item >= p.n_items[0]) return;
+  const int nb = blockIdx.x - item * p.n_blocks;
+  const int pool = p.items[4 * item + 0];
+  const int eidx = p.items[4 * item + 1];
+  const int ttile = p.items[4 * item + 2];
+  const PoolW& pw = p.pool[pool];
+  if (pw.mode != MODE) return;
+  if constexpr (MODE == DMQ_MODE_FP4) {
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb);
+    return;
+  }
+  switch (pw.bit) {
+    case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb); break;
+    case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb); break;
+    default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb); break;
   }
 }

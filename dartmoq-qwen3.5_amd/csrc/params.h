@@ -3,27 +3,35 @@
 #pragma once
 #include "common.h"
 
-struct RotParams {
-  const __half* x;         // [*, x_stride] fp16
-  long x_stride;
-  const int* row_index;    // optional: physical input row of logical row r
+#define DMQ_MAX_POOLS 4
+
+struct RotPool {
   const __half* rot;       // [*, 128, 128] fp16
-  int rows;                // logical rows (ignored when tiles are given)
-  int groups;              // groups per row
-  int rot_use_slice;       // tiled mode: 1 = matrices start at the expert's slice_start (down), 0 = at 0
-  // optional per-expert tiling: rows of a tile come from expert_info, matrices start at
-  // rot group (slice_start + g)
-  const int* expert_info;
-  const int* tiles;
-  const int* n_tiles;
-  int tile_rows;           // rows per entry of `tiles` (multiple of 16*TT)
-  // outputs (logical row r)
-  uint8_t* out;
+  uint8_t* out;            // codes by logical row
   long out_row_bytes;
   void* scale;             // fp16 / fp32 [rows, scale_stride] or u8 [rows, scale_stride] (FP4)
   int scale_stride;
-  int scale_fp32;
+  const int* expert_info;  // tiled pools: [n_experts, 4]
   float extra_scale;
+  int mode;                // pools whose mode differs from the kernel's are skipped
+  int hoisted;             // 1: every input row is rotated once; 0: rows follow the work items
+  int rot_use_slice;       // tiled: 1 = matrices start at the expert's slice_start (down), 0 = at 0
+};
+
+struct RotParams {
+  RotPool pool[DMQ_MAX_POOLS];
+  const __half* x;         // [*, x_stride] fp16
+  long x_stride;
+  const int* row_index;    // tiled pools: physical input row of logical row r (optional)
+  int rows;                // hoisted pools: number of input rows
+  int groups;              // groups per row
+  int n_hoisted;
+  int hoisted_pool[DMQ_MAX_POOLS];
+  int hoisted_items_per_pool;   // ceil(rows / (16*TT)) * groups
+  const int* items;        // [*, 4] pool, expert, row tile, unused
+  const int* n_items;
+  int tile_rows;           // rows per work item (multiple of 16*TT)
+  int scale_fp32;
 };
 
 struct QuantParams {
@@ -43,15 +51,15 @@ struct PlanParams {
   const int* counts;
   int experts;
   int pools;
-  int tile_rows;                 // rows per tile
-  int max_tiles;                 // capacity of each pool's tile list
+  int tile_rows;                 // rows per work item
+  int max_items;                 // capacity of the work-item list
   const int* slice_start_rows;   // [pools, experts] gate_up slice start (2*start) or -1 if not a member
   const int* slice_count_rows;   // [pools, experts] gate_up slice count (2*I)
   int* offsets;                  // [experts + 1]
   int* gu_info;                  // [pools, experts, 4]
   int* dn_info;                  // [pools, experts, 4]  slice in groups: start/128, I/128
-  int* n_tiles;                  // [pools, 4]
-  int* tiles;                    // [pools, max_tiles, 2]
+  int* n_items;                  // [1]
+  int* items;                    // [max_items, 4]
 };
 
 int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream);
@@ -60,9 +68,11 @@ int dmq_route_topk_launch(const void* logits, int logits_fp16, int tokens, int e
                           int renorm, float* out_w, int* out_idx, hipStream_t stream);
 int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int tokens, int k,
                              int* counts, const PlanParams& plan, int* sorted_tokens,
-                             float* sorted_weights, int* sorted_slots, hipStream_t stream);
-int dmq_tiles_from_info_launch(const int* expert_info, int experts, int tile_rows, int max_tiles,
-                               int* n_tiles, int* tiles, hipStream_t stream);
+                             float* sorted_weights, int* sorted_rows, hipStream_t stream);
+int dmq_items_from_info_launch(const int* expert_info, int experts, int tile_rows, int max_items,
+                               int pool, int* n_items, int* items, hipStream_t stream);
+int dmq_combine_launch(const float* slots, int k, const __half* add, long tokens, int hidden,
+                       __half* out, hipStream_t stream);
 int dmq_unpack_launch(const uint8_t* packed, long n_bytes, int bit, uint8_t* out, hipStream_t s);
 int dmq_dequant_tile_launch(const uint8_t* idx_gf, const __half* cb, const __half* norms, int n_total,
                             int g0, int g_cnt, int n0, int n_cnt, int bit, __half* out, hipStream_t s);

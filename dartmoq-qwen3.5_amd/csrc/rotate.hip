@@ -13,8 +13,12 @@
 // "A" operand, activation rows the "B" operand, so lane (t = lane % 16, q = lane / 16) ends
 // up with the 32 rotated values j = 16*jt + 4q + r (jt < 8, r < 4) of row t; the row maximum
 // is a 32-value in-lane reduction plus two cross-lane steps.
+//
+// One launch serves every bit pool of a layer.  "Hoisted" pools rotate all input rows once
+// (the rotation of gate_up does not depend on the expert); the others rotate only the rows
+// routed to their experts, following the layer's work-item list, and may pick the matrix by
+// expert (the down rotations).
 #include "params.h"
-
 
 __device__ __forceinline__ float wave_max16x4(float v) {
   v = fmaxf(v, __shfl_xor(v, 16, 64));
@@ -32,26 +36,38 @@ void dmq_rotate_kernel(RotParams p) {
   constexpr int ROWS_PER_ITEM = 16 * TT;
 
   long item = (long)blockIdx.x * 4 + wave;
-  const int g = (int)(item % p.groups);
-  const long rt = item / p.groups;
-
-  int r_first, r_end, rot_g;
-  if (p.tiles) {
-    const int sub = p.tile_rows / ROWS_PER_ITEM;          // items per tile entry
-    const long tile = rt / sub;
-    if (tile >= p.n_tiles[0]) return;
-    const int eidx = p.tiles[2 * tile];
-    const int ttile = p.tiles[2 * tile + 1];
-    const int ts = p.expert_info[4 * eidx + 0];
-    const int tc = p.expert_info[4 * eidx + 1];
-    r_first = ts + ttile * p.tile_rows + (int)(rt % sub) * ROWS_PER_ITEM;
-    r_end = ts + tc;
-    rot_g = (p.rot_use_slice ? p.expert_info[4 * eidx + 2] : 0) + g;
-  } else {
-    r_first = (int)rt * ROWS_PER_ITEM;
+  int pool, g, r_first, r_end, rot_g;
+  const int* row_index = nullptr;
+  const long hoisted_total = (long)p.n_hoisted * p.hoisted_items_per_pool;
+  if (item < hoisted_total) {
+    pool = p.hoisted_pool[item / p.hoisted_items_per_pool];
+    const long local = item % p.hoisted_items_per_pool;
+    g = (int)(local % p.groups);
+    r_first = (int)(local / p.groups) * ROWS_PER_ITEM;
     r_end = p.rows;
     rot_g = g;
+  } else {
+    if (!p.items) return;
+    item -= hoisted_total;
+    g = (int)(item % p.groups);
+    const long rt = item / p.groups;
+    const int sub = p.tile_rows / ROWS_PER_ITEM;          // waves per work item
+    const long tile = rt / sub;
+    if (tile >= p.n_items[0]) return;
+    pool = p.items[4 * tile];
+    if (p.pool[pool].hoisted) return;
+    const int eidx = p.items[4 * tile + 1];
+    const int ttile = p.items[4 * tile + 2];
+    const int* info = p.pool[pool].expert_info;
+    const int ts = info[4 * eidx + 0];
+    const int tc = info[4 * eidx + 1];
+    r_first = ts + ttile * p.tile_rows + (int)(rt % sub) * ROWS_PER_ITEM;
+    r_end = ts + tc;
+    rot_g = (p.pool[pool].rot_use_slice ? info[4 * eidx + 2] : 0) + g;
+    row_index = p.row_index;
   }
+  const RotPool& rp = p.pool[pool];
+  if (rp.mode != MODE) return;
   if (r_first >= r_end) return;
 
   int rlog[TT];
@@ -61,10 +77,10 @@ void dmq_rotate_kernel(RotParams p) {
   for (int t = 0; t < TT; ++t) {
     rlog[t] = r_first + t * 16 + l16;
     valid[t] = rlog[t] < r_end;
-    int phys = valid[t] ? (p.row_index ? p.row_index[rlog[t]] : rlog[t]) : 0;
+    int phys = valid[t] ? (row_index ? row_index[rlog[t]] : rlog[t]) : 0;
     xrow[t] = p.x + (long)phys * p.x_stride + g * DMQ_GS + 8 * q;
   }
-  const __half* prow = p.rot + (long)rot_g * (DMQ_GS * DMQ_GS) + (long)l16 * DMQ_GS + 8 * q;
+  const __half* prow = rp.rot + (long)rot_g * (DMQ_GS * DMQ_GS) + (long)l16 * DMQ_GS + 8 * q;
 
   float4_t acc[8][TT];
 #pragma unroll
@@ -91,7 +107,7 @@ void dmq_rotate_kernel(RotParams p) {
 
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
-    uint8_t* orow = p.out + (long)rlog[t] * p.out_row_bytes;
+    uint8_t* orow = rp.out + (long)rlog[t] * rp.out_row_bytes;
     if (MODE == DMQ_MODE_A16) {
       if (!valid[t]) continue;
 #pragma unroll
@@ -129,9 +145,9 @@ void dmq_rotate_kernel(RotParams p) {
         *(uint32_t*)(orow + g * DMQ_GS + j * 16 + 4 * q) = word;
       }
       if (q == 0) {
-        const float stored = sc * p.extra_scale;
-        if (p.scale_fp32) ((float*)p.scale)[(long)rlog[t] * p.scale_stride + g] = stored;
-        else ((__half*)p.scale)[(long)rlog[t] * p.scale_stride + g] = __float2half_rn(stored);
+        const float stored = sc * rp.extra_scale;
+        if (p.scale_fp32) ((float*)rp.scale)[(long)rlog[t] * rp.scale_stride + g] = stored;
+        else ((__half*)rp.scale)[(long)rlog[t] * rp.scale_stride + g] = __float2half_rn(stored);
       }
     } else {   // FP4: four MX blocks of 32 per group
       uint32_t sbytes = 0;
@@ -163,7 +179,7 @@ void dmq_rotate_kernel(RotParams p) {
         }
       }
       if (valid[t] && q == 0)
-        *(uint32_t*)((uint8_t*)p.scale + (long)rlog[t] * p.scale_stride + g * 4) = sbytes;
+        *(uint32_t*)((uint8_t*)rp.scale + (long)rlog[t] * rp.scale_stride + g * 4) = sbytes;
     }
   }
 }
@@ -171,7 +187,6 @@ void dmq_rotate_kernel(RotParams p) {
 // --------------------------------------------------------------------------------------------
 // Quantization of activations that are already rotated (no matrix product): one wave per
 // (row, group), two consecutive features per lane.
-
 template <int MODE>
 __global__ __launch_bounds__(256)
 void dmq_quantize_kernel(QuantParams p) {

@@ -14,6 +14,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
+ABI_VERSION = 2
+MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER = 0, 1, 2
 MODE_BY_NAME = {"wxa16": MODE_A16, "wxa8": MODE_A8, "wxfp8": MODE_FP8, "wxfp4": MODE_FP4}
@@ -24,19 +26,23 @@ _EXC = {1: ValueError, 2: ValueError, 3: ValueError, 4: ValueError, 5: ValueErro
         6: TypeError, 7: RuntimeError, 8: ValueError}
 
 
+class GemmPool(Structure):
+    _fields_ = [
+        ("w", c_void_p), ("norms", c_void_p), ("lut", c_void_p), ("expert_info", c_void_p),
+        ("act", c_void_p), ("act_scale", c_void_p), ("row_index", c_void_p),
+        ("n_total", c_int), ("bit", c_int), ("mode", c_int), ("w_scale_byte", c_int),
+    ]
+
+
 class GemmArgs(Structure):
     _fields_ = [
-        ("mode", c_int), ("bit", c_int), ("epi", c_int), ("tt", c_int),
-        ("act", c_void_p), ("act_row_bytes", c_long),
-        ("act_scale", c_void_p), ("act_scale_stride", c_int),
-        ("row_index", c_void_p),
-        ("w", c_void_p), ("norms", c_void_p), ("lut", c_void_p),
-        ("n_total", c_int), ("groups", c_int), ("n_out", c_int), ("half_width", c_int),
-        ("slice_is_groups", c_int), ("w_scale_byte", c_int),
-        ("expert_info", c_void_p), ("n_experts", c_int),
-        ("tiles", c_void_p), ("n_tiles", c_void_p), ("max_tiles", c_int),
+        ("mode", c_int), ("epi", c_int), ("tt", c_int), ("ks", c_int), ("n_pools", c_int),
+        ("pool", GemmPool * MAX_POOLS),
+        ("act_row_bytes", c_long), ("act_scale_stride", c_int),
+        ("groups", c_int), ("n_out", c_int), ("half_width", c_int), ("slice_is_groups", c_int),
+        ("items", c_void_p), ("n_items", c_void_p), ("max_items", c_int),
         ("out", c_void_p), ("out_stride", c_long),
-        ("row_weight", c_void_p), ("row_token", c_void_p), ("dbg_acc", c_void_p),
+        ("row_weight", c_void_p), ("row_slot", c_void_p), ("dbg_acc", c_void_p),
     ]
 
 
@@ -72,7 +78,7 @@ PROTOTYPES = {
                                c_void_p]),
     "dmq_route_permute": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                   c_int, c_int] + [c_void_p] * 10),
-    "dmq_build_tiles": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "dmq_build_tiles": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "dmq_rotate": (c_int, [c_int, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p,
                            c_long, c_void_p, c_int, c_int, c_float, c_int, c_void_p]),
     "dmq_rotate_tiled": (c_int, [c_int, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p,
@@ -81,11 +87,15 @@ PROTOTYPES = {
     "dmq_quantize_act": (c_int, [c_int, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_long,
                                  c_void_p, c_int, c_int, c_float, c_void_p]),
     "dmq_matmul_merged_gf": (c_int, [POINTER(GemmArgs), c_void_p]),
+    "dmq_combine_slots": (c_int, [c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p]),
     "dmq_finalize_f16": (c_int, [c_void_p, c_void_p, c_long, c_void_p, c_void_p]),
     "dmq_fill_zero": (c_int, [c_void_p, c_long, c_void_p]),
     "dmq_moe_workspace_bytes": (c_size_t, [POINTER(LayerDesc), c_int]),
     "dmq_moe_ffn_forward": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                    c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+                                    c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p]),
+    "dmq_moe_ffn_forward_staged": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int,
+                                           c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int,
+                                           POINTER(c_void_p), POINTER(c_long), c_void_p]),
 }
 
 _lib = None
@@ -104,6 +114,8 @@ def load() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
+        if lib.dmq_abi_version() != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} has ABI {lib.dmq_abi_version()}, expected {ABI_VERSION}: rebuild")
         _lib = lib
     return _lib
 

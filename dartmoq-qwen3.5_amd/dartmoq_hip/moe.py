@@ -23,6 +23,11 @@ from ._lib import (MODE_A16, MODE_A8, MODE_BY_NAME, MODE_FP4, MODE_FP8, LayerDes
 GROUP_SIZE = 128
 
 
+def _lib_max_pools() -> int:
+    from ._lib import MAX_POOLS
+    return MAX_POOLS
+
+
 class BitPoolWeights:
     """Runtime form of one bit pool (the reference's WxA16Weights, :32-265, after
     _build_group_first :177-233 and the subclasses' _get_bit_context)."""
@@ -114,7 +119,8 @@ class WxA16BitPartitionedGroupMoE:
         self.bit_list: list[int] = []
         self._desc = None
         self._workspace = None
-        self.tt_override = 0
+        self.tt_override = 0        # activation tiles of 16 rows per wave (0 = pick from tokens)
+        self.ks_override = 0        # waves splitting K inside a workgroup (0 = pick from tt)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -137,6 +143,13 @@ class WxA16BitPartitionedGroupMoE:
             moe.bit_weights[bit_str] = BitPoolWeights(bit, p["gate_up"], p["down"], offs, moe.device)
             moe.expert_offsets[bit_str] = offs
             moe.bit_list.append(bit)
+        if len(moe.bit_weights) > _lib_max_pools():
+            raise ValueError(f"at most {_lib_max_pools()} bit pools per layer")
+        for ex in range(num_experts):
+            homes = sum(1 for o in moe.expert_offsets.values() if o[ex + 1] > o[ex])
+            if homes != 1:
+                raise ValueError(f"expert {ex} belongs to {homes} bit pools; this build handles "
+                                 "layers whose experts live in exactly one pool")
         return moe
 
     @classmethod
@@ -240,7 +253,7 @@ class WxA16BitPartitionedGroupMoE:
         check(load().dmq_moe_ffn_forward(
             ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens,
             None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-            int(self.tt_override), stream), "moe_ffn_forward")
+            int(self.tt_override), int(self.ks_override), stream), "moe_ffn_forward")
         if orig_dtype != torch.float16:
             out = out.to(orig_dtype)
         return out.reshape(shape)
@@ -326,62 +339,43 @@ class HipStageProfiler:
         return stats
 
 
+STAGE_NAMES = ("sort_prep", "rotation", "merged_gate_up", "act_quant_down", "merged_down", "combine")
+
+
 @torch.no_grad()
 def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: torch.Tensor,
-                   topk_w: torch.Tensor, tt: int | None = None, profiler: HipStageProfiler | None = None):
-    """The same launches as dmq_moe_ffn_forward, issued stage by stage from Python so that each
-    one can be timed with events on the stream it runs on.  Returns (out fp16 [T, H], stats,
-    aux) where aux carries the routing plan (counts per expert) for byte accounting.  Stage
-    names follow the reference: sort_prep, rotation_hoisted, merged_gate_up, act_quant_down,
-    merged_down, scatter (fused into merged_down here), finalize."""
-    from ._lib import EPI_SCATTER, EPI_SILU
-    prof = profiler or HipStageProfiler(enabled=False)
+                   topk_w: torch.Tensor, tt: int = 0, ks: int = 0, profile: bool = True):
+    """dmq_moe_ffn_forward_staged: the production forward with an event recorded on the launch
+    stream after every stage.  Returns (out fp16 [T, H], {stage: ms}, aux) where aux carries the
+    per-expert routed-row counts (for byte accounting) and the tiling that was used.  Stage names
+    follow the reference's profiler: sort_prep, rotation (rotation_hoisted / act_quant),
+    merged_gate_up (with silu_mul fused), act_quant_down, merged_down (routing weight and scatter
+    fused), combine (the add of the scattered rows)."""
     x = x.half().contiguous()
-    tokens, hidden = x.shape
-    inter, e, k = moe.intermediate_size, moe.num_experts, moe.top_k
-    rows = tokens * k
-    if tt is None or tt <= 0:
-        tt = ops.pick_tt(rows, e)
-    rot_tt = 4 if tt == 4 else 1
-    desc, pool_arr, slice_start, slice_count, _keep = moe._descriptor()
-    prof.begin_round()
-    with prof.stage("sort_prep"):
-        plan = ops.route_permute(topk_idx.int().contiguous(), topk_w.float().contiguous(), e,
-                                 slice_start, slice_count, 16 * tt)
-    out32 = torch.zeros((tokens, hidden), dtype=torch.float32, device=x.device)
-    for pi, (bit_str, bw) in enumerate(moe.bit_weights.items()):
-        mode = moe.pool_mode(bw.bit)
-        ctx = bw.context(mode)
-        major = bool(pool_arr[pi].major)
-        gu_info, dn_info = plan["gu_info"][pi], plan["dn_info"][pi]
-        tiling = (plan["n_tiles"][pi], plan["tiles"][pi], plan["max_tiles"])
-        with prof.stage(f"rotation_hoisted.{bit_str}"):
-            if major:
-                xq, xs = ops.rotate(mode, x, bw.gu_rot, ctx["gu_extra"], tt=rot_tt)
-                row_index = plan["sorted_tokens"]
-            else:
-                xq, xs = ops.rotate_tiled(mode, x, bw.gu_rot, gu_info, tiling[0], tiling[1], 16 * tt,
-                                          tiling[2], rows, rot_per_expert=False,
-                                          extra_scale=ctx["gu_extra"],
-                                          row_index=plan["sorted_tokens"], tt=rot_tt)
-                row_index = None
-        with prof.stage(f"merged_gate_up.{bit_str}"):
-            act = ops.matmul_merged(mode, bw.bit, EPI_SILU, xq, xs, ctx["gu_w"], ctx["gu_norms"],
-                                    ctx["gu_lut"], gu_info, groups=hidden // GROUP_SIZE, n_out=inter,
-                                    half_width=inter, slice_is_groups=False, rows_total=rows,
-                                    row_index=row_index, w_scale_byte=ctx["gu_wsb"], tt=tt,
-                                    tiling=tiling)
-        with prof.stage(f"act_quant_down.{bit_str}"):
-            aq, as_ = ops.rotate_tiled(mode, act, bw.dn_rot, dn_info, tiling[0], tiling[1], 16 * tt,
-                                       tiling[2], rows, rot_per_expert=True,
-                                       extra_scale=ctx["dn_extra"], tt=rot_tt)
-        with prof.stage(f"merged_down.{bit_str}"):
-            ops.matmul_merged(mode, bw.bit, EPI_SCATTER, aq, as_, ctx["dn_w"], ctx["dn_norms"],
-                              ctx["dn_lut"], dn_info, groups=inter // GROUP_SIZE, n_out=hidden,
-                              slice_is_groups=True, rows_total=rows, out=out32, out_stride=hidden,
-                              w_scale_byte=ctx["dn_wsb"], row_weight=plan["sorted_weights"],
-                              row_token=plan["sorted_tokens"], tt=tt, tiling=tiling)
-    with prof.stage("finalize"):
-        out = ops.finalize_f16(out32)
-    stats = prof.end_round()
-    return out, stats, {"counts": plan["counts"], "tt": tt}
+    tokens = x.shape[0]
+    topk_idx = topk_idx.to(torch.int32).contiguous()
+    topk_w = topk_w.float().contiguous()
+    desc = moe._descriptor()[0]
+    ws = moe._get_workspace(tokens)
+    out = torch.empty_like(x)
+    stream = torch.cuda.current_stream(x.device)
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(len(STAGE_NAMES) + 1)]
+    handles = (ctypes.c_void_p * len(events))()
+    if profile:
+        for i, ev in enumerate(events):
+            ev.record(stream)                       # materialise the HIP event behind the object
+            handles[i] = ev.cuda_event
+    aux = (ctypes.c_long * 8)()
+    check(load().dmq_moe_ffn_forward_staged(
+        ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens, None,
+        out.data_ptr(), ws.data_ptr(), ws.numel(), int(tt or moe.tt_override),
+        int(ks or moe.ks_override), handles if profile else None, aux,
+        ctypes.c_void_p(stream.cuda_stream)), "moe_ffn_forward_staged")
+    torch.cuda.synchronize(x.device)
+    stats = {}
+    if profile:
+        for i, name in enumerate(STAGE_NAMES):
+            stats[name] = events[i].elapsed_time(events[i + 1])
+    counts = ws[aux[2]:aux[2] + 4 * moe.num_experts].view(torch.int32).clone()
+    n_items = int(ws[aux[4]:aux[4] + 4].view(torch.int32).item())
+    return out, stats, {"counts": counts, "tt": int(aux[0]), "ks": int(aux[1]), "n_items": n_items}

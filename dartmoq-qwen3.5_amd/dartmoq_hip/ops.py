@@ -120,39 +120,39 @@ def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_
     dev = topk_idx.device
     pools = slice_start.shape[0]
     rows = t * k
-    max_tiles = rows // tile_rows + num_experts
+    max_items = rows // tile_rows + num_experts
     i32 = dict(dtype=torch.int32, device=dev)
     res = {
         "counts": torch.empty(num_experts, **i32),
         "offsets": torch.empty(num_experts + 1, **i32),
         "sorted_tokens": torch.empty(rows, **i32),
         "sorted_weights": torch.empty(rows, dtype=torch.float32, device=dev),
-        "sorted_slots": torch.empty(rows, **i32),
+        "sorted_rows": torch.empty(rows, **i32),
         "gu_info": torch.empty((pools, num_experts, 4), **i32),
         "dn_info": torch.empty((pools, num_experts, 4), **i32),
-        "n_tiles": torch.zeros((pools, 4), **i32),
-        "tiles": torch.zeros((pools, max_tiles, 2), **i32),
-        "max_tiles": max_tiles, "tile_rows": tile_rows,
+        "n_items": torch.zeros(4, **i32),
+        "items": torch.zeros((max_items, 4), **i32),
+        "max_items": max_items, "tile_rows": tile_rows,
     }
     check(load().dmq_route_permute(
         _ptr(topk_idx.to(torch.int32).contiguous()), _ptr(topk_w.float().contiguous()), t, k,
         num_experts, pools, _ptr(slice_start.contiguous()), _ptr(slice_count.contiguous()), tile_rows,
-        max_tiles, _ptr(res["counts"]), _ptr(res["offsets"]), _ptr(res["sorted_tokens"]),
-        _ptr(res["sorted_weights"]), _ptr(res["sorted_slots"]), _ptr(res["gu_info"]),
-        _ptr(res["dn_info"]), _ptr(res["n_tiles"]), _ptr(res["tiles"]), _stream(dev)), "route_permute")
+        max_items, _ptr(res["counts"]), _ptr(res["offsets"]), _ptr(res["sorted_tokens"]),
+        _ptr(res["sorted_weights"]), _ptr(res["sorted_rows"]), _ptr(res["gu_info"]),
+        _ptr(res["dn_info"]), _ptr(res["n_items"]), _ptr(res["items"]), _stream(dev)), "route_permute")
     return res
 
 
-def build_tiles(expert_info: torch.Tensor, rows_total: int, tile_rows: int):
-    """(n_tiles int32[1], tiles int32[max_tiles, 2], max_tiles) for a device expert_info [E, 4]."""
+def build_tiles(expert_info: torch.Tensor, rows_total: int, tile_rows: int, pool: int = 0):
+    """(n_items int32[1], items int32[max_items, 4], max_items) for a device expert_info [E, 4]."""
     _need_cuda(expert_info)
     n_exp = expert_info.shape[0]
-    max_tiles = rows_total // tile_rows + n_exp
-    n_tiles = torch.zeros(4, dtype=torch.int32, device=expert_info.device)
-    tiles = torch.zeros((max_tiles, 2), dtype=torch.int32, device=expert_info.device)
-    check(load().dmq_build_tiles(_ptr(expert_info), n_exp, tile_rows, max_tiles, _ptr(n_tiles),
-                                 _ptr(tiles), _stream(expert_info.device)), "build_tiles")
-    return n_tiles, tiles, max_tiles
+    max_items = rows_total // tile_rows + n_exp
+    n_items = torch.zeros(4, dtype=torch.int32, device=expert_info.device)
+    items = torch.zeros((max_items, 4), dtype=torch.int32, device=expert_info.device)
+    check(load().dmq_build_tiles(_ptr(expert_info), n_exp, tile_rows, max_items, pool, _ptr(n_items),
+                                 _ptr(items), _stream(expert_info.device)), "build_tiles")
+    return n_items, items, max_items
 
 
 # ----------------------------------------------------------------------------- activations
@@ -173,15 +173,14 @@ def _alloc_codes(mode, rows, k, device, scale_fp32):
 
 
 def rotate(mode: int, x: torch.Tensor, rot: torch.Tensor, extra_scale: float = 1.0,
-           scale_fp32: bool = False, row_index: torch.Tensor | None = None, tt: int | None = None):
+           scale_fp32: bool = False, tt: int | None = None):
     """Rotate (and quantize for mode != A16) x[B, K] with rot[G, 128, 128]."""
     _need_cuda(x, rot)
     if x.dtype != torch.float16:
         x = x.half()
     x = x.contiguous()
     rot = rot.contiguous()
-    k = x.shape[1]
-    rows = x.shape[0] if row_index is None else row_index.numel()
+    rows, k = x.shape
     groups = k // GROUP_SIZE
     if k != groups * GROUP_SIZE:
         raise ValueError(f"K ({k}) must be a multiple of {GROUP_SIZE}")
@@ -190,23 +189,24 @@ def rotate(mode: int, x: torch.Tensor, rot: torch.Tensor, extra_scale: float = 1
     codes, scale, sstride = _alloc_codes(mode, rows, k, x.device, scale_fp32)
     if tt is None:
         tt = 4 if rows >= 1024 else 1
-    check(load().dmq_rotate(mode, _ptr(x), x.stride(0), _ptr(row_index), _ptr(rot), rows, groups,
+    check(load().dmq_rotate(mode, _ptr(x), x.stride(0), None, _ptr(rot), rows, groups,
                             _ptr(codes), codes.stride(0) * codes.element_size(), _ptr(scale), sstride,
                             int(scale_fp32), float(extra_scale), tt, _stream(x.device)), "rotate")
     return codes, scale
 
 
-def rotate_tiled(mode, x, rot, expert_info, n_tiles, tiles, tile_rows, max_tiles, rows_out,
+def rotate_tiled(mode, x, rot, expert_info, n_items, items, tile_rows, max_items, rows_out,
                  rot_per_expert=True, extra_scale=1.0, row_index=None, tt=1):
-    """Per-expert rotation: rows of expert e use rot[slice_start_e + g]."""
+    """Rotation of rows grouped by expert: rows of expert e use rot[slice_start_e + g] when
+    ``rot_per_expert`` (else rot[g]); ``row_index`` gathers the input rows."""
     _need_cuda(x, rot, expert_info)
     x = x.contiguous()
     k = x.shape[1]
     groups = k // GROUP_SIZE
     codes, scale, sstride = _alloc_codes(mode, rows_out, k, x.device, False)
     check(load().dmq_rotate_tiled(mode, _ptr(x), x.stride(0), _ptr(row_index), _ptr(rot.contiguous()),
-                                  int(rot_per_expert), groups, _ptr(expert_info), _ptr(tiles),
-                                  _ptr(n_tiles), tile_rows, max_tiles, _ptr(codes),
+                                  int(rot_per_expert), groups, _ptr(expert_info), _ptr(items),
+                                  _ptr(n_items), tile_rows, max_items, _ptr(codes),
                                   codes.stride(0) * codes.element_size(), _ptr(scale), sstride, 0,
                                   float(extra_scale), tt, _stream(x.device)), "rotate_tiled")
     return codes, scale
@@ -237,43 +237,85 @@ def pick_tt(rows_total: int, n_experts: int) -> int:
     return 1 if avg <= 8 else (2 if avg <= 48 else 4)
 
 
+def pick_ks(tt: int) -> int:
+    return {1: 4, 2: 2, 4: 1}[tt]
+
+
+def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=None, w_scale_byte=127):
+    """One pool entry of a merged launch (a dict of device tensors and scalars)."""
+    return dict(mode=mode, bit=bit, act=act, act_scale=act_scale, w=w, norms=norms, lut=lut,
+                expert_info=expert_info, row_index=row_index, w_scale_byte=w_scale_byte)
+
+
+def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
+                 tt, ks=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
+                 row_weight=None, row_slot=None, dbg_acc=None):
+    """Merged dequant-GEMM launch over up to four pools sharing one work-item list."""
+    a = GemmArgs()
+    a.mode, a.epi, a.tt, a.ks, a.n_pools = mode, epi, tt, ks, len(pools)
+    dev = None
+    for i, p in enumerate(pools):
+        _need_cuda(p["act"], p["w"], p["norms"], p["expert_info"])
+        dev = p["act"].device
+        _check_bit(p["bit"])
+        q = a.pool[i]
+        q.w, q.norms = p["w"].data_ptr(), p["norms"].data_ptr()
+        q.lut = p["lut"].data_ptr() if p["lut"] is not None else None
+        q.expert_info = p["expert_info"].data_ptr()
+        q.act = p["act"].data_ptr()
+        q.act_scale = p["act_scale"].data_ptr() if p["act_scale"] is not None else None
+        q.row_index = p["row_index"].data_ptr() if p["row_index"] is not None else None
+        q.n_total, q.bit, q.mode, q.w_scale_byte = p["w"].shape[1], p["bit"], p["mode"], int(p["w_scale_byte"])
+    first = next(p for p in pools if p["mode"] == mode)
+    if act_row_bytes is None:
+        act_row_bytes = first["act"].stride(0) * first["act"].element_size()
+    if act_scale_stride is None:
+        act_scale_stride = first["act_scale"].stride(0) if first["act_scale"] is not None else 0
+    a.act_row_bytes, a.act_scale_stride = act_row_bytes, act_scale_stride
+    a.groups, a.n_out, a.half_width, a.slice_is_groups = groups, n_out, half_width, int(slice_is_groups)
+    a.items, a.n_items, a.max_items = items.data_ptr(), n_items.data_ptr(), max_items
+    a.out, a.out_stride = out.data_ptr(), out_stride
+    a.row_weight = row_weight.data_ptr() if row_weight is not None else None
+    a.row_slot = row_slot.data_ptr() if row_slot is not None else None
+    a.dbg_acc = dbg_acc.data_ptr() if dbg_acc is not None else None
+    check(load().dmq_matmul_merged_gf(ctypes.byref(a), _stream(dev)), "matmul_merged_gf")
+    return out
+
+
 def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *, groups, n_out,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
-                  row_index=None, w_scale_byte=127, row_weight=None, row_token=None, tt=None,
+                  row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0,
                   tiling=None, dbg_acc=None):
-    """One merged dequant-GEMM launch.  ``expert_info`` is an int32 device tensor [E, 4]."""
+    """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
-    dev = act.device
+    _check_bit(bit)
     n_exp = expert_info.shape[0]
     if tt is None:
         tt = pick_tt(rows_total, n_exp)
     if tiling is None:
         tiling = build_tiles(expert_info, rows_total, 16 * tt)
-    n_tiles, tiles, max_tiles = tiling
+    n_items, items, max_items = tiling
     if out is None:
         if epi == EPI_SCATTER:
-            raise ValueError("scatter epilogue needs a caller-provided fp32 accumulator")
-        out = torch.empty((rows_total, n_out), dtype=torch.float16, device=dev)
+            raise ValueError("scatter epilogue needs a caller-provided fp32 slot buffer")
+        out = torch.empty((rows_total, n_out), dtype=torch.float16, device=act.device)
         out_stride = n_out
-    a = GemmArgs()
-    a.mode, a.bit, a.epi, a.tt = mode, bit, epi, tt
-    a.act = act.data_ptr()
-    a.act_row_bytes = act.stride(0) * act.element_size()
-    a.act_scale = act_scale.data_ptr() if act_scale is not None else None
-    a.act_scale_stride = act_scale.stride(0) if act_scale is not None else 0
-    a.row_index = row_index.data_ptr() if row_index is not None else None
-    a.w, a.norms = w.data_ptr(), norms.data_ptr()
-    a.lut = lut.data_ptr() if lut is not None else None
-    a.n_total = w.shape[1]
-    a.groups, a.n_out, a.half_width = groups, n_out, half_width
-    a.slice_is_groups, a.w_scale_byte = int(slice_is_groups), int(w_scale_byte)
-    a.expert_info, a.n_experts = expert_info.data_ptr(), n_exp
-    a.tiles, a.n_tiles, a.max_tiles = tiles.data_ptr(), n_tiles.data_ptr(), max_tiles
-    a.out, a.out_stride = out.data_ptr(), out_stride if out_stride is not None else out.stride(0)
-    a.row_weight = row_weight.data_ptr() if row_weight is not None else None
-    a.row_token = row_token.data_ptr() if row_token is not None else None
-    a.dbg_acc = dbg_acc.data_ptr() if dbg_acc is not None else None
-    check(load().dmq_matmul_merged_gf(ctypes.byref(a), _stream(dev)), "matmul_merged_gf")
+    pool = gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index, w_scale_byte)
+    return matmul_pools(mode, epi, [pool], items, n_items, max_items, groups=groups, n_out=n_out,
+                        slice_is_groups=slice_is_groups, tt=tt, ks=ks, out=out,
+                        out_stride=out_stride if out_stride is not None else out.stride(0),
+                        half_width=half_width, row_weight=row_weight, row_slot=row_slot,
+                        dbg_acc=dbg_acc)
+
+
+def combine_slots(slots: torch.Tensor, top_k: int, add: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = fp16(sum_j slots[t*k + j] (+ add[t])), slots fp32 [T*k, H]."""
+    _need_cuda(slots)
+    rows, hidden = slots.shape
+    tokens = rows // top_k
+    out = torch.empty((tokens, hidden), dtype=torch.float16, device=slots.device)
+    check(load().dmq_combine_slots(_ptr(slots), top_k, _ptr(add), tokens, hidden, _ptr(out),
+                                   _stream(slots.device)), "combine_slots")
     return out
 
 

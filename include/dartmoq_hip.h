@@ -20,6 +20,8 @@
  *   mode                  DMQ_MODE_A16 / A8 / FP8 / FP4
  *   expert_info           int32 [n_experts, 4] = token_start, token_count,
  *                         slice_start, slice_count   (device memory)
+ *   work items            int32 [n, 4] = pool, expert index, row tile inside the expert, 0;
+ *                         a row tile covers tile_rows = 16*tt activation rows
  */
 #ifndef DARTMOQ_HIP_H
 #define DARTMOQ_HIP_H
@@ -36,9 +38,13 @@ enum {
   DMQ_ERR_MODE = 5, DMQ_ERR_NULL = 6, DMQ_ERR_HIP = 7, DMQ_ERR_LIMIT = 8
 };
 enum { DMQ_MODE_A16 = 0, DMQ_MODE_A8 = 1, DMQ_MODE_FP8 = 2, DMQ_MODE_FP4 = 3 };
+/* STORE: fp16 [rows, n_out].  SILU: fp16 silu(gate)*up [rows, I].  SCATTER: fp32 routing-weighted
+ * rows stored at out[row_slot[r]] (one slot per (token, top-k slot)); dmq_combine_slots adds
+ * the k slots of each token in slot order. */
 enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
+#define DMQ_MAX_POOLS 4
 
-/* Library / build identification: returns the ABI version (currently 1). */
+/* Library / build identification: returns the ABI version (currently 2). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -88,17 +94,19 @@ int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts,
  *   slice_count [pools, experts] int32: 2*I
  * Outputs (device, int32 unless noted):
  *   counts [experts], offsets [experts+1], sorted_tokens [tokens*k],
- *   sorted_weights fp32 [tokens*k], sorted_slots [tokens*k] (may be NULL),
- *   gu_info / dn_info [pools, experts, 4], n_tiles [pools, 4], tiles [pools, max_tiles, 2]. */
+ *   sorted_weights fp32 [tokens*k], sorted_rows [tokens*k] (token*k + slot of each sorted row),
+ *   gu_info / dn_info [pools, experts, 4], n_items [1], items [max_items, 4] (all pools,
+ *   pool-major, experts ascending). */
 int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
                       int pools, const void* slice_start, const void* slice_count, int tile_rows,
-                      int max_tiles, void* counts, void* offsets, void* sorted_tokens,
-                      void* sorted_weights, void* sorted_slots, void* gu_info, void* dn_info,
-                      void* n_tiles, void* tiles, void* stream);
+                      int max_items, void* counts, void* offsets, void* sorted_tokens,
+                      void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
+                      void* n_items, void* items, void* stream);
 
-/* Tile list for a caller-built expert_info: n_tiles int32[1], tiles int32 [max_tiles, 2]. */
-int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_tiles,
-                    void* n_tiles, void* tiles, void* stream);
+/* Work items for a caller-built expert_info: n_items int32[1], items int32 [max_items, 4]
+ * with the given pool id. */
+int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_items,
+                    int pool, void* n_items, void* items, void* stream);
 
 /* ------------------------------------------------------------------ activations */
 
@@ -114,14 +122,14 @@ int dmq_rotate(int mode, const void* x, long x_stride, const void* row_index, co
                int rows, int groups, void* out, long out_row_bytes, void* scale,
                int scale_stride, int scale_fp32, float extra_scale, int tt, void* stream);
 
-/* Same, for rows grouped by expert: tile entry (e, i) covers rows token_start + i*tile_rows ..
- * With rot_per_expert != 0 group g of expert e uses rot[slice_start_e + g] (the per-expert
- * down rotations, seed + original_start of triton_kernels.py:1310), otherwise rot[g].
- * max_tiles bounds the tile list. */
+/* Same, for rows grouped by expert: work item (pool, e, i) covers rows
+ * token_start_e + i*tile_rows .. of expert_info.  With rot_per_expert != 0 group g of expert e
+ * uses rot[slice_start_e + g] (the per-expert down rotations, seed + original_start of
+ * triton_kernels.py:1310), otherwise rot[g].  max_items bounds the item list. */
 int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_index,
-                     const void* rot, int rot_per_expert, int groups, const void* expert_info, const void* tiles,
-                     const void* n_tiles, int tile_rows, int max_tiles, void* out,
-                     long out_row_bytes, void* scale, int scale_stride, int scale_fp32,
+                     const void* rot, int rot_per_expert, int groups, const void* expert_info,
+                     const void* items, const void* n_items, int tile_rows, int max_items,
+                     void* out, long out_row_bytes, void* scale, int scale_stride, int scale_fp32,
                      float extra_scale, int tt, void* stream);
 
 /* quantize_act_per_token_group (triton_kernels_a8.py:384-421), ..._fp8
@@ -134,48 +142,59 @@ int dmq_quantize_act(int mode, const void* x, int x_fp32, long x_stride, int row
 /* ------------------------------------------------------------------ dequant GEMMs */
 
 typedef struct {
-  int mode;                 /* DMQ_MODE_* */
-  int bit;                  /* index width of idx_gf (FP4 reads folded e2m1: pass the pool bit) */
-  int epi;                  /* DMQ_EPI_* */
-  int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4 */
-  const void* act;          /* activation codes, row-major */
-  long act_row_bytes;
-  const void* act_scale;    /* fp16 [rows, act_scale_stride] (A8/FP8), u8 (FP4), NULL (A16) */
-  int act_scale_stride;
-  const void* row_index;    /* optional gather of activation rows (int32) */
   const void* w;            /* idx_gf, or folded e2m1 [G, N, 64] for FP4 */
   const void* norms;        /* norms_gf */
   const void* lut;          /* fp16 / int8 / e4m3 codebook; unused for FP4 */
-  int n_total;              /* N of the shared weight */
+  const void* expert_info;
+  const void* act;          /* activation codes of this pool, row-major */
+  const void* act_scale;    /* fp16 [rows, act_scale_stride] (A8/FP8), u8 (FP4), NULL (A16) */
+  const void* row_index;    /* optional gather of activation rows (int32) */
+  int n_total;              /* N of the pool's weight */
+  int bit;                  /* index width of idx_gf (FP4 reads folded e2m1: pass the pool bit) */
+  int mode;                 /* must equal the launch mode; other pools are skipped */
+  int w_scale_byte;         /* FP4: 127 + E0 */
+} dmq_gemm_pool;
+
+typedef struct {
+  int mode;                 /* DMQ_MODE_* */
+  int epi;                  /* DMQ_EPI_* */
+  int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4 */
+  int ks;                   /* waves of a workgroup splitting K: 0 = pick, else 1, 2 or 4 */
+  int n_pools;
+  dmq_gemm_pool pool[DMQ_MAX_POOLS];
+  long act_row_bytes;
+  int act_scale_stride;
   int groups;               /* groups contracted per expert */
   int n_out;                /* output features per row (SILU: I) */
   int half_width;           /* SILU: I */
   int slice_is_groups;      /* 0 gate_up (slice offsets rows), 1 down (slice offsets groups) */
-  int w_scale_byte;         /* FP4: 127 + E0 */
-  const void* expert_info;
-  int n_experts;
-  const void* tiles;        /* from dmq_build_tiles / dmq_route_permute, tile_rows == 16*tt */
-  const void* n_tiles;
-  int max_tiles;
-  void* out;                /* STORE/SILU: fp16 [rows, out_stride]; SCATTER: fp32 [tokens, out_stride] */
+  const void* items;        /* from dmq_build_tiles / dmq_route_permute, tile_rows == 16*tt */
+  const void* n_items;
+  int max_items;
+  void* out;                /* STORE/SILU: fp16 [rows, out_stride]; SCATTER: fp32 [slots, out_stride] */
   long out_stride;
   const void* row_weight;   /* SCATTER: fp32 routing weight per row */
-  const void* row_token;    /* SCATTER: int32 destination token per row */
-  void* dbg_acc;            /* A8, tt == 1, STORE only: int32 [rows, groups, n_out] or NULL */
+  const void* row_slot;     /* SCATTER: int32 destination slot row per row */
+  void* dbg_acc;            /* A8, tt == 1, ks == 1, STORE only: int32 [rows, groups, n_out] or NULL */
 } dmq_gemm_args;
 
-/* Merged (one launch per bit pool) dequant GEMM.  Stands in for
+/* Merged dequant GEMM: one launch for all bit pools of a layer that share `mode`.  Stands in for
  *   triton_fused_matmul_merged_rows_gf / _merged_in_features_gf   (triton_kernels.py:1482-1615)
  *   wxa8_matmul_merged_rows_gf / _merged_in_features_gf           (triton_kernels_a8.py:959-1068)
  *   wxfp8_matmul_merged_rows_gf / _merged_in_features_gf          (triton_kernels_fp8.py:641-750)
  *   wxfp4_matmul_merged_rows_gf / _merged_in_features_gf          (triton_kernels_fp4.py:740-874)
  * and, with a one-row expert_info, for the per-expert *_grouped_slice_rows_gf /
  * *_grouped_slice_in_features_gf / *_grouped_gf wrappers.  DMQ_EPI_SILU fuses
- * F.silu(gate) * up (bit_partitioned_moe.py:925-930), DMQ_EPI_SCATTER fuses the routing
- * weight and index_add_ (:965-967) into fp32 atomics. */
+ * F.silu(gate) * up (bit_partitioned_moe.py:925-930); DMQ_EPI_SCATTER fuses the routing
+ * weight and the scatter of :965-967 (the add is dmq_combine_slots). */
 int dmq_matmul_merged_gf(const dmq_gemm_args* args, void* stream);
 
-/* fp16(out32 (+ add16)) over n elements (n % 4 == 0): final store of the scatter target. */
+/* out[t, h] = fp16( sum_{j<k} slots[t*k + j, h] (+ add[t, h]) ): the index_add_ of
+ * bit_partitioned_moe.py:967 with a fixed summation order.  hidden % 4 == 0. */
+int dmq_combine_slots(const void* slots_f32, int k, const void* add_f16, long tokens, int hidden,
+                      void* out_f16, void* stream);
+
+/* fp16(out32 (+ add16)) over n elements (n % 4 == 0). */
 int dmq_finalize_f16(const void* acc_f32, const void* add_f16, long n, void* out_f16, void* stream);
 /* Zero-fill n bytes (n % 4 == 0) with a kernel (usable under graph capture). */
 int dmq_fill_zero(void* ptr, long n_bytes, void* stream);
@@ -195,7 +214,7 @@ typedef struct {
 } dmq_pool_desc;
 
 typedef struct {
-  int hidden, inter, experts, top_k, pools;
+  int hidden, inter, experts, top_k, pools;    /* pools <= DMQ_MAX_POOLS */
   const dmq_pool_desc* pool;      /* host array [pools] */
   const void* slice_start;        /* device int32 [pools, experts] (2*start or -1) */
   const void* slice_count;        /* device int32 [pools, experts] (2*I) */
@@ -208,10 +227,21 @@ size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens);
  * and its WxA8 / WxFP8 / WxFP4 subclasses, routed experts only:
  *   x fp16 [tokens, hidden]; topk_idx int32 / topk_w fp32 [tokens, top_k];
  *   out fp16 [tokens, hidden] = sum_k w * down_e(silu(gate_e(x)) * up_e(x)) (+ add_f16).
- * tt <= 0 picks the activation tile count from tokens. */
+ * Every expert must belong to exactly one pool.  tt <= 0 / ks <= 0 pick the tiling from tokens. */
 int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                         const void* topk_w, int tokens, const void* add_f16, void* out,
-                        void* workspace, size_t workspace_bytes, int tt, void* stream);
+                        void* workspace, size_t workspace_bytes, int tt, int ks, void* stream);
+
+/* Same forward with instrumentation, the role of the reference's CudaStageProfiler
+ * (turboquant_utils/cuda_profiler.py:51-174): stage_events (optional) is a host array of 7
+ * hipEvent_t recorded on `stream` before the first launch and after each stage (sort_prep,
+ * rotation, merged_gate_up, act_quant_down, merged_down, combine); aux_out (optional) is a host
+ * long[8] that receives tt, ks, the byte offset of counts[experts] inside the workspace,
+ * max_items and the byte offset of n_items. */
+int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
+                               const void* topk_w, int tokens, const void* add_f16, void* out,
+                               void* workspace, size_t workspace_bytes, int tt, int ks,
+                               void* const* stage_events, void* aux_out, void* stream);
 
 #ifdef __cplusplus
 }

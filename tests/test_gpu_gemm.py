@@ -133,7 +133,7 @@ def test_wxa8_int32_accumulators_exact(bit):
     dbg = torch.zeros(rows_total, k // 128, n_slice, dtype=torch.int32, device="cuda")
     ops.matmul_merged(A8, bit, STORE, codes.cuda(), s.half().cuda(), idx_gf.cuda(), norms_gf.cuda(),
                       q_lut.cuda(), torch.tensor(info, dtype=torch.int32).cuda(), groups=k // 128,
-                      n_out=n_slice, slice_is_groups=False, rows_total=rows_total, tt=1, dbg_acc=dbg)
+                      n_out=n_slice, slice_is_groups=False, rows_total=rows_total, tt=1, ks=1, dbg_acc=dbg)
     torch.cuda.synchronize()
     w = q_lut.long()[packing.unpack_nbit(idx_gf, bit, 128).long()]          # [G, N, 128]
     for e, (ts, cnt, ss, sc) in enumerate(info):
@@ -146,7 +146,7 @@ def test_silu_and_scatter_epilogues():
     """gate_up with fused SiLU*up and down with fused weight + scatter-add (WxA16, 2-bit)."""
     from dartmoq_hip import ops
     bit, k, inter, hidden = 2, 256, 128, 256
-    counts = [9, 40, 2]
+    counts = [9, 40, 2]                        # 51 rows = 17 tokens x 3 slots
     starts, rows_total = _expert_rows(counts)
     g = torch.Generator().manual_seed(5)
     idx_gf, norms_gf, cb = _pool(bit, 2 * inter * len(counts), k, 41)
@@ -161,22 +161,49 @@ def test_silu_and_scatter_epilogues():
     ref_act = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
     torch.testing.assert_close(act, ref_act, rtol=4e-3, atol=4e-3 * ref_act.abs().max().item())
 
-    # scatter: rows map to 12 tokens with weights; compare against STORE + index_add
+    # scatter: routing-weighted rows land in their (token, slot) rows, combine adds the slots
     didx, dnorms, dcb = _pool(bit, hidden, inter * len(counts), 43)
     a = (torch.randn(rows_total, inter, generator=g) * 0.5).half()
     dinfo = [(starts[e], counts[e], e * (inter // 128), inter // 128) for e in range(len(counts))]
     dinfo_dev = torch.tensor(dinfo, dtype=torch.int32).cuda()
-    tok = torch.randint(0, 12, (rows_total,), generator=g, dtype=torch.int32)
+    top_k = 3
+    slot = torch.randperm(rows_total, generator=g).int()          # rows_total == 17 tokens * 3
     wts = torch.rand(rows_total, generator=g)
     dcommon = dict(groups=inter // 128, n_out=hidden, slice_is_groups=True, rows_total=rows_total, tt=1)
     dn = ops.matmul_merged(A16, bit, STORE, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(),
                            dinfo_dev, **dcommon).float().cpu()
-    acc = torch.zeros(12, hidden, dtype=torch.float32, device="cuda")
+    slots = torch.full((rows_total, hidden), float("nan"), dtype=torch.float32, device="cuda")
     ops.matmul_merged(A16, bit, SCATTER, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(),
-                      dinfo_dev, out=acc, out_stride=hidden, row_weight=wts.cuda(),
-                      row_token=tok.cuda(), **dcommon)
-    ref = torch.zeros(12, hidden).index_add_(0, tok.long(), dn * wts.unsqueeze(1))
-    torch.testing.assert_close(acc.cpu(), ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+                      dinfo_dev, out=slots, out_stride=hidden, row_weight=wts.cuda(),
+                      row_slot=slot.cuda(), **dcommon)
+    out = ops.combine_slots(slots, top_k).float().cpu()
+    ref_slots = torch.zeros(rows_total, hidden)
+    ref_slots[slot.long()] = dn * wts.unsqueeze(1)
+    ref = ref_slots.reshape(rows_total // top_k, top_k, hidden).sum(1)
+    torch.testing.assert_close(out, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("tt,ks", [(1, 4), (1, 1), (2, 2), (2, 1), (4, 1), (4, 2)])
+def test_k_split_variants_agree(tt, ks):
+    """Every (row tile, K split) instantiation computes the same GEMM."""
+    from dartmoq_hip import ops
+    bit, k, n_slice = 2, 1024, 256
+    counts = [3, 70, 0, 21]
+    starts, rows_total = _expert_rows(counts)
+    idx_gf, norms_gf, cb = _pool(bit, n_slice * len(counts), k, 77)
+    g = torch.Generator().manual_seed(tt * 10 + ks)
+    x = (torch.randn(rows_total, k, generator=g) * 0.5).half()
+    info = [(starts[e], counts[e], e * n_slice, n_slice) for e in range(len(counts))]
+    out = ops.matmul_merged(A16, bit, STORE, x.cuda(), None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(),
+                            torch.tensor(info, dtype=torch.int32).cuda(), groups=k // 128,
+                            n_out=n_slice, slice_is_groups=False, rows_total=rows_total, tt=tt, ks=ks)
+    w = cb.float()[packing.unpack_nbit(idx_gf, bit, 128).long()]
+    ref = torch.zeros(rows_total, n_slice)
+    for e, (ts, cnt, ss, sc) in enumerate(info):
+        wl = w[:, ss:ss + sc].permute(1, 0, 2).reshape(n_slice, -1)
+        ref[ts:ts + cnt] = moe.lut_gemm(x[ts:ts + cnt].float(), torch.ones(cnt, k // 128), wl,
+                                        norms_gf[:, ss:ss + sc].float().t(), 128)
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
 
 
 def test_gemm_argument_errors():

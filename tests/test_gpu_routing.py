@@ -63,13 +63,13 @@ def test_permute_matches_oracle(tokens, tile_rows):
     assert torch.equal(res["offsets"].cpu().long(), offs)
     assert torch.equal(res["counts"].cpu().long(), offs[1:] - offs[:-1])
     assert torch.equal(res["sorted_tokens"].cpu().long(), toks)
-    assert torch.equal(res["sorted_slots"].cpu().long(), slots)
+    assert torch.equal(res["sorted_rows"].cpu().long(), toks * k + slots)
     assert torch.equal(res["sorted_weights"].cpu(), wts)
-    # pool partition: expert_info rows and tile lists
+    # pool partition: expert_info rows and the layer's work-item list (pool-major)
+    exp_items = []
     for pi, b in enumerate(bits):
         gu = res["gu_info"][pi].cpu()
         dn = res["dn_info"][pi].cpu()
-        exp_tiles = []
         for e in range(experts):
             member = expert_bit[e] == b
             cnt = int(offs[e + 1] - offs[e]) if member else 0
@@ -78,7 +78,7 @@ def test_permute_matches_oracle(tokens, tile_rows):
             if member:
                 assert gu[e, 2] == start[pi, e] and gu[e, 3] == 2 * inter
                 assert dn[e, 2] == start[pi, e] // 256 and dn[e, 3] == inter // 128
-            exp_tiles += [(e, i) for i in range(-(-cnt // tile_rows))]
-        n = int(res["n_tiles"][pi, 0])
-        assert n == len(exp_tiles)
-        assert [tuple(r) for r in res["tiles"][pi, :n].cpu().tolist()] == exp_tiles
+            exp_items += [(pi, e, i, 0) for i in range(-(-cnt // tile_rows))]
+    n = int(res["n_items"][0])
+    assert n == len(exp_items)
+    assert [tuple(r) for r in res["items"][:n].cpu().tolist()] == exp_items

@@ -27,11 +27,11 @@ def test_library_exports_every_declared_symbol():
     from dartmoq_hip import _lib
     lib = _lib.load()
     declared = _declared_symbols()
-    assert len(declared) >= 17
+    assert len(declared) >= 19
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/dartmoq_hip.h but not exported"
     assert set(declared) == set(_lib.PROTOTYPES), "ctypes prototypes and header disagree"
-    assert lib.dmq_abi_version() == 1
+    assert lib.dmq_abi_version() == 2
     assert lib.dmq_status_string(0) == b"ok"
     assert b"bit width" in lib.dmq_status_string(1)
 
@@ -46,15 +46,20 @@ def test_argument_validation_without_gpu():
     assert lib.dmq_dequant_tile(p, p, None, 16, 0, 1, 8, 16, 2, p, None) == 3          # n0+n_cnt > N
     assert lib.dmq_fold_indices_to_e2m1(p, p, 4, 8, p, None) == 1
     assert lib.dmq_route_topk(None, 0, 1, 8, 2, 0, p, p, None) == 6                   # null logits
-    assert lib.dmq_build_tiles(p, 4, 24, 8, p, p, None) == 2                          # tile not /16
+    assert lib.dmq_build_tiles(p, 4, 24, 8, 0, p, p, None) == 2                       # tile not /16
     assert lib.dmq_finalize_f16(p, None, 7, p, None) == 2
     assert lib.dmq_fill_zero(p, 6, None) == 2
     a = _lib.GemmArgs()
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 8                       # no pools
+    a.n_pools = 1
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 1                       # bit 0
-    a.bit, a.mode, a.tt = 2, 9, 1
+    a.pool[0].bit, a.mode, a.tt = 2, 9, 1
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # bad mode
-    a.mode = 0
+    a.mode, a.ks = 0, 3
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # bad K split
+    a.ks = 0
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 6                       # null pointers
+    assert lib.dmq_combine_slots(p, 8, None, 4, 6, p, None) == 2                      # hidden % 4
     with pytest.raises(ValueError):
         _lib.check(2, "demo")
     with pytest.raises(TypeError):
@@ -70,9 +75,11 @@ def test_workspace_size_formula():
     small = lib.dmq_moe_workspace_bytes(ctypes.byref(d), 64)
     big = lib.dmq_moe_workspace_bytes(ctypes.byref(d), 4096)
     r = 4096 * 8
-    # dominated by x codes [R, H] fp16 + act/actq [R, I] fp16 + fp32 output [T, H]
-    assert big >= r * 2048 * 2 + 2 * r * 512 * 2 + 4096 * 2048 * 4
-    assert big < 1.3 * (r * 2048 * 2 + 2 * r * 512 * 2 + 4096 * 2048 * 4) + (1 << 22)
+    # dominated by the fp32 slot rows [R, H], x codes by routed row [R, H] and by token
+    # [pools, T, H] (2 bytes per element) and act / act codes [R, I]
+    main = r * 2048 * 4 + r * 2048 * 2 + 3 * 4096 * 2048 * 2 + 2 * r * 512 * 2
+    assert big >= main
+    assert big < 1.15 * main + (1 << 22)
     assert small < big
 
 

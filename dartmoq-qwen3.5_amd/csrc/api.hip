@@ -21,9 +21,9 @@ static inline int scale_stride_for(int mode, int k) {
 
 static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE_FP4; }
 
-// K split across the four waves of a workgroup: small row tiles want parallelism along K,
-// large ones keep the waves on different output features
-static inline int pick_ks(int tt) { return tt == 1 ? 4 : (tt == 2 ? 2 : 1); }
+// K split across the four waves of a workgroup: a handful of routed rows leaves most CUs idle
+// unless every wave takes a quarter of K; otherwise the waves own different output features
+static inline int pick_ks(int tt, long rows) { return (tt == 1 && rows <= 64) ? 4 : 1; }
 
 extern "C" {
 
@@ -178,7 +178,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (!dmq_valid_bit(a->pool[i].bit)) return DMQ_ERR_BIT;
   if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
   if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SCATTER) return DMQ_ERR_MODE;
-  const int ks = a->ks > 0 ? a->ks : pick_ks(a->tt);
+  const int ks = a->ks > 0 ? a->ks : 1;
   if (!dmq_gemm_config_ok(a->tt, ks)) return DMQ_ERR_MODE;
   if (!a->items || !a->n_items || !a->out) return DMQ_ERR_NULL;
   for (int i = 0; i < a->n_pools; ++i) {
@@ -344,7 +344,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
   if (P > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
   if (tt <= 0) tt = pick_tt(tokens, K, E);
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
-  if (ks <= 0) ks = pick_ks(tt);
+  if (ks <= 0) ks = pick_ks(tt, (long)tokens * K);
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   const int rot_tt = (tt == 4) ? 4 : 1;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);

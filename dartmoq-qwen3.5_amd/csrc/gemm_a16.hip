@@ -2,3 +2,9 @@
 #include "gemm_dispatch.h"
 
 int dmq_gemm_launch_a16(const GemmLaunch& L) { return dmq_gemm_launch_mode<DMQ_MODE_A16>(L); }
+
+#ifdef DMQ_TRACE
+extern "C" int dmq_trace_read(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(dmq_trace_buf), sizeof(long long) * 256);
+}
+#endif

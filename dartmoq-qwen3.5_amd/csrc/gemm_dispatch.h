@@ -13,10 +13,10 @@ struct GemmLaunch {
   hipStream_t stream;
 };
 
-// instantiated (tt, ks) pairs: decode (1,4) (1,1); mid (2,2) (2,1); prefill (4,1) (4,2)
+// instantiated (tt, ks) pairs: 16-row tiles with K split over the waves (1,4) or not (1,1),
+// 32- and 64-row tiles with LDS-staged activations (2,1) (4,1)
 static inline bool dmq_gemm_config_ok(int tt, int ks) {
-  return (tt == 1 && (ks == 4 || ks == 1)) || (tt == 2 && (ks == 2 || ks == 1)) ||
-         (tt == 4 && (ks == 1 || ks == 2));
+  return (tt == 1 && (ks == 4 || ks == 1)) || (tt == 2 && ks == 1) || (tt == 4 && ks == 1);
 }
 
 template <int MODE, int TT, int KS, int EPI, bool DBG>
@@ -46,10 +46,8 @@ static int dmq_gemm_launch_mode(const GemmLaunch& L) {
     return DMQ_ERR_MODE;
   if (L.tt == 1 && L.ks == 4) return dmq_gemm_launch_epi<MODE, 1, 4>(L);
   if (L.tt == 1 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 1, 1>(L);
-  if (L.tt == 2 && L.ks == 2) return dmq_gemm_launch_epi<MODE, 2, 2>(L);
   if (L.tt == 2 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 2, 1>(L);
   if (L.tt == 4 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 4, 1>(L);
-  if (L.tt == 4 && L.ks == 2) return dmq_gemm_launch_epi<MODE, 4, 2>(L);
   return DMQ_ERR_MODE;
 }
 

@@ -4,10 +4,8 @@
 //
 // One launch covers every bit pool of a layer: a work item is (pool, expert, tile of 16*TT
 // activation rows) and a workgroup of four waves handles one item for one block of output
-// features.  Inside the workgroup the waves split the output features (ROWPARTS) and / or the
-// quantization groups (KS way split of K, reduced through LDS at the end); each wave owns NT
-// tiles of 16 weight rows and TT tiles of 16 activation rows and walks its share of K one
-// group (128 features) at a time:
+// features.  Each wave owns NT tiles of 16 weight rows and TT tiles of 16 activation rows and
+// walks K one quantization group (128 features) at a time:
 //
 //   * weights are the MFMA "A" operand: lane (n = lane % 16, q = lane / 16) owns the 32
 //     features [32q, 32q+32) of row n inside the group, i.e. 4*BIT consecutive packed
@@ -20,11 +18,27 @@
 //
 // The same mapping serves all four precision modes: a group is 4 MFMA steps of K=32
 // (fp16, e4m3), 2 steps of K=64 (int8) or 1 MX-scaled step of K=128 (e2m1).
+//
+// Two ways of feeding the waves, chosen by the K split KS:
+//   KS > 1  (few activation rows, HBM-bound on the packed weights): the four waves share the
+//           weight rows and split the groups; every wave issues the loads of its whole K
+//           slice (up to PF groups) before computing, so one memory latency covers the
+//           slice, and the partial sums meet in LDS at the end.
+//   KS == 1 (many activation rows): the waves take different weight rows and share the
+//           activation tile, which is staged once per group in LDS (double buffered,
+//           16-byte chunks XOR-swizzled by row so the operand reads spread over the banks).
 #pragma once
 #include "common.h"
 #include "lut.h"
 
-#define DMQ_MAX_POOLS 4
+#ifdef DMQ_TRACE
+static __device__ long long dmq_trace_buf[256];
+#define DMQ_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x == 0) { \
+    dmq_trace_buf[2 * (i)] = __builtin_readcyclecounter(); \
+    dmq_trace_buf[2 * (i) + 1] = wall_clock64(); } } while (0)
+#else
+#define DMQ_MARK(i)
+#endif
 
 struct PoolW {
   const uint8_t* w;            // [G_total, n_total, ppg] packed indices (FP4: folded e2m1, ppg = 64)
@@ -55,9 +69,9 @@ struct GemmParams {
   // outputs
   __half* out;                 // STORE / SILU: fp16 [rows, out_stride]
   long out_stride;
-  float* out_slots;            // SLOT: fp32 [rows, out_stride] addressed by row_slot[r]
-  const float* row_weight;     // SLOT: routing weight of logical row r
-  const int* row_slot;         // SLOT: destination row (token * top_k + slot) of logical row r
+  float* out_slots;            // SCATTER: fp32 [slots, out_stride] addressed by row_slot[r]
+  const float* row_weight;     // SCATTER: routing weight of logical row r
+  const int* row_slot;         // SCATTER: destination row (token * top_k + slot) of logical row r
   int* dbg_acc;                // optional int32 [rows, groups, n_out] per-group accumulators (A8)
 };
 
@@ -109,26 +123,55 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
   }
 }
 
-// LDS needed by the K-split reduction: every wave parks NT*TT tiles of 64 lanes x 4 floats
-template <int NT, int TT, int KS> struct RedGeom {
-  static constexpr int FLOATS = (KS > 1) ? 4 * NT * TT * 256 : 4; };
+// Groups in flight per wave on the staged path.  WW registers hold one (group, n-tile) of packed
+// weights; few activation rows leave registers for a deep ring, which is what hides the HBM
+// latency when a workgroup has little arithmetic per group.
+#ifndef DMQ_RING_TT1
+#define DMQ_RING_TT1 16
+#endif
+#ifndef DMQ_RING_TT2
+#define DMQ_RING_TT2 8
+#endif
+#ifndef DMQ_RING_TT4
+#define DMQ_RING_TT4 4
+#endif
+template <int WW, int TT> constexpr int dmq_ring_depth() {
+  constexpr int words = (TT == 1) ? DMQ_RING_TT1 : (TT == 2 ? DMQ_RING_TT2 : DMQ_RING_TT4);
+  constexpr int d = words / WW;                     // words of packed weights per n-tile in flight
+  return d < 2 ? 2 : (d > 8 ? 8 : d);
+}
+
+// Tiling facts shared by the kernel and its host launcher.
+template <int MODE, int NT, int TT, int KS> struct GemmGeom {
+  static constexpr int AW = ModeTraits<MODE>::ACT_WORDS;          // activation words per lane and group
+  static constexpr int AB = AW * 16;                              // activation bytes per row and group
+  static constexpr bool STAGE = (KS == 1);                        // activations through LDS
+  static constexpr int PF = 4;                                    // direct path: groups in flight
+  // staged path: one LDS slot = activation tile + norms of the 64*NT weight rows + tile scales
+  static constexpr int SLOT = 16 * TT * AB + 128 * NT + 64 * TT;
+  static constexpr int STAGE_BYTES = STAGE ? 2 * SLOT : 0;
+  static constexpr int RED_BYTES = (KS > 1) ? 4 * NT * TT * 1024 : 0;
+  static constexpr int SMEM2 = STAGE_BYTES > RED_BYTES ? (STAGE_BYTES > 16 ? STAGE_BYTES : 16)
+                                                       : (RED_BYTES > 16 ? RED_BYTES : 16);
+};
 
 template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
-                                              float* red, int eidx, int ttile, int nb) {
+                                              uint8_t* smem2, int eidx, int ttile, int nb) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
+  using GG = GemmGeom<MODE, NT, TT, KS>;
   constexpr int WW = WeightWords<MODE, BIT>::N;
-  constexpr int AW = T::ACT_WORDS;
+  constexpr int AW = GG::AW;
+  constexpr int AB = GG::AB;
+  constexpr bool STAGE = GG::STAGE;
+  constexpr int PF = GG::PF;
   constexpr int ROWPARTS = 4 / KS;                                   // waves along the features
   constexpr int UNIT = (EPI == DMQ_EPI_SILU) ? 2 : 1;                // tiles finalized together
   constexpr int UNITS = NT / UNIT;
   constexpr int FEAT_TILES = NT / UNIT;                              // output tiles per wave
   constexpr int PPG = (MODE == DMQ_MODE_FP4) ? 64 : (DMQ_GS * BIT / 8);
   static_assert(NT % UNIT == 0, "SiLU epilogue pairs gate/up tiles");
-
-  if (MODE != DMQ_MODE_FP4) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
-  __syncthreads();
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -145,12 +188,13 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   const int feat0 = (nb * ROWPARTS + rowpart) * (FEAT_TILES * 16);   // first output feature of the wave
   const bool wave_active = feat0 < p.n_out;                          // wave-uniform
 
-  // weight row of each n-tile
+  // weight row of each n-tile (inactive waves alias the first block; they never store)
+  const int featw = wave_active ? feat0 : 0;
   int wrow[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    if (EPI == DMQ_EPI_SILU) wrow[j] = slice_start + ((j & 1) ? p.half_width : 0) + feat0 + (j >> 1) * 16;
-    else wrow[j] = (p.slice_is_groups ? 0 : slice_start) + feat0 + j * 16;
+    if (EPI == DMQ_EPI_SILU) wrow[j] = slice_start + ((j & 1) ? p.half_width : 0) + featw + (j >> 1) * 16;
+    else wrow[j] = (p.slice_is_groups ? 0 : slice_start) + featw + j * 16;
   }
   const int g_base = p.slice_is_groups ? slice_start : 0;
   const int g_lo = (p.groups * kpart) / KS;
@@ -177,139 +221,285 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 #pragma unroll
     for (int t = 0; t < TT; ++t) total_acc[j][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  if (wave_active && g_lo < g_hi) {
-    uint32_t pk_n[NT][WW];
-    uint32_t xa_n[TT][AW];
-
-    auto fetch = [&](int g) {
-      const long gg = (long)(g_base + g) * pw.n_total;
+  // ---- loads of one group: packed weights, norms, activation scales (+ activations when direct)
+  auto load_weights = [&](int g, uint32_t (&pk)[NT][WW], uint2_t (&nr)[NT]) {
+    const long gg = (long)(g_base + g) * pw.n_total;
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        dmq_load_words<WW>(pw.w + (gg + wrow[j] + l16) * PPG + q * (WW * 4), pk_n[j]);
+    for (int j = 0; j < NT; ++j) {
+      dmq_load_words<WW>(pw.w + (gg + wrow[j] + l16) * PPG + q * (WW * 4), pk[j]);
+      nr[j] = *(const uint2_t*)(pw.norms + gg + wrow[j] + 4 * q);
+    }
+  };
+  auto load_scales = [&](int g, float (&xs)[TT], int (&xsb)[TT]) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      xs[t] = 1.0f; xsb[t] = 127;
+      if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
+        xs[t] = avalid[t] ? (float)((const __half*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g]
+                          : 0.f;
+      } else if (MODE == DMQ_MODE_FP4) {
+        if (avalid[t])
+          xsb[t] = ((const uint8_t*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g * 4 + q];
+      }
+    }
+  };
+  auto load_acts = [&](int g, uint32_t (&xa)[TT][AW]) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      if (avalid[t]) {
+        dmq_load_words<AW>(arow[t] + (long)g * (AW * 16), xa[t]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < AW; ++i) xa[t][i] = 0u;
+      }
+    }
+  };
+
+  // ---- MFMA work of one group
+  // The look-ups of n-tile j + 1 are issued before the MFMAs of n-tile j, so their LDS latency
+  // hides behind matrix work even when the wave has the SIMD to itself.
+  constexpr int OPW = (MODE == DMQ_MODE_FP8) ? 2 : 4;                // operand words per MFMA step
+  constexpr int WQ = (MODE == DMQ_MODE_FP4) ? 1 : T::STEPS * OPW;
+  auto dequant_tile = [&](const uint32_t (&pkj)[WW], uint32_t (&w)[WQ]) {
+    if constexpr (MODE != DMQ_MODE_FP4) {
+#pragma unroll
+      for (int s = 0; s < T::STEPS; ++s) dmq_dequant_step<MODE, BIT>(tbl, lane_base, pkj, s, w + s * OPW);
+    }
+  };
+  auto compute = [&](int g, const uint32_t (&pk)[NT][WW], const uint2_t (&nr)[NT],
+                     const uint32_t (&xa)[TT][AW], const float (&xs)[TT], const int (&xsb)[TT]) {
+    uint32_t wqb[2][WQ];
+    dequant_tile(pk[0], wqb[0]);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      if (j + 1 < NT) dequant_tile(pk[j + 1], wqb[(j + 1) & 1]);
+      const uint32_t (&wq)[WQ] = wqb[j & 1];
+      acc_t acc[TT];
+#pragma unroll
+      for (int t = 0; t < TT; ++t) acc[t] = (acc_t){0, 0, 0, 0};
+#pragma unroll
+      for (int s = 0; s < T::STEPS; ++s) {
+        if constexpr (MODE == DMQ_MODE_A16) {
+          half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[4 * s], wq[4 * s + 1], wq[4 * s + 2],
+                                                            wq[4 * s + 3]});
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            half8_t b = __builtin_bit_cast(half8_t, (uint4_t){xa[t][4 * s], xa[t][4 * s + 1],
+                                                              xa[t][4 * s + 2], xa[t][4 * s + 3]});
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[t], 0, 0, 0);
+          }
+        } else if constexpr (MODE == DMQ_MODE_A8) {
+          int4_t a = {(int)wq[4 * s], (int)wq[4 * s + 1], (int)wq[4 * s + 2], (int)wq[4 * s + 3]};
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            int4_t b = {(int)xa[t][4 * s], (int)xa[t][4 * s + 1], (int)xa[t][4 * s + 2],
+                        (int)xa[t][4 * s + 3]};
+            acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[t], 0, 0, 0);
+          }
+        } else if constexpr (MODE == DMQ_MODE_FP8) {
+          long a = (long)(((uint64_t)wq[2 * s + 1] << 32) | wq[2 * s]);
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            long b = (long)(((uint64_t)xa[t][2 * s + 1] << 32) | xa[t][2 * s]);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, b, acc[t], 0, 0, 0);
+          }
+        } else {
+          int8_t8 a = {(int)pk[j][0], (int)pk[j][1], (int)pk[j][2], (int)pk[j][3], 0, 0, 0, 0};
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            int8_t8 b = {(int)xa[t][0], (int)xa[t][1], (int)xa[t][2], (int)xa[t][3], 0, 0, 0, 0};
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                a, b, acc[t], 4, 4, 0, pw.w_scale_byte, 0, xsb[t]);
+          }
+        }
+      }
+      const half4_t h = __builtin_bit_cast(half4_t, nr[j]);
+      const float nrm[4] = {(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
-        if (avalid[t]) {
-          dmq_load_words<AW>(arow[t] + (long)g * (AW * 16), xa_n[t]);
-        } else {
 #pragma unroll
-          for (int i = 0; i < AW; ++i) xa_n[t][i] = 0u;
+        for (int r = 0; r < 4; ++r) {
+          float v = (float)acc[t][r];
+          if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) v = v * xs[t];
+          total_acc[j][t][r] += v * nrm[r];
+        }
+        if (DBG && MODE == DMQ_MODE_A8 && avalid[t] && wave_active) {
+          int4_t* d = (int4_t*)(p.dbg_acc + ((long)rlog[t] * p.groups + g) * p.n_out +
+                                feat0 + j * 16 + 4 * q);
+          *d = __builtin_bit_cast(int4_t, acc[t]);
+        }
+      }
+    }
+  };
+
+  if constexpr (!STAGE) {
+    // ------------------------------------------------------------------ direct path
+    uint32_t pk[PF][NT][WW];
+    uint2_t nr[PF][NT];
+    uint32_t xa[PF][TT][AW];
+    float xs[PF][TT];
+    int xsb[PF][TT];
+    auto load_chunk = [&](int g0) {
+#pragma unroll
+      for (int u = 0; u < PF; ++u) {
+        if (g0 + u < g_hi) {
+          load_weights(g0 + u, pk[u], nr[u]);
+          load_acts(g0 + u, xa[u]);
+          load_scales(g0 + u, xs[u], xsb[u]);
         }
       }
     };
+    // the first chunk is in flight while the look-up table is built
+    if (g_lo < g_hi) load_chunk(g_lo);
+    if (MODE != DMQ_MODE_FP4) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
+    __syncthreads();
+    for (int g0 = g_lo; g0 < g_hi; g0 += PF) {
+      if (g0 != g_lo) load_chunk(g0);
+#pragma unroll
+      for (int u = 0; u < PF; ++u)
+        if (g0 + u < g_hi) compute(g0 + u, pk[u], nr[u], xa[u], xs[u], xsb[u]);
+    }
+  } else {
+    // ------------------------------------------------------------------ LDS-staged operands
+    // Per group the workgroup shares one LDS slot: the 16*TT x AB activation tile (16-byte
+    // chunks XOR-swizzled by row), the 64*NT norms of its weight rows and the activation
+    // scales of the tile.  All of it and the packed weights travel D groups ahead of the MFMA
+    // work in rings of registers; the slot of group g + 1 is written while group g computes.
+    // Loads retire in order, so each iteration requests slot data before weights: the wait
+    // for the slot of group g + 1 then never covers weights younger than group g + 1.
+    constexpr int NC = AB / 16;                       // chunks per row
+    constexpr int CPT = (TT * NC >= 16) ? TT * NC / 16 : 1;   // chunks per thread
+    constexpr int TPR = NC / CPT;                     // threads per row
+    constexpr int ACT_BYTES = 16 * TT * AB;
+    constexpr int NORM_OFF = ACT_BYTES;
+    constexpr int SCALE_OFF = NORM_OFF + 128 * NT;
+    constexpr int SLOT = GG::SLOT;
+    constexpr bool SCALED = (MODE != DMQ_MODE_A16);
+    static_assert(NT <= 4, "a wave stages the norms of at most four n-tiles");
+    const int srow = threadIdx.x / TPR;               // >= 16*TT for threads without a chunk
+    const int sc0 = (threadIdx.x % TPR) * CPT;
+    const int s_rlog = r_first + srow;
+    const bool s_active = srow < 16 * TT;
+    const bool s_valid = s_active && s_rlog < r_end;
+    const int s_phys = s_valid ? (pw.row_index ? pw.row_index[s_rlog] : s_rlog) : 0;
+    const uint8_t* s_src = pw.act + (long)s_phys * p.act_row_bytes + sc0 * 16;
+    // lane (l16, q) stages the norm of row l16 of its wave's n-tile q
+    const bool n_active = q < NT;
+    const int n_row = (EPI == DMQ_EPI_SILU)
+        ? slice_start + ((q & 1) ? p.half_width : 0) + featw + (q >> 1) * 16 + l16
+        : (p.slice_is_groups ? 0 : slice_start) + featw + q * 16 + l16;
+    // thread t < 16*TT stages the scale word of tile row t
+    const int c_rlog = r_first + (int)threadIdx.x;
+    const bool c_active = SCALED && threadIdx.x < 16 * TT;
+    const bool c_valid = c_active && c_rlog < r_end;
+    const int c_phys = c_valid ? (pw.row_index ? pw.row_index[c_rlog] : c_rlog) : 0;
+    uint8_t* stage = smem2;
 
-    fetch(g_lo);
-    for (int g = g_lo; g < g_hi; ++g) {
-      uint32_t pk[NT][WW];
-      uint32_t xa[TT][AW];
+    struct Staged { uint4_t a[CPT]; uint32_t nrm; uint32_t sc; };
+    auto stage_load = [&](int g, Staged& sr) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int i = 0; i < WW; ++i) pk[j][i] = pk_n[j][i];
-#pragma unroll
-      for (int t = 0; t < TT; ++t)
-#pragma unroll
-        for (int i = 0; i < AW; ++i) xa[t][i] = xa_n[t][i];
-
-      // per-group scales: 4 consecutive norms per n-tile, one activation scale per token tile
-      const long gg = (long)(g_base + g) * pw.n_total;
-      float nrm[NT][4];
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        half4_t h = *(const half4_t*)(pw.norms + gg + wrow[j] + 4 * q);
-        nrm[j][0] = (float)h[0]; nrm[j][1] = (float)h[1];
-        nrm[j][2] = (float)h[2]; nrm[j][3] = (float)h[3];
+      for (int c = 0; c < CPT; ++c)
+        sr.a[c] = s_valid ? *(const uint4_t*)(s_src + (long)g * AB + c * 16) : (uint4_t){0u, 0u, 0u, 0u};
+      sr.nrm = n_active ? *(const uint16_t*)(pw.norms + (long)(g_base + g) * pw.n_total + n_row) : 0u;
+      sr.sc = 0u;
+      if constexpr (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
+        if (c_valid) sr.sc = ((const uint16_t*)pw.act_scale)[(long)c_phys * p.act_scale_stride + g];
+      } else if constexpr (MODE == DMQ_MODE_FP4) {
+        sr.sc = 0x7f7f7f7fu;
+        if (c_valid)
+          sr.sc = *(const uint32_t*)((const uint8_t*)pw.act_scale + (long)c_phys * p.act_scale_stride + g * 4);
       }
-      float xs[TT];
-      int xsb[TT];
+    };
+    auto stage_store = [&](int buf, const Staged& sr) {
+      uint8_t* slot = stage + buf * SLOT;
+      if (s_active) {
+        uint8_t* base = slot + srow * AB;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c)
+          *(uint4_t*)(base + (((sc0 + c) ^ (srow & (NC - 1))) * 16)) = sr.a[c];
+      }
+      if (n_active) *(uint16_t*)(slot + NORM_OFF + ((wave * NT + q) * 16 + l16) * 2) = (uint16_t)sr.nrm;
+      if (c_active) *(uint32_t*)(slot + SCALE_OFF + threadIdx.x * 4) = sr.sc;
+    };
+    auto stage_read = [&](int buf, uint32_t (&xa)[TT][AW], uint2_t (&nr)[NT], float (&xs)[TT],
+                          int (&xsb)[TT]) {
+      const uint8_t* slot = stage + buf * SLOT;
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
+        const int row = t * 16 + l16;
+        const uint8_t* base = slot + row * AB;
+#pragma unroll
+        for (int i = 0; i < AW / 4; ++i) {
+          const int c = q * (AW / 4) + i;
+          uint4_t v = *(const uint4_t*)(base + ((c ^ (row & (NC - 1))) * 16));
+          xa[t][4 * i] = v.x; xa[t][4 * i + 1] = v.y; xa[t][4 * i + 2] = v.z; xa[t][4 * i + 3] = v.w;
+        }
         xs[t] = 1.0f; xsb[t] = 127;
-        if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
-          xs[t] = avalid[t] ? (float)((const __half*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g]
-                            : 0.f;
-        } else if (MODE == DMQ_MODE_FP4) {
-          if (avalid[t])
-            xsb[t] = ((const uint8_t*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g * 4 + q];
+        if constexpr (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
+          xs[t] = (float)__builtin_bit_cast(_Float16, *(const uint16_t*)(slot + SCALE_OFF + row * 4));
+        } else if constexpr (MODE == DMQ_MODE_FP4) {
+          xsb[t] = *(const uint8_t*)(slot + SCALE_OFF + row * 4 + q);
         }
       }
-
-      if (g + 1 < g_hi) fetch(g + 1);
-
-      acc_t acc[NT][TT];
 #pragma unroll
       for (int j = 0; j < NT; ++j)
+        nr[j] = *(const uint2_t*)(slot + NORM_OFF + ((wave * NT + j) * 16 + 4 * q) * 2);
+    };
+    auto load_packed = [&](int g, uint32_t (&pk)[NT][WW]) {
+      const long gg = (long)(g_base + g) * pw.n_total;
 #pragma unroll
-        for (int t = 0; t < TT; ++t) acc[j][t] = (acc_t){0, 0, 0, 0};
+      for (int j = 0; j < NT; ++j)
+        dmq_load_words<WW>(pw.w + (gg + wrow[j] + l16) * PPG + q * (WW * 4), pk[j]);
+    };
 
+    // Every load below is unconditional (group indices past the end are clamped to the last
+    // group, whose data is simply fetched again) and ring entry u is refilled only after its
+    // last use in program order: the loaded registers then carry straight across the loop's
+    // back edge, with no copy that would have to wait for loads still in flight.
+    constexpr int D = dmq_ring_depth<WW, TT>();
+    static_assert(D % 2 == 0, "the LDS slot of a ring entry is fixed by its parity");
+    uint32_t pkb[D][NT][WW];
+    Staged srb[D];
+    const int g_last = g_hi - 1;
 #pragma unroll
-      for (int s = 0; s < T::STEPS; ++s) {
+    for (int u = 0; u < D; ++u) {
+      const int gl = (g_lo + u < g_last) ? g_lo + u : g_last;
+      stage_load(gl, srb[u]);
+      load_packed(gl, pkb[u]);
+    }
+    DMQ_MARK(1);
+    if (MODE != DMQ_MODE_FP4) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
+    DMQ_MARK(2);
+    stage_store(0, srb[0]);
+    __syncthreads();
+    DMQ_MARK(3);
+    for (int gb = g_lo; gb < g_hi; gb += D) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          if constexpr (MODE == DMQ_MODE_A16) {
-            uint32_t wq[4];
-            dmq_dequant_step<MODE, BIT>(tbl, lane_base, pk[j], s, wq);
-            half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[0], wq[1], wq[2], wq[3]});
-#pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              half8_t b = __builtin_bit_cast(half8_t, (uint4_t){xa[t][4 * s], xa[t][4 * s + 1],
-                                                                xa[t][4 * s + 2], xa[t][4 * s + 3]});
-              acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j][t], 0, 0, 0);
-            }
-          } else if constexpr (MODE == DMQ_MODE_A8) {
-            uint32_t wq[4];
-            dmq_dequant_step<MODE, BIT>(tbl, lane_base, pk[j], s, wq);
-            int4_t a = {(int)wq[0], (int)wq[1], (int)wq[2], (int)wq[3]};
-#pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              int4_t b = {(int)xa[t][4 * s], (int)xa[t][4 * s + 1], (int)xa[t][4 * s + 2],
-                          (int)xa[t][4 * s + 3]};
-              acc[j][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[j][t], 0, 0, 0);
-            }
-          } else if constexpr (MODE == DMQ_MODE_FP8) {
-            uint32_t wq[2];
-            dmq_dequant_step<MODE, BIT>(tbl, lane_base, pk[j], s, wq);
-            long a = (long)(((uint64_t)wq[1] << 32) | wq[0]);
-#pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              long b = (long)(((uint64_t)xa[t][2 * s + 1] << 32) | xa[t][2 * s]);
-              acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, b, acc[j][t], 0, 0, 0);
-            }
-          } else {
-            int8_t8 a = {(int)pk[j][0], (int)pk[j][1], (int)pk[j][2], (int)pk[j][3], 0, 0, 0, 0};
-#pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              int8_t8 b = {(int)xa[t][0], (int)xa[t][1], (int)xa[t][2], (int)xa[t][3], 0, 0, 0, 0};
-              acc[j][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                  a, b, acc[j][t], 4, 4, 0, pw.w_scale_byte, 0, xsb[t]);
-            }
-          }
+      for (int u = 0; u < D; ++u) {
+        const int g = gb + u;
+        const int gl = (g + D < g_last) ? g + D : g_last;
+        stage_load(gl, srb[u]);                        // entry u went to LDS one step ago
+        if (g < g_hi) {                                // uniform over the workgroup
+          uint32_t xa[TT][AW];
+          uint2_t nr[NT];
+          float xs[TT];
+          int xsb[TT];
+          stage_read(u & 1, xa, nr, xs, xsb);
+          compute(g, pkb[u], nr, xa, xs, xsb);
         }
+        load_packed(gl, pkb[u]);
+        stage_store((u & 1) ^ 1, srb[(u + 1) % D]);
+        __syncthreads();
+        DMQ_MARK(4 + g);
       }
-
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int t = 0; t < TT; ++t) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float v = (float)acc[j][t][r];
-            if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) v = v * xs[t];
-            total_acc[j][t][r] += v * nrm[j][r];
-          }
-          if (DBG && MODE == DMQ_MODE_A8 && avalid[t]) {
-            int4_t* d = (int4_t*)(p.dbg_acc + ((long)rlog[t] * p.groups + g) * p.n_out +
-                                  feat0 + j * 16 + 4 * q);
-            *d = __builtin_bit_cast(int4_t, acc[j][t]);
-          }
-        }
     }
   }
 
   // ------------------------------------------------------------------ K-split reduction
   // unit u (a tile, or a gate/up pair) is finalized by the wave with kpart == owner(u); the
   // other waves of the K group park their partial sums in LDS.
-  if (KS > 1) {
-    float4_t* red4 = (float4_t*)red;
+  if constexpr (KS > 1) {
+    float4_t* red4 = (float4_t*)smem2;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       const int owner = ((j / UNIT) * KS) / UNITS;
@@ -363,6 +553,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       }
     }
   }
+  DMQ_MARK(60);
 }
 
 template <int MODE, int TT, int EPI, int KS, bool DBG>
@@ -370,8 +561,9 @@ __global__ __launch_bounds__(256)
 void dmq_gemm_gf_kernel(GemmParams p) {
   constexpr int NT = 4;
   __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
-  __shared__ __attribute__((aligned(16))) float red[RedGeom<NT, TT, KS>::FLOATS];
+  __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2];
 
+  DMQ_MARK(0);
   const int item = blockIdx.x / p.n_blocks;
   if (item >= p.n_items[0]) return;
   const int nb = blockIdx.x - item * p.n_blocks;
@@ -381,12 +573,12 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE) return;
   if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb);
-    return;
-  }
-  switch (pw.bit) {
-    case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb); break;
-    case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb); break;
-    default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, red, eidx, ttile, nb); break;
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb);
+  } else {
+    switch (pw.bit) {
+      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb); break;
+      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb); break;
+      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb); break;
+    }
   }
 }

@@ -237,8 +237,8 @@ def pick_tt(rows_total: int, n_experts: int) -> int:
     return 1 if avg <= 8 else (2 if avg <= 48 else 4)
 
 
-def pick_ks(tt: int) -> int:
-    return {1: 4, 2: 2, 4: 1}[tt]
+def pick_ks(tt: int, rows_total: int) -> int:
+    return 4 if (tt == 1 and rows_total <= 64) else 1
 
 
 def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=None, w_scale_byte=127):

@@ -159,7 +159,7 @@ typedef struct {
   int mode;                 /* DMQ_MODE_* */
   int epi;                  /* DMQ_EPI_* */
   int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4 */
-  int ks;                   /* waves of a workgroup splitting K: 0 = pick, else 1, 2 or 4 */
+  int ks;                   /* waves of a workgroup splitting K: 0 = 1; 4 or 1 for tt == 1, else 1 */
   int n_pools;
   dmq_gemm_pool pool[DMQ_MAX_POOLS];
   long act_row_bytes;

@@ -183,7 +183,7 @@ def test_silu_and_scatter_epilogues():
     torch.testing.assert_close(out, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
 
 
-@pytest.mark.parametrize("tt,ks", [(1, 4), (1, 1), (2, 2), (2, 1), (4, 1), (4, 2)])
+@pytest.mark.parametrize("tt,ks", [(1, 4), (1, 1), (2, 1), (4, 1)])
 def test_k_split_variants_agree(tt, ks):
     """Every (row tile, K split) instantiation computes the same GEMM."""
     from dartmoq_hip import ops

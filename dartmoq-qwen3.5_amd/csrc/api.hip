@@ -27,7 +27,7 @@ static inline int pick_ks(int tt, long rows) { return (tt == 1 && rows <= 64) ? 
 
 extern "C" {
 
-int dmq_abi_version(void) { return 2; }
+int dmq_abi_version(void) { return 3; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -84,23 +84,37 @@ int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts,
                                (int*)out_idx, (hipStream_t)stream);
 }
 
+size_t dmq_route_scratch_bytes(int tokens, int k, int experts) {
+  if (tokens <= 0 || k <= 0 || experts <= 0) return 0;
+  int chunk_rows, n_chunks;
+  dmq_sort_chunks((long)tokens * k, &chunk_rows, &n_chunks);
+  return (size_t)n_chunks * experts * sizeof(int);
+}
+
 int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
                       int pools, const void* slice_start, const void* slice_count, int tile_rows,
                       int max_items, void* counts, void* offsets, void* sorted_tokens,
                       void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
-                      void* n_items, void* items, void* stream) {
+                      void* n_items, void* items, void* scratch, size_t scratch_bytes,
+                      void* stream) {
   if (!topk_idx || !topk_w || !slice_start || !slice_count || !counts || !offsets ||
-      !sorted_tokens || !sorted_weights || !sorted_rows || !gu_info || !dn_info || !n_items || !items)
+      !sorted_tokens || !sorted_weights || !sorted_rows || !gu_info || !dn_info || !n_items ||
+      !items || !scratch)
     return DMQ_ERR_NULL;
   if (tokens <= 0 || k <= 0 || experts <= 0 || pools <= 0) return DMQ_ERR_SHAPE;
-  if (pools > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
+  if (pools > DMQ_MAX_POOLS || experts > DMQ_SORT_MAX_EXPERTS) return DMQ_ERR_LIMIT;
   if (tile_rows <= 0 || tile_rows % 16) return DMQ_ERR_ALIGN;
-  PlanParams plan{(const int*)counts, experts, pools, tile_rows, max_items,
-                  (const int*)slice_start, (const int*)slice_count, (int*)offsets, (int*)gu_info,
-                  (int*)dn_info, (int*)n_items, (int*)items};
-  return dmq_route_permute_launch((const int*)topk_idx, (const float*)topk_w, tokens, k, (int*)counts,
-                                  plan, (int*)sorted_tokens, (float*)sorted_weights,
-                                  (int*)sorted_rows, (hipStream_t)stream);
+  if (scratch_bytes < dmq_route_scratch_bytes(tokens, k, experts)) return DMQ_ERR_LIMIT;
+  PlanParams plan{};
+  plan.counts = (int*)counts; plan.hist = (int*)scratch;
+  dmq_sort_chunks((long)tokens * k, &plan.chunk_rows, &plan.n_chunks);
+  plan.experts = experts; plan.pools = pools; plan.tile_rows = tile_rows; plan.max_items = max_items;
+  plan.slice_start_rows = (const int*)slice_start; plan.slice_count_rows = (const int*)slice_count;
+  plan.offsets = (int*)offsets; plan.gu_info = (int*)gu_info; plan.dn_info = (int*)dn_info;
+  plan.n_items = (int*)n_items; plan.items = (int*)items;
+  return dmq_route_permute_launch((const int*)topk_idx, (const float*)topk_w, tokens, k, plan,
+                                  (int*)sorted_tokens, (float*)sorted_weights, (int*)sorted_rows,
+                                  (hipStream_t)stream);
 }
 
 int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_items, int pool,
@@ -272,6 +286,8 @@ struct MoeWorkspace {
   uint8_t* xq[DMQ_MAX_POOLS];        // hoisted pools: codes by token; others share xq_rows
   uint8_t* xq_scale[DMQ_MAX_POOLS];
   uint8_t *xq_rows, *xq_rows_scale, *act, *actq, *actq_scale;
+  void* sort_scratch;
+  size_t sort_scratch_bytes;
   int max_items, tile_rows;
   size_t bytes;
 };
@@ -299,6 +315,8 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.gu_info = (int*)take(P * E * 16);
   w.dn_info = (int*)take(P * E * 16);
   w.n_items = (int*)take(16);
+  w.sort_scratch_bytes = dmq_route_scratch_bytes(tokens, L->top_k, L->experts);
+  w.sort_scratch = take(w.sort_scratch_bytes);
   w.items = (int*)take((size_t)w.max_items * 16);
   w.slots = (float*)take(R * H * 4);
   for (size_t i = 0; i < DMQ_MAX_POOLS; ++i) {
@@ -373,7 +391,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
   rc = dmq_route_permute(topk_idx, topk_w, tokens, K, E, P, layer->slice_start, layer->slice_count,
                          w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
                          w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items, w.items,
-                         stream);
+                         w.sort_scratch, w.sort_scratch_bytes, stream);
   if (rc) return rc;
   mark(1);
 

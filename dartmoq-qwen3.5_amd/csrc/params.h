@@ -47,8 +47,23 @@ struct QuantParams {
   float extra_scale;
 };
 
+// Chunking of the routed rows for the counting sort: at most DMQ_SORT_MAX_CHUNKS chunks of a
+// multiple of 64 rows.
+#define DMQ_SORT_MAX_EXPERTS 2048
+#define DMQ_SORT_MAX_CHUNKS 64
+static inline void dmq_sort_chunks(long rows, int* chunk_rows, int* n_chunks) {
+  long cr = (rows + DMQ_SORT_MAX_CHUNKS - 1) / DMQ_SORT_MAX_CHUNKS;
+  cr = (cr + 63) / 64 * 64;
+  if (cr < 64) cr = 64;
+  *chunk_rows = (int)cr;
+  *n_chunks = (int)((rows + cr - 1) / cr);
+}
+
 struct PlanParams {
-  const int* counts;
+  int* counts;                   // [experts] rows per expert (written by the plan kernel)
+  int* hist;                     // [n_chunks, experts] chunk histogram, then chunk start positions
+  int chunk_rows;
+  int n_chunks;
   int experts;
   int pools;
   int tile_rows;                 // rows per work item
@@ -67,7 +82,7 @@ int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
 int dmq_route_topk_launch(const void* logits, int logits_fp16, int tokens, int experts, int k,
                           int renorm, float* out_w, int* out_idx, hipStream_t stream);
 int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int tokens, int k,
-                             int* counts, const PlanParams& plan, int* sorted_tokens,
+                             const PlanParams& plan, int* sorted_tokens,
                              float* sorted_weights, int* sorted_rows, hipStream_t stream);
 int dmq_items_from_info_launch(const int* expert_info, int experts, int tile_rows, int max_items,
                                int pool, int* n_items, int* items, hipStream_t stream);

@@ -1,13 +1,14 @@
 // Top-k routing and token permutation: sort the T*k routed rows by expert (stable) and
 // partition the experts of every bit pool into tiles of activation rows, all on the device
-// (no host synchronisation, no atomics, deterministic output order).
+// (no host synchronisation, no global atomics, deterministic output order).
 //
-//   1. dmq_topk_kernel         one wave per token: softmax statistics + k arg-max rounds
-//   2. dmq_expert_count_kernel one wave per expert: count rows routed to it
-//   3. dmq_plan_kernel         one workgroup: exclusive scan -> offsets, per-pool expert_info
-//                              and the work-item list (pool, expert, row tile) of the layer
-//   4. dmq_expert_fill_kernel  one wave per expert: write its rows in (token, slot) order
-//   5. dmq_combine_kernel      out[t] = sum over the k slot rows of token t (fixed order)
+//   1. dmq_topk_kernel        one wave per token: softmax statistics + k arg-max rounds
+//   2. dmq_chunk_count_kernel one wave per chunk of rows: per-chunk expert histogram (LDS)
+//   3. dmq_plan_kernel        one workgroup: counts, exclusive scan -> offsets, start position
+//                             of every (chunk, expert), per-pool expert_info and the work-item
+//                             list (pool, expert, row tile) of the layer
+//   4. dmq_chunk_fill_kernel  one wave per chunk: write its rows to their sorted positions
+//   5. dmq_combine_kernel     out[t] = sum over the k slot rows of token t (fixed order)
 #include "params.h"
 
 // ------------------------------------------------------------------------------ top-k
@@ -74,34 +75,29 @@ void dmq_topk_kernel(const T* logits, int tokens, int experts, int k, int renorm
 }
 
 // ------------------------------------------------------------------------------ counting
-// Each lane inspects 8 consecutive rows per step (two 16-byte loads), a wave 512 rows.
-__device__ __forceinline__ void load8(const int* p, int base, int rows, int* v) {
-  if (base + 8 <= rows) {
-    int4_t a = *(const int4_t*)(p + base);
-    int4_t b = *(const int4_t*)(p + base + 4);
-    v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3];
-    v[4] = b[0]; v[5] = b[1]; v[6] = b[2]; v[7] = b[3];
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (base + i < rows) ? p[base + i] : -1;
-  }
-}
-
+// The routed rows (token-major, k per token) are cut into chunks of chunk_rows; one wave owns a
+// chunk and walks it 64 rows at a time.  hist[c, e] first holds the number of rows of chunk c
+// routed to expert e; the plan kernel turns it into the position of the first such row in the
+// expert-sorted order, which makes the permutation a stable counting sort.
 __global__ __launch_bounds__(256)
-void dmq_expert_count_kernel(const int* topk_idx, int rows, int experts, int* counts) {
+void dmq_chunk_count_kernel(const int* topk_idx, int rows, int experts, int chunk_rows, int n_chunks,
+                            int* hist) {
+  __shared__ int cnt_all[4 * DMQ_SORT_MAX_EXPERTS];
   const int lane = threadIdx.x & 63;
-  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (e >= experts) return;
-  int c = 0;
-  for (int base = lane * 8; base < rows; base += 512) {
-    int v[8];
-    load8(topk_idx, base, rows, v);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) c += (v[i] == e) ? 1 : 0;
+  const int wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 4 + wave;
+  if (c >= n_chunks) return;
+  int* cnt = cnt_all + wave * DMQ_SORT_MAX_EXPERTS;
+  for (int e = lane; e < experts; e += 64) cnt[e] = 0;
+  __builtin_amdgcn_wave_barrier();
+  const int r0 = c * chunk_rows;
+  const int r1 = min(rows, r0 + chunk_rows);
+  for (int r = r0 + lane; r < r1; r += 64) {
+    const int e = topk_idx[r];
+    if (e >= 0 && e < experts) atomicAdd(&cnt[e], 1);
   }
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) c += __shfl_xor(c, m, 64);
-  if (lane == 0) counts[e] = c;
+  __builtin_amdgcn_wave_barrier();
+  for (int e = lane; e < experts; e += 64) hist[(long)c * experts + e] = cnt[e];
 }
 
 // inclusive scan over the 1024 threads of the workgroup (16 waves)
@@ -127,6 +123,13 @@ void dmq_plan_kernel(PlanParams p) {
   __shared__ int carry;
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
+  // rows per expert: column sums of the chunk histogram
+  for (int e = tid; e < p.experts; e += 1024) {
+    int total = 0;
+#pragma unroll 8
+    for (int c = 0; c < p.n_chunks; ++c) total += p.hist[(long)c * p.experts + e];
+    p.counts[e] = total;
+  }
   __syncthreads();
   // expert offsets: exclusive scan of counts, 1024 experts per pass
   for (int base = 0; base < p.experts; base += 1024) {
@@ -140,6 +143,20 @@ void dmq_plan_kernel(PlanParams p) {
   }
   if (tid == 0) p.offsets[0] = 0;
   __syncthreads();
+  // hist[c, e] <- position of the first row of chunk c routed to expert e
+  for (int e = tid; e < p.experts; e += 1024) {
+    int at = p.offsets[e + 1] - p.counts[e];
+    for (int c0 = 0; c0 < p.n_chunks; c0 += 8) {
+      int h[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) h[i] = (c0 + i < p.n_chunks) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (c0 + i < p.n_chunks) p.hist[(long)(c0 + i) * p.experts + e] = at;
+        at += h[i];
+      }
+    }
+  }
 
   // per-pool expert_info and the work-item list, pools in caller order, experts ascending
   if (tid == 0) carry = 0;
@@ -175,41 +192,41 @@ void dmq_plan_kernel(PlanParams p) {
   if (tid == 0) p.n_items[0] = min(carry, p.max_items);
 }
 
+// Stable scatter of one chunk.  The rows of one token name distinct experts, so the lanes of a
+// token bump distinct counters; tokens are taken one after the other and LDS executes a wave's
+// operations in order, hence rows of an expert keep their original order.
 __global__ __launch_bounds__(256)
-void dmq_expert_fill_kernel(const int* topk_idx, const float* topk_w, int rows, int k, int experts,
-                            const int* offsets, int* sorted_tokens, float* sorted_weights,
-                            int* sorted_rows) {
+void dmq_chunk_fill_kernel(const int* topk_idx, const float* topk_w, int rows, int k, int experts,
+                           int chunk_rows, int n_chunks, const int* hist, int* sorted_tokens,
+                           float* sorted_weights, int* sorted_rows) {
+  __shared__ int pos_all[4 * DMQ_SORT_MAX_EXPERTS];
   const int lane = threadIdx.x & 63;
-  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (e >= experts) return;
-  int pos = offsets[e];
-  const int end = offsets[e + 1];
-  if (pos == end) return;
-  for (int base0 = 0; base0 < rows; base0 += 512) {
-    const int base = base0 + lane * 8;
-    int v[8];
-    load8(topk_idx, base, rows, v);
-    int hits = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) hits += (v[i] == e) ? 1 : 0;
-    int incl = hits;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      int o = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += o;
+  const int wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 4 + wave;
+  if (c >= n_chunks) return;
+  int* pos = pos_all + wave * DMQ_SORT_MAX_EXPERTS;
+  for (int e = lane; e < experts; e += 64) pos[e] = hist[(long)c * experts + e];
+  __builtin_amdgcn_wave_barrier();
+  const int r0 = c * chunk_rows;
+  const int r1 = min(rows, r0 + chunk_rows);
+  for (int base = r0; base < r1; base += 64) {
+    const int r = base + lane;
+    const bool in = r < r1;
+    const int e = in ? topk_idx[r] : -1;
+    const float w = in ? topk_w[r] : 0.f;
+    const bool hit = e >= 0 && e < experts;
+    const int tok = r / k;
+    const int tok_first = base / k;
+    const int tok_last = (min(base + 64, r1) - 1) / k;
+    int at = -1;
+    for (int t = tok_first; t <= tok_last; ++t) {
+      if (hit && tok == t) at = atomicAdd(&pos[e], 1);
     }
-    int at = pos + incl - hits;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (v[i] == e) {
-        const int r = base + i;
-        sorted_tokens[at] = r / k;
-        sorted_weights[at] = topk_w[r];
-        sorted_rows[at] = r;
-        ++at;
-      }
+    if (at >= 0) {
+      sorted_tokens[at] = tok;
+      sorted_weights[at] = w;
+      sorted_rows[at] = r;
     }
-    pos += __shfl(incl, 63, 64);
   }
 }
 
@@ -281,16 +298,18 @@ int dmq_route_topk_launch(const void* logits, int logits_fp16, int tokens, int e
 }
 
 int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int tokens, int k,
-                             int* counts, const PlanParams& plan, int* sorted_tokens,
+                             const PlanParams& plan, int* sorted_tokens,
                              float* sorted_weights, int* sorted_rows, hipStream_t stream) {
   const int rows = tokens * k;
   const int experts = plan.experts;
-  const int grid_e = (experts + 3) / 4;
-  hipLaunchKernelGGL(dmq_expert_count_kernel, dim3(grid_e), dim3(256), 0, stream, topk_idx, rows,
-                     experts, counts);
+  if (experts > DMQ_SORT_MAX_EXPERTS) return DMQ_ERR_LIMIT;
+  const int grid_c = (plan.n_chunks + 3) / 4;
+  hipLaunchKernelGGL(dmq_chunk_count_kernel, dim3(grid_c), dim3(256), 0, stream, topk_idx, rows,
+                     experts, plan.chunk_rows, plan.n_chunks, plan.hist);
   hipLaunchKernelGGL(dmq_plan_kernel, dim3(1), dim3(1024), 0, stream, plan);
-  hipLaunchKernelGGL(dmq_expert_fill_kernel, dim3(grid_e), dim3(256), 0, stream, topk_idx, topk_w,
-                     rows, k, experts, plan.offsets, sorted_tokens, sorted_weights, sorted_rows);
+  hipLaunchKernelGGL(dmq_chunk_fill_kernel, dim3(grid_c), dim3(256), 0, stream, topk_idx, topk_w,
+                     rows, k, experts, plan.chunk_rows, plan.n_chunks, plan.hist, sorted_tokens,
+                     sorted_weights, sorted_rows);
   return dmq_check_launch();
 }
 

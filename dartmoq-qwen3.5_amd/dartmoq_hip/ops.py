@@ -134,12 +134,15 @@ def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_
         "items": torch.zeros((max_items, 4), **i32),
         "max_items": max_items, "tile_rows": tile_rows,
     }
+    scratch = torch.empty(max(1, load().dmq_route_scratch_bytes(t, k, num_experts)),
+                          dtype=torch.uint8, device=dev)
     check(load().dmq_route_permute(
         _ptr(topk_idx.to(torch.int32).contiguous()), _ptr(topk_w.float().contiguous()), t, k,
         num_experts, pools, _ptr(slice_start.contiguous()), _ptr(slice_count.contiguous()), tile_rows,
         max_items, _ptr(res["counts"]), _ptr(res["offsets"]), _ptr(res["sorted_tokens"]),
         _ptr(res["sorted_weights"]), _ptr(res["sorted_rows"]), _ptr(res["gu_info"]),
-        _ptr(res["dn_info"]), _ptr(res["n_items"]), _ptr(res["items"]), _stream(dev)), "route_permute")
+        _ptr(res["dn_info"]), _ptr(res["n_items"]), _ptr(res["items"]), _ptr(scratch),
+        scratch.numel(), _stream(dev)), "route_permute")
     return res
 
 

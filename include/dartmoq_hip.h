@@ -44,7 +44,7 @@ enum { DMQ_MODE_A16 = 0, DMQ_MODE_A8 = 1, DMQ_MODE_FP8 = 2, DMQ_MODE_FP4 = 3 };
 enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 
-/* Library / build identification: returns the ABI version (currently 2). */
+/* Library / build identification: returns the ABI version (currently 3). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -96,12 +96,16 @@ int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts,
  *   counts [experts], offsets [experts+1], sorted_tokens [tokens*k],
  *   sorted_weights fp32 [tokens*k], sorted_rows [tokens*k] (token*k + slot of each sorted row),
  *   gu_info / dn_info [pools, experts, 4], n_items [1], items [max_items, 4] (all pools,
- *   pool-major, experts ascending). */
+ *   pool-major, experts ascending).
+ * scratch: device memory of at least dmq_route_scratch_bytes(tokens, k, experts) bytes
+ * (per-chunk expert histograms of the counting sort).  experts <= 2048. */
+size_t dmq_route_scratch_bytes(int tokens, int k, int experts);
 int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
                       int pools, const void* slice_start, const void* slice_count, int tile_rows,
                       int max_items, void* counts, void* offsets, void* sorted_tokens,
                       void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
-                      void* n_items, void* items, void* stream);
+                      void* n_items, void* items, void* scratch, size_t scratch_bytes,
+                      void* stream);
 
 /* Work items for a caller-built expert_info: n_items int32[1], items int32 [max_items, 4]
  * with the given pool id. */

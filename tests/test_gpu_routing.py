@@ -82,3 +82,22 @@ def test_permute_matches_oracle(tokens, tile_rows):
     n = int(res["n_items"][0])
     assert n == len(exp_items)
     assert [tuple(r) for r in res["items"][:n].cpu().tolist()] == exp_items
+
+
+@pytest.mark.parametrize("tokens,experts,k", [(700, 100, 3), (1000, 37, 1), (333, 300, 5), (5000, 256, 8)])
+def test_permute_odd_shapes(tokens, experts, k):
+    """Tokens whose k rows straddle the 64-row steps of the sort, expert counts off the wave size."""
+    from dartmoq_hip import ops
+    logits = routing.zipf_logits(tokens, experts, seed=7 * tokens + k)
+    w, idx = routing.route_topk(logits, k)
+    toks, wts, slots, offs = routing.sort_by_expert(idx, w, experts)
+    start = torch.arange(experts, dtype=torch.int32).reshape(1, experts) * 512
+    count = torch.full((1, experts), 512, dtype=torch.int32)
+    res = ops.route_permute(idx.cuda().int(), w.cuda(), experts, start.cuda(), count.cuda(), 16)
+    torch.cuda.synchronize()
+    assert torch.equal(res["offsets"].cpu().long(), offs)
+    assert torch.equal(res["sorted_tokens"].cpu().long(), toks)
+    assert torch.equal(res["sorted_rows"].cpu().long(), toks * k + slots)
+    assert torch.equal(res["sorted_weights"].cpu(), wts)
+    n = int(res["n_items"][0])
+    assert n == int(sum(-(-int(c) // 16) for c in (offs[1:] - offs[:-1])))

@@ -20,8 +20,11 @@
  *   mode                  DMQ_MODE_A16 / A8 / FP8 / FP4
  *   expert_info           int32 [n_experts, 4] = token_start, token_count,
  *                         slice_start, slice_count   (device memory)
- *   work items            int32 [n, 4] = pool, expert index, row tile inside the expert, 0;
- *                         a row tile covers tile_rows = 16*tt activation rows
+ *   work items            int32 [n, DMQ_ITEM_WORDS] = pool, expert index, row tile inside the
+ *                         expert, token_start, token_count, slice_start in weight rows
+ *                         (gate_up), slice_start in groups (down), 0; a row tile covers
+ *                         tile_rows = 16*tt activation rows.  Items made by dmq_build_tiles
+ *                         carry the slice_start of their expert_info in both slice fields.
  */
 #ifndef DARTMOQ_HIP_H
 #define DARTMOQ_HIP_H
@@ -43,6 +46,7 @@ enum { DMQ_MODE_A16 = 0, DMQ_MODE_A8 = 1, DMQ_MODE_FP8 = 2, DMQ_MODE_FP4 = 3 };
  * the k slots of each token in slot order. */
 enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
+#define DMQ_ITEM_WORDS 8
 
 /* Library / build identification: returns the ABI version (currently 3). */
 int dmq_abi_version(void);
@@ -95,7 +99,7 @@ int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts,
  * Outputs (device, int32 unless noted):
  *   counts [experts], offsets [experts+1], sorted_tokens [tokens*k],
  *   sorted_weights fp32 [tokens*k], sorted_rows [tokens*k] (token*k + slot of each sorted row),
- *   gu_info / dn_info [pools, experts, 4], n_items [1], items [max_items, 4] (all pools,
+ *   gu_info / dn_info [pools, experts, 4], n_items [1], items [max_items, DMQ_ITEM_WORDS] (all pools,
  *   pool-major, experts ascending).
  * scratch: device memory of at least dmq_route_scratch_bytes(tokens, k, experts) bytes
  * (per-chunk expert histograms of the counting sort).  experts <= 2048. */

@@ -132,7 +132,7 @@ int dmq_rotate(int mode, const void* x, long x_stride, const void* row_index, co
                int scale_fp32, float extra_scale, int tt, void* stream) {
   if (rows <= 0) return DMQ_OK;
   if (!valid_mode(mode)) return DMQ_ERR_MODE;
-  if (tt != 1 && tt != 4) return DMQ_ERR_MODE;
+  if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
   if (row_index) return DMQ_ERR_MODE;    // gathered rows go through dmq_rotate_tiled
   if (!x || !rot || !out) return DMQ_ERR_NULL;
   if (mode != DMQ_MODE_A16 && !scale) return DMQ_ERR_NULL;
@@ -157,7 +157,7 @@ int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_ind
   if (!expert_info || !items || !n_items) return DMQ_ERR_NULL;
   if (max_items <= 0) return DMQ_OK;
   if (!valid_mode(mode)) return DMQ_ERR_MODE;
-  if (tt != 1 && tt != 4) return DMQ_ERR_MODE;
+  if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
   if (tile_rows <= 0 || tile_rows % (16 * tt)) return DMQ_ERR_ALIGN;
   if (!x || !rot || !out) return DMQ_ERR_NULL;
   if (mode != DMQ_MODE_A16 && !scale) return DMQ_ERR_NULL;
@@ -230,7 +230,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
   p.out = (__half*)a->out;
   p.out_stride = a->out_stride;
-  p.out_slots = (float*)a->out;
+  p.out_slots = (__half*)a->out;
   p.row_weight = (const float*)a->row_weight;
   p.row_slot = (const int*)a->row_slot;
   p.dbg_acc = (int*)a->dbg_acc;
@@ -251,12 +251,12 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   return DMQ_ERR_MODE;
 }
 
-int dmq_combine_slots(const void* slots_f32, int k, const void* add_f16, long tokens, int hidden,
+int dmq_combine_slots(const void* slots_f16, int k, const void* add_f16, long tokens, int hidden,
                       void* out_f16, void* stream) {
-  if (!slots_f32 || !out_f16) return DMQ_ERR_NULL;
+  if (!slots_f16 || !out_f16) return DMQ_ERR_NULL;
   if (k <= 0 || hidden <= 0) return DMQ_ERR_SHAPE;
-  if (hidden % 4) return DMQ_ERR_ALIGN;
-  return dmq_combine_launch((const float*)slots_f32, k, (const __half*)add_f16, tokens, hidden,
+  if (hidden % 8) return DMQ_ERR_ALIGN;
+  return dmq_combine_launch((const __half*)slots_f16, k, (const __half*)add_f16, tokens, hidden,
                             (__half*)out_f16, (hipStream_t)stream);
 }
 
@@ -282,7 +282,8 @@ int dmq_fill_zero(void* ptr, long n_bytes, void* stream) {
 // ------------------------------------------------------------------------------- whole layer
 struct MoeWorkspace {
   int *counts, *offsets, *sorted_tokens, *sorted_rows, *gu_info, *dn_info, *n_items, *items;
-  float *sorted_weights, *slots;
+  float* sorted_weights;
+  uint8_t* slots;                    // fp16 [tokens * top_k, hidden]
   uint8_t* xq[DMQ_MAX_POOLS];        // hoisted pools: codes by token; others share xq_rows
   uint8_t* xq_scale[DMQ_MAX_POOLS];
   uint8_t *xq_rows, *xq_rows_scale, *act, *actq, *actq_scale;
@@ -296,7 +297,7 @@ static inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static int pick_tt(int tokens, int top_k, int experts) {
   const long avg = (long)tokens * top_k / (experts > 0 ? experts : 1);
-  return avg <= 8 ? 1 : (avg <= 48 ? 2 : 4);
+  return avg <= 8 ? 1 : 2;      // 64-row tiles run one workgroup per CU and measured slower
 }
 
 static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* base) {
@@ -317,8 +318,8 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.n_items = (int*)take(16);
   w.sort_scratch_bytes = dmq_route_scratch_bytes(tokens, L->top_k, L->experts);
   w.sort_scratch = take(w.sort_scratch_bytes);
-  w.items = (int*)take((size_t)w.max_items * 16);
-  w.slots = (float*)take(R * H * 4);
+  w.items = (int*)take((size_t)w.max_items * DMQ_ITEM_WORDS * sizeof(int));
+  w.slots = take(R * H * 2);
   for (size_t i = 0; i < DMQ_MAX_POOLS; ++i) {
     // every pool gets a by-token buffer so the size does not depend on which pools are hoisted
     w.xq[i] = i < P ? take((size_t)tokens * H * 2) : nullptr;
@@ -364,7 +365,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
   if (ks <= 0) ks = pick_ks(tt, (long)tokens * K);
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
-  const int rot_tt = (tt == 4) ? 4 : 1;
+  const int rot_tt = tt;               // a rotation wave covers one row tile of the work items
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
   if (w.bytes > workspace_bytes) return DMQ_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;

@@ -29,6 +29,7 @@
 //           16-byte chunks XOR-swizzled by row so the operand reads spread over the banks).
 #pragma once
 #include "common.h"
+#include <type_traits>
 #include "lut.h"
 
 #ifdef DMQ_TRACE
@@ -63,13 +64,13 @@ struct GemmParams {
   int half_width;              // SiLU epilogue: I (gate rows [0,I), up rows [I,2I) of the slice)
   int slice_is_groups;         // 0: slice_start offsets weight rows; 1: offsets groups (down)
   // work list
-  const int* items;            // [*, 4] pool, expert index, token tile inside the expert, unused
+  const int* items;            // [max_items, DMQ_ITEM_WORDS] work-item records, meaningful below n_items
   const int* n_items;          // device scalar
   int n_blocks;                // workgroups along the output features
   // outputs
   __half* out;                 // STORE / SILU: fp16 [rows, out_stride]
   long out_stride;
-  float* out_slots;            // SCATTER: fp32 [slots, out_stride] addressed by row_slot[r]
+  __half* out_slots;           // SCATTER: fp16 [slots, out_stride] addressed by row_slot[r]
   const float* row_weight;     // SCATTER: routing weight of logical row r
   const int* row_slot;         // SCATTER: destination row (token * top_k + slot) of logical row r
   int* dbg_acc;                // optional int32 [rows, groups, n_out] per-group accumulators (A8)
@@ -102,35 +103,42 @@ template <int N> __device__ __forceinline__ void dmq_load_words(const uint8_t* p
   }
 }
 
-// Expand the packed bytes of MFMA step `s` into the lane's operand words.
-template <int MODE, int BIT>
+// Expand the packed bytes of MFMA step S into the lane's operand words.
+template <int MODE, int BIT, int S>
 __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t lane_base,
-                                                 const uint32_t* pk, int s, uint32_t* w) {
+                                                 const uint32_t* pk, uint32_t* w) {
   using T = ModeTraits<MODE>;
   using G = LutGeom<BIT, T::ES>;
   constexpr int BYTES = (4 * BIT) / T::STEPS;           // packed bytes per step
-#pragma unroll
-  for (int b = 0; b < BYTES; ++b) {
-    const int bi = s * BYTES + b;
-    const uint32_t byte = (pk[bi >> 2] >> ((bi & 3) * 8)) & 0xffu;
-    if (G::EB >= 4) {
-      dmq_lut_read<BIT, T::ES>(tbl, lane_base, byte, w + b * (G::EB / 4));
+  auto one = [&](auto bc) {
+    constexpr int b = decltype(bc)::value;
+    constexpr int bi = S * BYTES + b;
+    if constexpr (G::EB >= 4) {
+      dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], w + b * (G::EB / 4));
     } else {                                            // two one-byte elements per look-up
       uint32_t v;
-      dmq_lut_read<BIT, T::ES>(tbl, lane_base, byte, &v);
+      dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], &v);
       if (b & 1) w[b >> 1] |= v << 16; else w[b >> 1] = v;
     }
+  };
+  one(std::integral_constant<int, 0>{});
+  if constexpr (BYTES > 1) one(std::integral_constant<int, 1>{});
+  if constexpr (BYTES > 2) { one(std::integral_constant<int, 2>{}); one(std::integral_constant<int, 3>{}); }
+  if constexpr (BYTES > 4) {
+    one(std::integral_constant<int, 4>{}); one(std::integral_constant<int, 5>{});
+    one(std::integral_constant<int, 6>{}); one(std::integral_constant<int, 7>{});
   }
+  static_assert(BYTES <= 8, "at most eight packed bytes per MFMA step");
 }
 
 // Groups in flight per wave on the staged path.  WW registers hold one (group, n-tile) of packed
-// weights; few activation rows leave registers for a deep ring, which is what hides the HBM
-// latency when a workgroup has little arithmetic per group.
+// weights.  Rings of 8 words (16-row tiles) and 4 words (32-row tiles) keep three resp. two
+// workgroups resident per CU; deeper rings cost a workgroup of occupancy and measured slower.
 #ifndef DMQ_RING_TT1
-#define DMQ_RING_TT1 16
+#define DMQ_RING_TT1 8
 #endif
 #ifndef DMQ_RING_TT2
-#define DMQ_RING_TT2 8
+#define DMQ_RING_TT2 4
 #endif
 #ifndef DMQ_RING_TT4
 #define DMQ_RING_TT4 4
@@ -157,7 +165,8 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
 
 template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
-                                              uint8_t* smem2, int eidx, int ttile, int nb) {
+                                              uint8_t* smem2, int token_start, int token_count,
+                                              int slice_start, int ttile, int nb) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   using GG = GemmGeom<MODE, NT, TT, KS>;
@@ -180,10 +189,6 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   const int kpart = wave % KS;
   const int rowpart = wave / KS;
   const uint32_t lane_base = (MODE == DMQ_MODE_FP4) ? 0u : dmq_lut_lane_base<BIT, T::ES>(lane);
-
-  const int token_start = pw.expert_info[4 * eidx + 0];
-  const int token_count = pw.expert_info[4 * eidx + 1];
-  const int slice_start = pw.expert_info[4 * eidx + 2];
 
   const int feat0 = (nb * ROWPARTS + rowpart) * (FEAT_TILES * 16);   // first output feature of the wave
   const bool wave_active = feat0 < p.n_out;                          // wave-uniform
@@ -262,8 +267,12 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr int WQ = (MODE == DMQ_MODE_FP4) ? 1 : T::STEPS * OPW;
   auto dequant_tile = [&](const uint32_t (&pkj)[WW], uint32_t (&w)[WQ]) {
     if constexpr (MODE != DMQ_MODE_FP4) {
-#pragma unroll
-      for (int s = 0; s < T::STEPS; ++s) dmq_dequant_step<MODE, BIT>(tbl, lane_base, pkj, s, w + s * OPW);
+      dmq_dequant_step<MODE, BIT, 0>(tbl, lane_base, pkj, w);
+      if constexpr (T::STEPS > 1) dmq_dequant_step<MODE, BIT, 1>(tbl, lane_base, pkj, w + OPW);
+      if constexpr (T::STEPS > 2) {
+        dmq_dequant_step<MODE, BIT, 2>(tbl, lane_base, pkj, w + 2 * OPW);
+        dmq_dequant_step<MODE, BIT, 3>(tbl, lane_base, pkj, w + 3 * OPW);
+      }
     }
   };
   auto compute = [&](int g, const uint32_t (&pk)[NT][WW], const uint2_t (&nr)[NT],
@@ -382,32 +391,48 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     const bool s_active = srow < 16 * TT;
     const bool s_valid = s_active && s_rlog < r_end;
     const int s_phys = s_valid ? (pw.row_index ? pw.row_index[s_rlog] : s_rlog) : 0;
-    const uint8_t* s_src = pw.act + (long)s_phys * p.act_row_bytes + sc0 * 16;
+    const uint32_t s_off = (uint32_t)s_phys * (uint32_t)p.act_row_bytes + sc0 * 16;
     // lane (l16, q) stages the norm of row l16 of its wave's n-tile q
     const bool n_active = q < NT;
-    const int n_row = (EPI == DMQ_EPI_SILU)
+    const uint32_t n_off = 2u * (uint32_t)((EPI == DMQ_EPI_SILU)
         ? slice_start + ((q & 1) ? p.half_width : 0) + featw + (q >> 1) * 16 + l16
-        : (p.slice_is_groups ? 0 : slice_start) + featw + q * 16 + l16;
+        : (p.slice_is_groups ? 0 : slice_start) + featw + q * 16 + l16);
     // thread t < 16*TT stages the scale word of tile row t
     const int c_rlog = r_first + (int)threadIdx.x;
     const bool c_active = SCALED && threadIdx.x < 16 * TT;
     const bool c_valid = c_active && c_rlog < r_end;
     const int c_phys = c_valid ? (pw.row_index ? pw.row_index[c_rlog] : c_rlog) : 0;
+    const uint32_t c_off = (uint32_t)c_phys * (uint32_t)p.act_scale_stride * (MODE == DMQ_MODE_FP4 ? 1u : 2u);
+    uint32_t w_off[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) w_off[j] = (uint32_t)(wrow[j] + l16) * PPG + q * (WW * 4);
     uint8_t* stage = smem2;
 
     struct Staged { uint4_t a[CPT]; uint32_t nrm; uint32_t sc; };
+    // every address is a workgroup-uniform base (scalar registers) plus a 32-bit lane offset
+    // fixed for the item; the empty asm keeps the zero-extension of the offset next to the
+    // load, which is the form the scalar-base addressing mode of global loads needs
+    const uint8_t* const act_p = pw.act;
+    const uint8_t* const norms_p = (const uint8_t*)pw.norms;
+    const uint8_t* const scale_p = (const uint8_t*)pw.act_scale;
+    const uint8_t* const w_p = pw.w;
+    const long group_rows = pw.n_total;
+    auto lane_off = [](uint32_t o) { asm volatile("" : "+v"(o)); return o; };
     auto stage_load = [&](int g, Staged& sr) {
+      const uint8_t* abase = act_p + (long)g * AB;
 #pragma unroll
       for (int c = 0; c < CPT; ++c)
-        sr.a[c] = s_valid ? *(const uint4_t*)(s_src + (long)g * AB + c * 16) : (uint4_t){0u, 0u, 0u, 0u};
-      sr.nrm = n_active ? *(const uint16_t*)(pw.norms + (long)(g_base + g) * pw.n_total + n_row) : 0u;
+        sr.a[c] = s_valid ? *(const uint4_t*)(abase + lane_off(s_off) + c * 16) : (uint4_t){0u, 0u, 0u, 0u};
+      const uint8_t* nbase = norms_p + (long)(g_base + g) * group_rows * 2;
+      sr.nrm = n_active ? *(const uint16_t*)(nbase + lane_off(n_off)) : 0u;
       sr.sc = 0u;
       if constexpr (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
-        if (c_valid) sr.sc = ((const uint16_t*)pw.act_scale)[(long)c_phys * p.act_scale_stride + g];
+        const uint8_t* sbase = scale_p + (long)g * 2;
+        if (c_valid) sr.sc = *(const uint16_t*)(sbase + lane_off(c_off));
       } else if constexpr (MODE == DMQ_MODE_FP4) {
+        const uint8_t* sbase = scale_p + (long)g * 4;
         sr.sc = 0x7f7f7f7fu;
-        if (c_valid)
-          sr.sc = *(const uint32_t*)((const uint8_t*)pw.act_scale + (long)c_phys * p.act_scale_stride + g * 4);
+        if (c_valid) sr.sc = *(const uint32_t*)(sbase + lane_off(c_off));
       }
     };
     auto stage_store = [&](int buf, const Staged& sr) {
@@ -446,10 +471,9 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         nr[j] = *(const uint2_t*)(slot + NORM_OFF + ((wave * NT + j) * 16 + 4 * q) * 2);
     };
     auto load_packed = [&](int g, uint32_t (&pk)[NT][WW]) {
-      const long gg = (long)(g_base + g) * pw.n_total;
+      const uint8_t* wbase = w_p + (long)(g_base + g) * group_rows * PPG;
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        dmq_load_words<WW>(pw.w + (gg + wrow[j] + l16) * PPG + q * (WW * 4), pk[j]);
+      for (int j = 0; j < NT; ++j) dmq_load_words<WW>(wbase + lane_off(w_off[j]), pk[j]);
     };
 
     // Every load below is unconditional (group indices past the end are clamped to the last
@@ -461,6 +485,10 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     uint32_t pkb[D][NT][WW];
     Staged srb[D];
     const int g_last = g_hi - 1;
+    // the codebook entries of this thread's table row are requested first: they arrive while
+    // the weights are still in flight and the table is ready one memory latency after launch
+    uint32_t lutw[4];
+    if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_fetch<BIT, T::ES>(pw.lut, threadIdx.x, lutw);
 #pragma unroll
     for (int u = 0; u < D; ++u) {
       const int gl = (g_lo + u < g_last) ? g_lo + u : g_last;
@@ -468,7 +496,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       load_packed(gl, pkb[u]);
     }
     DMQ_MARK(1);
-    if (MODE != DMQ_MODE_FP4) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
+    if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_store_wave<BIT, T::ES>(tbl, wave, lutw);
     DMQ_MARK(2);
     stage_store(0, srb[0]);
     __syncthreads();
@@ -548,8 +576,9 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + (j >> 1) * 16 + 4 * q) = h;
       } else {
         const float rw = p.row_weight[rlog[t]];
-        float4_t v = total_acc[j][t] * rw;
-        *(float4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat0 + j * 16 + 4 * q) = v;
+        const float4_t v = total_acc[j][t] * rw;
+        const half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+        *(half4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat0 + j * 16 + 4 * q) = h;
       }
     }
   }
@@ -565,20 +594,26 @@ void dmq_gemm_gf_kernel(GemmParams p) {
 
   DMQ_MARK(0);
   const int item = blockIdx.x / p.n_blocks;
-  if (item >= p.n_items[0]) return;
   const int nb = blockIdx.x - item * p.n_blocks;
-  const int pool = p.items[4 * item + 0];
-  const int eidx = p.items[4 * item + 1];
-  const int ttile = p.items[4 * item + 2];
+  // the record is fetched together with the item count; it is only trusted below the count
+  const int4_t* rec = (const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * item);
+  const int4_t r0 = rec[0];
+  const int4_t r1 = rec[1];
+  if (item >= p.n_items[0]) return;
+  const int pool = r0[0];
+  const int ttile = r0[2];
+  const int token_start = r0[3];
+  const int token_count = r1[0];
+  const int slice_start = p.slice_is_groups ? r1[2] : r1[1];
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE) return;
   if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb);
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb);
   } else {
     switch (pw.bit) {
-      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb); break;
-      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb); break;
-      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, eidx, ttile, nb); break;
+      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb); break;
+      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb); break;
+      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb); break;
     }
   }
 }

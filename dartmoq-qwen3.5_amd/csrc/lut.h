@@ -3,48 +3,82 @@
 // A packed weight byte carries 8/BIT codebook indices.  The table maps a byte
 // value straight to its 8/BIT dequantized elements (fp16 for WxA16, one byte
 // each for the int8 / e4m3 look-ups), so dequantizing costs one LDS read per
-// packed byte.  Every entry is replicated across a 128-byte row; lane L reads
-// the copy at (L % copies) so that the lanes of a wave hit distinct LDS banks
-// whatever byte values they look up.  The table always occupies 32 KiB.
+// packed byte.  Every entry is replicated across a row of DMQ_LUT_ROW bytes; lane L
+// reads the copy at (L % copies) so that the lanes of a wave hit distinct LDS banks
+// whatever byte values they look up.  128-byte rows (a 32 KiB table) measured faster than
+// 256-byte rows on MI355X: three workgroups fit a CU instead of two, which outweighs the
+// cheaper address arithmetic ((byte << 8) | lane offset is one byte permute) of wide rows.
 #pragma once
 #include "common.h"
 
-#define DMQ_LUT_BYTES (256 * 128)
+#ifndef DMQ_LUT_ROW
+#define DMQ_LUT_ROW 128
+#endif
+#define DMQ_LUT_BYTES (256 * DMQ_LUT_ROW)
 
 template <int BIT, int ES>   // ES = bytes per dequantized element (2: fp16, 1: int8 / e4m3)
 struct LutGeom {
   static constexpr int ELEMS = 8 / BIT;                 // elements per packed byte
   static constexpr int EB = ELEMS * ES;                 // payload bytes per entry
   static constexpr int STRIDE = EB < 4 ? 4 : EB;        // bytes between copies
-  static constexpr int COPIES = 128 / STRIDE;
+  static constexpr int COPIES = DMQ_LUT_ROW / STRIDE;
 };
 
-// Build the table with the whole workgroup (blockDim.x threads); caller syncs afterwards.
+// Entry `e` of the table: the codebook values of the 8/BIT indices packed in byte value e.
 template <int BIT, int ES>
-__device__ __forceinline__ void dmq_lut_build(uint8_t* tbl, const void* codebook) {
+__device__ __forceinline__ void dmq_lut_fetch(const void* codebook, int e, uint32_t (&w)[4]) {
   using G = LutGeom<BIT, ES>;
   constexpr uint32_t mask = (1u << BIT) - 1u;
-  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
-    uint32_t w[4] = {0u, 0u, 0u, 0u};
+  w[0] = w[1] = w[2] = w[3] = 0u;
 #pragma unroll
-    for (int j = 0; j < G::ELEMS; ++j) {
-      uint32_t idx = ((uint32_t)e >> (j * BIT)) & mask;
-      if (ES == 2) {
-        uint32_t v = ((const uint16_t*)codebook)[idx];
-        w[j >> 1] |= v << ((j & 1) * 16);
-      } else {
-        uint32_t v = ((const uint8_t*)codebook)[idx];
-        w[j >> 2] |= v << ((j & 3) * 8);
-      }
-    }
-    uint8_t* row = tbl + e * 128;
-#pragma unroll
-    for (int c = 0; c < G::COPIES; ++c) {
-      uint32_t* dst = (uint32_t*)(row + c * G::STRIDE);
-#pragma unroll
-      for (int i = 0; i < (G::STRIDE / 4); ++i) dst[i] = w[i];
+  for (int j = 0; j < G::ELEMS; ++j) {
+    uint32_t idx = ((uint32_t)e >> (j * BIT)) & mask;
+    if (ES == 2) {
+      uint32_t v = ((const uint16_t*)codebook)[idx];
+      w[j >> 1] |= v << ((j & 1) * 16);
+    } else {
+      uint32_t v = ((const uint8_t*)codebook)[idx];
+      w[j >> 2] |= v << ((j & 3) * 8);
     }
   }
+}
+
+// Write the 64 entries a wave fetched (lane i holds entry 64*wave + i) with all their copies.
+// Each store covers 256 contiguous bytes, one dword per lane, so it touches every LDS bank once;
+// the entry words are broadcast from the lane that fetched them.
+template <int BIT, int ES>
+__device__ __forceinline__ void dmq_lut_store_wave(uint8_t* tbl, int wave, const uint32_t (&w)[4]) {
+  using G = LutGeom<BIT, ES>;
+  constexpr int DW = G::STRIDE / 4;                     // dwords per copy
+  constexpr int RPW = 256 / DMQ_LUT_ROW;                // table rows per 256-byte store
+  const int lane = threadIdx.x & 63;
+  const int d = lane % DW;
+  uint32_t* dst = (uint32_t*)(tbl + (long)wave * 64 * DMQ_LUT_ROW) + lane;
+#pragma unroll
+  for (int t = 0; t < 64 / RPW; ++t) {
+    uint32_t v = 0u;
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      const int i = t * RPW + r;                        // entry of this wave, compile-time
+      uint32_t e = __builtin_amdgcn_readlane(w[0], i);
+      if (DW > 1) { const uint32_t e1 = __builtin_amdgcn_readlane(w[1], i); e = (d == 1) ? e1 : e; }
+      if (DW > 2) {
+        const uint32_t e2 = __builtin_amdgcn_readlane(w[2], i);
+        const uint32_t e3 = __builtin_amdgcn_readlane(w[3], i);
+        e = (d == 2) ? e2 : ((d == 3) ? e3 : e);
+      }
+      v = (RPW == 1 || (lane * 4) / DMQ_LUT_ROW == r) ? e : v;
+    }
+    dst[t * 64] = v;
+  }
+}
+
+// Build the table with a workgroup of 256 threads; caller syncs afterwards.
+template <int BIT, int ES>
+__device__ __forceinline__ void dmq_lut_build(uint8_t* tbl, const void* codebook) {
+  uint32_t w[4];
+  dmq_lut_fetch<BIT, ES>(codebook, threadIdx.x, w);
+  dmq_lut_store_wave<BIT, ES>(tbl, threadIdx.x >> 6, w);
 }
 
 template <int BIT, int ES>
@@ -53,12 +87,19 @@ __device__ __forceinline__ uint32_t dmq_lut_lane_base(int lane) {
   return (uint32_t)(lane % G::COPIES) * G::STRIDE;
 }
 
-// Look one packed byte up.  out receives EB bytes (rounded up to whole words).
-template <int BIT, int ES>
-__device__ __forceinline__ void dmq_lut_read(const uint8_t* tbl, uint32_t lane_base,
-                                             uint32_t byte, uint32_t* out) {
+// Look up byte K (0..3) of a packed word.  out receives EB bytes (rounded up to whole words).
+template <int BIT, int ES, int K>
+__device__ __forceinline__ void dmq_lut_read_word(const uint8_t* tbl, uint32_t lane_base,
+                                                  uint32_t word, uint32_t* out) {
   using G = LutGeom<BIT, ES>;
-  const uint8_t* p = tbl + (byte << 7) + lane_base;
+  uint32_t off;
+  if (DMQ_LUT_ROW == 256) {
+    // result bytes: [0] lane offset, [1] byte K of the word, [2] = [3] = 0
+    off = __builtin_amdgcn_perm(word, lane_base, 0x0c0c0400u + ((uint32_t)K << 8));
+  } else {
+    off = (((word >> (8 * K)) & 0xffu) * DMQ_LUT_ROW) + lane_base;
+  }
+  const uint8_t* p = tbl + off;
   if (G::EB == 2) {
     out[0] = *(const uint16_t*)p;
   } else if (G::EB == 4) {
@@ -70,4 +111,11 @@ __device__ __forceinline__ void dmq_lut_read(const uint8_t* tbl, uint32_t lane_b
     uint4_t v = *(const uint4_t*)p;
     out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
   }
+}
+
+// Look one packed byte value up.
+template <int BIT, int ES>
+__device__ __forceinline__ void dmq_lut_read(const uint8_t* tbl, uint32_t lane_base,
+                                             uint32_t byte, uint32_t* out) {
+  dmq_lut_read_word<BIT, ES, 0>(tbl, lane_base, byte & 0xffu, out);
 }

@@ -28,7 +28,7 @@ struct RotParams {
   int n_hoisted;
   int hoisted_pool[DMQ_MAX_POOLS];
   int hoisted_items_per_pool;   // ceil(rows / (16*TT)) * groups
-  const int* items;        // [*, 4] pool, expert, row tile, unused
+  const int* items;        // [*, DMQ_ITEM_WORDS] work-item records
   const int* n_items;
   int tile_rows;           // rows per work item (multiple of 16*TT)
   int scale_fp32;
@@ -74,7 +74,7 @@ struct PlanParams {
   int* gu_info;                  // [pools, experts, 4]
   int* dn_info;                  // [pools, experts, 4]  slice in groups: start/128, I/128
   int* n_items;                  // [1]
-  int* items;                    // [max_items, 4]
+  int* items;                    // [max_items, DMQ_ITEM_WORDS]
 };
 
 int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream);
@@ -86,7 +86,7 @@ int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int token
                              float* sorted_weights, int* sorted_rows, hipStream_t stream);
 int dmq_items_from_info_launch(const int* expert_info, int experts, int tile_rows, int max_items,
                                int pool, int* n_items, int* items, hipStream_t stream);
-int dmq_combine_launch(const float* slots, int k, const __half* add, long tokens, int hidden,
+int dmq_combine_launch(const __half* slots, int k, const __half* add, long tokens, int hidden,
                        __half* out, hipStream_t stream);
 int dmq_unpack_launch(const uint8_t* packed, long n_bytes, int bit, uint8_t* out, hipStream_t s);
 int dmq_dequant_tile_launch(const uint8_t* idx_gf, const __half* cb, const __half* norms, int n_total,

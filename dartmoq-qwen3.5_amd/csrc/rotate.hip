@@ -54,16 +54,15 @@ void dmq_rotate_kernel(RotParams p) {
     const int sub = p.tile_rows / ROWS_PER_ITEM;          // waves per work item
     const long tile = rt / sub;
     if (tile >= p.n_items[0]) return;
-    pool = p.items[4 * tile];
+    const int* it = p.items + DMQ_ITEM_WORDS * tile;
+    pool = it[0];
     if (p.pool[pool].hoisted) return;
-    const int eidx = p.items[4 * tile + 1];
-    const int ttile = p.items[4 * tile + 2];
-    const int* info = p.pool[pool].expert_info;
-    const int ts = info[4 * eidx + 0];
-    const int tc = info[4 * eidx + 1];
+    const int ttile = it[2];
+    const int ts = it[3];
+    const int tc = it[4];
     r_first = ts + ttile * p.tile_rows + (int)(rt % sub) * ROWS_PER_ITEM;
     r_end = ts + tc;
-    rot_g = (p.pool[pool].rot_use_slice ? info[4 * eidx + 2] : 0) + g;
+    rot_g = (p.pool[pool].rot_use_slice ? it[6] : 0) + g;
     row_index = p.row_index;
   }
   const RotPool& rp = p.pool[pool];
@@ -250,6 +249,7 @@ static int launch_rotate(const RotParams& p, long items, int tt, hipStream_t str
   const int grid = (int)((items + 3) / 4);
   if (grid <= 0) return DMQ_OK;
   if (tt == 4) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 4>), dim3(grid), dim3(256), 0, stream, p);
+  else if (tt == 2) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 2>), dim3(grid), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 1>), dim3(grid), dim3(256), 0, stream, p);
   return dmq_check_launch();
 }

@@ -121,16 +121,44 @@ __global__ __launch_bounds__(1024)
 void dmq_plan_kernel(PlanParams p) {
   __shared__ int wave_tot[16];
   __shared__ int carry;
+  __shared__ int partial[1024];
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
+  // The chunk axis of the histogram is split over `parts` threads per expert so that all 1024
+  // threads load; a thread keeps at most 16 loads in flight.
+  int epad = 64;
+  while (epad < p.experts && epad < 1024) epad <<= 1;
+  const int parts = 1024 / epad;
+  const int part = tid / epad;
+  const int el = tid % epad;
+  const int cpp = (p.n_chunks + parts - 1) / parts;
+  const int c_lo = part * cpp;
+  const int c_hi = min(p.n_chunks, c_lo + cpp);
+  auto chunk_sum = [&](int e) {
+    int sum = 0;
+    if (e < p.experts) {
+      for (int c0 = c_lo; c0 < c_hi; c0 += 16) {
+        int h[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) h[i] = (c0 + i < c_hi) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += h[i];
+      }
+    }
+    return sum;
+  };
   // rows per expert: column sums of the chunk histogram
-  for (int e = tid; e < p.experts; e += 1024) {
-    int total = 0;
-#pragma unroll 8
-    for (int c = 0; c < p.n_chunks; ++c) total += p.hist[(long)c * p.experts + e];
-    p.counts[e] = total;
+  for (int ebase = 0; ebase < p.experts; ebase += epad) {
+    const int e = ebase + el;
+    partial[tid] = chunk_sum(e);
+    __syncthreads();
+    if (part == 0 && e < p.experts) {
+      int total = 0;
+      for (int q = 0; q < parts; ++q) total += partial[q * epad + el];
+      p.counts[e] = total;
+    }
+    __syncthreads();
   }
-  __syncthreads();
   // expert offsets: exclusive scan of counts, 1024 experts per pass
   for (int base = 0; base < p.experts; base += 1024) {
     const int e = base + tid;
@@ -144,18 +172,25 @@ void dmq_plan_kernel(PlanParams p) {
   if (tid == 0) p.offsets[0] = 0;
   __syncthreads();
   // hist[c, e] <- position of the first row of chunk c routed to expert e
-  for (int e = tid; e < p.experts; e += 1024) {
-    int at = p.offsets[e + 1] - p.counts[e];
-    for (int c0 = 0; c0 < p.n_chunks; c0 += 8) {
-      int h[8];
+  for (int ebase = 0; ebase < p.experts; ebase += epad) {
+    const int e = ebase + el;
+    partial[tid] = chunk_sum(e);
+    __syncthreads();
+    if (e < p.experts) {
+      int at = p.offsets[e + 1] - p.counts[e];
+      for (int q = 0; q < part; ++q) at += partial[q * epad + el];
+      for (int c0 = c_lo; c0 < c_hi; c0 += 16) {
+        int h[16];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) h[i] = (c0 + i < p.n_chunks) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
+        for (int i = 0; i < 16; ++i) h[i] = (c0 + i < c_hi) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if (c0 + i < p.n_chunks) p.hist[(long)(c0 + i) * p.experts + e] = at;
-        at += h[i];
+        for (int i = 0; i < 16; ++i) {
+          if (c0 + i < c_hi) p.hist[(long)(c0 + i) * p.experts + e] = at;
+          at += h[i];
+        }
       }
     }
+    __syncthreads();
   }
 
   // per-pool expert_info and the work-item list, pools in caller order, experts ascending
@@ -164,24 +199,27 @@ void dmq_plan_kernel(PlanParams p) {
   for (int pool = 0; pool < p.pools; ++pool) {
     for (int base = 0; base < p.experts; base += 1024) {
       const int e = base + tid;
-      int ntile = 0;
+      int ntile = 0, ts = 0, tc = 0, gu_ss = 0, dn_ss = 0;
       if (e < p.experts) {
         const int ss = p.slice_start_rows[pool * p.experts + e];
         const int sc = p.slice_count_rows[pool * p.experts + e];
-        const int tc = (ss >= 0) ? p.counts[e] : 0;
-        const int ts = p.offsets[e + 1] - p.counts[e];
+        tc = (ss >= 0) ? p.counts[e] : 0;
+        ts = p.offsets[e + 1] - p.counts[e];
+        gu_ss = ss >= 0 ? ss : 0;
+        dn_ss = ss >= 0 ? ss / (2 * DMQ_GS) : 0;
         ntile = (tc + p.tile_rows - 1) / p.tile_rows;
         int* gi = p.gu_info + ((long)pool * p.experts + e) * 4;
-        gi[0] = ts; gi[1] = tc; gi[2] = ss >= 0 ? ss : 0; gi[3] = sc;
+        gi[0] = ts; gi[1] = tc; gi[2] = gu_ss; gi[3] = sc;
         int* di = p.dn_info + ((long)pool * p.experts + e) * 4;
-        di[0] = ts; di[1] = tc; di[2] = ss >= 0 ? ss / (2 * DMQ_GS) : 0; di[3] = sc / (2 * DMQ_GS);
+        di[0] = ts; di[1] = tc; di[2] = dn_ss; di[3] = sc / (2 * DMQ_GS);
       }
       const int incl = block_scan_incl(ntile, wave_tot);
       const int first = incl - ntile + carry;
       for (int i = 0; i < ntile; ++i) {
         if (first + i < p.max_items) {
-          int* it = p.items + 4L * (first + i);
-          it[0] = pool; it[1] = e; it[2] = i; it[3] = 0;
+          int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * (first + i));
+          it[0] = (int4_t){pool, e, i, ts};
+          it[1] = (int4_t){tc, gu_ss, dn_ss, 0};
         }
       }
       __syncthreads();
@@ -241,9 +279,11 @@ void dmq_items_from_info_kernel(const int* expert_info, int experts, int tile_ro
   __syncthreads();
   for (int base = 0; base < experts; base += 1024) {
     const int e = base + tid;
-    int ntile = 0;
+    int ntile = 0, ts = 0, tc = 0, ss = 0;
     if (e < experts) {
-      const int tc = expert_info[4 * e + 1];
+      ts = expert_info[4 * e + 0];
+      tc = expert_info[4 * e + 1];
+      ss = expert_info[4 * e + 2];
       const int sc = expert_info[4 * e + 3];
       ntile = (tc > 0 && sc > 0) ? (tc + tile_rows - 1) / tile_rows : 0;
     }
@@ -251,8 +291,9 @@ void dmq_items_from_info_kernel(const int* expert_info, int experts, int tile_ro
     const int first = incl - ntile + carry;
     for (int i = 0; i < ntile; ++i)
       if (first + i < max_items) {
-        int* it = items + 4L * (first + i);
-        it[0] = pool; it[1] = e; it[2] = i; it[3] = 0;
+        int4_t* it = (int4_t*)(items + (long)DMQ_ITEM_WORDS * (first + i));
+        it[0] = (int4_t){pool, e, i, ts};
+        it[1] = (int4_t){tc, ss, ss, 0};
       }
     __syncthreads();
     if (tid == 1023) carry = incl + carry;
@@ -261,24 +302,32 @@ void dmq_items_from_info_kernel(const int* expert_info, int experts, int tile_ro
   if (tid == 0) n_items[0] = min(carry, max_items);
 }
 
-// out[t, h] = fp16( sum_{j<k} slots[t*k + j, h]  (+ add[t, h]) ), slots summed in slot order
+// out[t, h] = fp16( sum_{j<k} slots[t*k + j, h]  (+ add[t, h]) ): fp16 slots summed in fp32 in
+// slot order (the reference accumulates the same fp16 expert rows with index_add_ in fp16)
 __global__ __launch_bounds__(256)
-void dmq_combine_kernel(const float* slots, int k, const __half* add, long tokens, int hidden,
+void dmq_combine_kernel(const __half* slots, int k, const __half* add, long tokens, int hidden,
                         __half* out) {
-  const int hv = hidden / 4;
+  const int hv = hidden / 8;
   const long total = tokens * hv;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (long)gridDim.x * blockDim.x) {
     const long t = i / hv;
-    const int h = (int)(i % hv) * 4;
-    float4_t s = {0.f, 0.f, 0.f, 0.f};
-    for (int j = 0; j < k; ++j) s += *(const float4_t*)(slots + (t * k + j) * hidden + h);
-    if (add) {
-      half4_t a = *(const half4_t*)(add + t * hidden + h);
-      s[0] += (float)a[0]; s[1] += (float)a[1]; s[2] += (float)a[2]; s[3] += (float)a[3];
+    const int h = (int)(i % hv) * 8;
+    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < k; ++j) {
+      const half8_t v = *(const half8_t*)(slots + (t * k + j) * hidden + h);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) s[c] += (float)v[c];
     }
-    half4_t o = {(_Float16)s[0], (_Float16)s[1], (_Float16)s[2], (_Float16)s[3]};
-    *(half4_t*)(out + t * hidden + h) = o;
+    if (add) {
+      const half8_t a = *(const half8_t*)(add + t * hidden + h);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) s[c] += (float)a[c];
+    }
+    half8_t o;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) o[c] = (_Float16)s[c];
+    *(half8_t*)(out + t * hidden + h) = o;
   }
 }
 
@@ -320,9 +369,9 @@ int dmq_items_from_info_launch(const int* expert_info, int experts, int tile_row
   return dmq_check_launch();
 }
 
-int dmq_combine_launch(const float* slots, int k, const __half* add, long tokens, int hidden,
+int dmq_combine_launch(const __half* slots, int k, const __half* add, long tokens, int hidden,
                        __half* out, hipStream_t stream) {
-  const long total = tokens * (hidden / 4);
+  const long total = tokens * (hidden / 8);
   if (total <= 0) return DMQ_OK;
   long g = (total + 255) / 256;
   if (g > 16384) g = 16384;

@@ -15,6 +15,7 @@ from ._lib import (EPI_SCATTER, EPI_SILU, EPI_STORE, MODE_A16, MODE_A8, MODE_FP4
                    check, load)
 
 GROUP_SIZE = 128
+ITEM_WORDS = 8          # int32 words of a work-item record (DMQ_ITEM_WORDS)
 
 
 def _ptr(t):
@@ -131,7 +132,7 @@ def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_
         "gu_info": torch.empty((pools, num_experts, 4), **i32),
         "dn_info": torch.empty((pools, num_experts, 4), **i32),
         "n_items": torch.zeros(4, **i32),
-        "items": torch.zeros((max_items, 4), **i32),
+        "items": torch.zeros((max_items, ITEM_WORDS), **i32),
         "max_items": max_items, "tile_rows": tile_rows,
     }
     scratch = torch.empty(max(1, load().dmq_route_scratch_bytes(t, k, num_experts)),
@@ -152,7 +153,7 @@ def build_tiles(expert_info: torch.Tensor, rows_total: int, tile_rows: int, pool
     n_exp = expert_info.shape[0]
     max_items = rows_total // tile_rows + n_exp
     n_items = torch.zeros(4, dtype=torch.int32, device=expert_info.device)
-    items = torch.zeros((max_items, 4), dtype=torch.int32, device=expert_info.device)
+    items = torch.zeros((max_items, ITEM_WORDS), dtype=torch.int32, device=expert_info.device)
     check(load().dmq_build_tiles(_ptr(expert_info), n_exp, tile_rows, max_items, pool, _ptr(n_items),
                                  _ptr(items), _stream(expert_info.device)), "build_tiles")
     return n_items, items, max_items
@@ -237,7 +238,7 @@ def quantize_act(mode: int, x_rot: torch.Tensor, extra_scale: float = 1.0, scale
 
 def pick_tt(rows_total: int, n_experts: int) -> int:
     avg = rows_total / max(n_experts, 1)
-    return 1 if avg <= 8 else (2 if avg <= 48 else 4)
+    return 1 if avg <= 8 else 2
 
 
 def pick_ks(tt: int, rows_total: int) -> int:
@@ -300,7 +301,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
     n_items, items, max_items = tiling
     if out is None:
         if epi == EPI_SCATTER:
-            raise ValueError("scatter epilogue needs a caller-provided fp32 slot buffer")
+            raise ValueError("scatter epilogue needs a caller-provided fp16 slot buffer")
         out = torch.empty((rows_total, n_out), dtype=torch.float16, device=act.device)
         out_stride = n_out
     pool = gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index, w_scale_byte)
@@ -312,8 +313,10 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
 
 
 def combine_slots(slots: torch.Tensor, top_k: int, add: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t] = fp16(sum_j slots[t*k + j] (+ add[t])), slots fp32 [T*k, H]."""
+    """out[t] = fp16(sum_j slots[t*k + j] (+ add[t])), slots fp16 [T*k, H], summed in fp32."""
     _need_cuda(slots)
+    if slots.dtype != torch.float16:
+        raise TypeError("slots must be float16")
     rows, hidden = slots.shape
     tokens = rows // top_k
     out = torch.empty((tokens, hidden), dtype=torch.float16, device=slots.device)

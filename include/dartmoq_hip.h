@@ -41,9 +41,9 @@ enum {
   DMQ_ERR_MODE = 5, DMQ_ERR_NULL = 6, DMQ_ERR_HIP = 7, DMQ_ERR_LIMIT = 8
 };
 enum { DMQ_MODE_A16 = 0, DMQ_MODE_A8 = 1, DMQ_MODE_FP8 = 2, DMQ_MODE_FP4 = 3 };
-/* STORE: fp16 [rows, n_out].  SILU: fp16 silu(gate)*up [rows, I].  SCATTER: fp32 routing-weighted
+/* STORE: fp16 [rows, n_out].  SILU: fp16 silu(gate)*up [rows, I].  SCATTER: fp16 routing-weighted
  * rows stored at out[row_slot[r]] (one slot per (token, top-k slot)); dmq_combine_slots adds
- * the k slots of each token in slot order. */
+ * the k slots of each token in fp32, in slot order. */
 enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
@@ -179,7 +179,7 @@ typedef struct {
   const void* items;        /* from dmq_build_tiles / dmq_route_permute, tile_rows == 16*tt */
   const void* n_items;
   int max_items;
-  void* out;                /* STORE/SILU: fp16 [rows, out_stride]; SCATTER: fp32 [slots, out_stride] */
+  void* out;                /* STORE/SILU: fp16 [rows, out_stride]; SCATTER: fp16 [slots, out_stride] */
   long out_stride;
   const void* row_weight;   /* SCATTER: fp32 routing weight per row */
   const void* row_slot;     /* SCATTER: int32 destination slot row per row */
@@ -198,8 +198,8 @@ typedef struct {
 int dmq_matmul_merged_gf(const dmq_gemm_args* args, void* stream);
 
 /* out[t, h] = fp16( sum_{j<k} slots[t*k + j, h] (+ add[t, h]) ): the index_add_ of
- * bit_partitioned_moe.py:967 with a fixed summation order.  hidden % 4 == 0. */
-int dmq_combine_slots(const void* slots_f32, int k, const void* add_f16, long tokens, int hidden,
+ * bit_partitioned_moe.py:967 with a fixed summation order and an fp32 sum.  hidden % 8 == 0. */
+int dmq_combine_slots(const void* slots_f16, int k, const void* add_f16, long tokens, int hidden,
                       void* out_f16, void* stream);
 
 /* fp16(out32 (+ add16)) over n elements (n % 4 == 0). */

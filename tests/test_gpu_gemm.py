@@ -172,7 +172,7 @@ def test_silu_and_scatter_epilogues():
     dcommon = dict(groups=inter // 128, n_out=hidden, slice_is_groups=True, rows_total=rows_total, tt=1)
     dn = ops.matmul_merged(A16, bit, STORE, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(),
                            dinfo_dev, **dcommon).float().cpu()
-    slots = torch.full((rows_total, hidden), float("nan"), dtype=torch.float32, device="cuda")
+    slots = torch.full((rows_total, hidden), float("nan"), dtype=torch.float16, device="cuda")
     ops.matmul_merged(A16, bit, SCATTER, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(),
                       dinfo_dev, out=slots, out_stride=hidden, row_weight=wts.cuda(),
                       row_slot=slot.cuda(), **dcommon)

@@ -78,7 +78,8 @@ def test_permute_matches_oracle(tokens, tile_rows):
             if member:
                 assert gu[e, 2] == start[pi, e] and gu[e, 3] == 2 * inter
                 assert dn[e, 2] == start[pi, e] // 256 and dn[e, 3] == inter // 128
-            exp_items += [(pi, e, i, 0) for i in range(-(-cnt // tile_rows))]
+            exp_items += [(pi, e, i, int(offs[e]), cnt, int(start[pi, e]), int(start[pi, e]) // 256, 0)
+                          for i in range(-(-cnt // tile_rows))]
     n = int(res["n_items"][0])
     assert n == len(exp_items)
     assert [tuple(r) for r in res["items"][:n].cpu().tolist()] == exp_items

@@ -59,7 +59,7 @@ def test_argument_validation_without_gpu():
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # bad K split
     a.ks = 0
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 6                       # null pointers
-    assert lib.dmq_combine_slots(p, 8, None, 4, 6, p, None) == 2                      # hidden % 4
+    assert lib.dmq_combine_slots(p, 8, None, 4, 6, p, None) == 2                      # hidden % 8
     with pytest.raises(ValueError):
         _lib.check(2, "demo")
     with pytest.raises(TypeError):
@@ -75,9 +75,9 @@ def test_workspace_size_formula():
     small = lib.dmq_moe_workspace_bytes(ctypes.byref(d), 64)
     big = lib.dmq_moe_workspace_bytes(ctypes.byref(d), 4096)
     r = 4096 * 8
-    # dominated by the fp32 slot rows [R, H], x codes by routed row [R, H] and by token
+    # dominated by the fp16 slot rows [R, H], x codes by routed row [R, H] and by token
     # [pools, T, H] (2 bytes per element) and act / act codes [R, I]
-    main = r * 2048 * 4 + r * 2048 * 2 + 3 * 4096 * 2048 * 2 + 2 * r * 512 * 2
+    main = r * 2048 * 2 + r * 2048 * 2 + 3 * 4096 * 2048 * 2 + 2 * r * 512 * 2
     assert big >= main
     assert big < 1.15 * main + (1 << 22)
     assert small < big

@@ -25,9 +25,16 @@ static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE
 // unless every wave takes a quarter of K; otherwise the waves own different output features
 static inline int pick_ks(int tt, long rows) { return (tt == 1 && rows <= 64) ? 4 : 1; }
 
+// Feature blocks one workgroup walks back to back.  With few row tiles every block gets its own
+// workgroup (parallelism); with many, a workgroup amortizes its start-up over several blocks.
+static inline int pick_nbl(long rows, int tt) {
+  const long tiles = rows / (16 * tt);
+  return tiles >= 1024 ? 4 : (tiles >= 384 ? 2 : 1);
+}
+
 extern "C" {
 
-int dmq_abi_version(void) { return 3; }
+int dmq_abi_version(void) { return 4; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -228,6 +235,11 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.n_items = (const int*)a->n_items;
   const int feat_per_block = (4 / ks) * feat_per_wave;
   p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
+  // several n-blocks per workgroup need every block complete and the waves on distinct features
+  int nbl = a->nbl > 0 ? a->nbl : 1;
+  if (ks > 1 || a->n_out % feat_per_block) nbl = 1;
+  if (nbl > p.n_blocks) nbl = p.n_blocks;
+  p.nbl = nbl;
   p.out = (__half*)a->out;
   p.out_stride = a->out_stride;
   p.out_slots = (__half*)a->out;
@@ -239,7 +251,8 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   L.ks = ks;
   L.dbg = a->dbg_acc != nullptr;
   L.stream = (hipStream_t)stream;
-  const long work = (long)a->max_items * p.n_blocks;
+  long work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl);
+  work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;      // every XCD gets the same number of slots
   if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
   L.grid = (int)work;
   switch (a->mode) {
@@ -297,7 +310,9 @@ static inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static int pick_tt(int tokens, int top_k, int experts) {
   const long avg = (long)tokens * top_k / (experts > 0 ? experts : 1);
-  return avg <= 8 ? 1 : 2;      // 64-row tiles run one workgroup per CU and measured slower
+  // 64-row tiles pay off once padding is small: they halve the look-ups per row but run two
+  // workgroups per CU instead of three
+  return avg <= 8 ? 1 : (avg <= 160 ? 2 : 4);
 }
 
 static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* base) {
@@ -342,14 +357,15 @@ size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens) {
 
 int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                         const void* topk_w, int tokens, const void* add_f16, void* out,
-                        void* workspace, size_t workspace_bytes, int tt, int ks, void* stream) {
+                        void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
+                        void* stream) {
   return dmq_moe_ffn_forward_staged(layer, x, topk_idx, topk_w, tokens, add_f16, out, workspace,
-                                    workspace_bytes, tt, ks, nullptr, nullptr, stream);
+                                    workspace_bytes, tt, ks, nbl, nullptr, nullptr, stream);
 }
 
 int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                                const void* topk_w, int tokens, const void* add_f16, void* out,
-                               void* workspace, size_t workspace_bytes, int tt, int ks,
+                               void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
                                void* const* stage_events, void* aux_out, void* stream) {
   if (!layer || !x || !topk_idx || !topk_w || !out || !workspace || !layer->pool) return DMQ_ERR_NULL;
   auto mark = [&](int i) {
@@ -365,6 +381,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
   if (ks <= 0) ks = pick_ks(tt, (long)tokens * K);
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
+  if (nbl <= 0) nbl = pick_nbl((long)tokens * K, tt);
   const int rot_tt = tt;               // a rotation wave covers one row tile of the work items
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
   if (w.bytes > workspace_bytes) return DMQ_ERR_LIMIT;
@@ -374,6 +391,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
     long* aux = (long*)aux_out;
     aux[0] = tt; aux[1] = ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
     aux[3] = w.max_items; aux[4] = (long)((uint8_t*)w.n_items - (uint8_t*)workspace);
+    aux[5] = nbl;
   }
   mark(0);
 
@@ -432,7 +450,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
     dmq_gemm_args g{};
-    g.mode = mode; g.epi = DMQ_EPI_SILU; g.tt = tt; g.ks = ks; g.n_pools = P;
+    g.mode = mode; g.epi = DMQ_EPI_SILU; g.tt = tt; g.ks = ks; g.nbl = nbl; g.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = pd.major != 0;
@@ -480,7 +498,7 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
     dmq_gemm_args d{};
-    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt; d.ks = ks; d.n_pools = P;
+    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt; d.ks = ks; d.nbl = nbl; d.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       d.pool[i] = dmq_gemm_pool{pd.dn_w, pd.dn_norms, pd.dn_lut, w.dn_info + (size_t)i * E * 4,

@@ -27,7 +27,11 @@ static inline int dmq_check_launch() {
 static inline bool dmq_valid_bit(int bit) { return bit == 1 || bit == 2 || bit == 4; }
 
 // ---------------------------------------------------------------- device helpers
-__device__ __forceinline__ float dmq_silu(float x) { return x / (1.0f + __expf(-x)); }
+// silu(x) = x * sigmoid(x); the hardware reciprocal (1 ulp) replaces the IEEE division, the
+// result is rounded to fp16 by every caller
+__device__ __forceinline__ float dmq_silu(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
 
 // OCP e4m3fn encode of a finite fp32 already clamped to [-448, 448]; round to nearest even.
 __device__ __forceinline__ uint32_t dmq_f32_to_e4m3(float f) {

@@ -37,8 +37,18 @@ static __device__ long long dmq_trace_buf[256];
 #define DMQ_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x == 0) { \
     dmq_trace_buf[2 * (i)] = __builtin_readcyclecounter(); \
     dmq_trace_buf[2 * (i) + 1] = wall_clock64(); } } while (0)
+// per-workgroup wall-clock stamps (100 MHz): [0] entry, [1] table ready, [2] exit, [3] hardware id
+#define DMQ_WG_SLOTS 8192
+#ifndef DMQ_TRACE_EPI
+#define DMQ_TRACE_EPI DMQ_EPI_SILU
+#endif
+static __device__ long long dmq_wg_buf[DMQ_WG_SLOTS * 4];
+#define DMQ_WG_MARK(i) do { if (EPI == DMQ_TRACE_EPI && threadIdx.x == 0 && blockIdx.x < DMQ_WG_SLOTS) { \
+    dmq_wg_buf[blockIdx.x * 4 + (i)] = wall_clock64(); \
+    if ((i) == 0) dmq_wg_buf[blockIdx.x * 4 + 3] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)); } } while (0)
 #else
 #define DMQ_MARK(i)
+#define DMQ_WG_MARK(i)
 #endif
 
 struct PoolW {
@@ -66,7 +76,8 @@ struct GemmParams {
   // work list
   const int* items;            // [max_items, DMQ_ITEM_WORDS] work-item records, meaningful below n_items
   const int* n_items;          // device scalar
-  int n_blocks;                // workgroups along the output features
+  int n_blocks;                // blocks of output features per item
+  int nbl;                     // consecutive blocks one workgroup walks (1 unless KS == 1)
   // outputs
   __half* out;                 // STORE / SILU: fp16 [rows, out_stride]
   long out_stride;
@@ -134,6 +145,13 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
 // Groups in flight per wave on the staged path.  WW registers hold one (group, n-tile) of packed
 // weights.  Rings of 8 words (16-row tiles) and 4 words (32-row tiles) keep three resp. two
 // workgroups resident per CU; deeper rings cost a workgroup of occupancy and measured slower.
+#define DMQ_XCDS 8          // accelerator dies of an MI355X; the grid is a multiple of it
+#ifndef DMQ_SCHED
+#define DMQ_SCHED 1
+#endif
+#ifndef DMQ_FOLD_MIN_TT
+#define DMQ_FOLD_MIN_TT 2
+#endif
 #ifndef DMQ_RING_TT1
 #define DMQ_RING_TT1 8
 #endif
@@ -166,7 +184,7 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
 template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
                                               uint8_t* smem2, int token_start, int token_count,
-                                              int slice_start, int ttile, int nb) {
+                                              int slice_start, int ttile, int nb, int nbc) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   using GG = GemmGeom<MODE, NT, TT, KS>;
@@ -180,6 +198,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr int UNITS = NT / UNIT;
   constexpr int FEAT_TILES = NT / UNIT;                              // output tiles per wave
   constexpr int PPG = (MODE == DMQ_MODE_FP4) ? 64 : (DMQ_GS * BIT / 8);
+  constexpr int FPB = ROWPARTS * FEAT_TILES * 16;                    // output features per n-block
   static_assert(NT % UNIT == 0, "SiLU epilogue pairs gate/up tiles");
 
   const int lane = threadIdx.x & 63;
@@ -192,6 +211,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 
   const int feat0 = (nb * ROWPARTS + rowpart) * (FEAT_TILES * 16);   // first output feature of the wave
   const bool wave_active = feat0 < p.n_out;                          // wave-uniform
+  int feat_k = feat0;                                                // same, for the n-block in progress
 
   // weight row of each n-tile (inactive waves alias the first block; they never store)
   const int featw = wave_active ? feat0 : 0;
@@ -275,10 +295,47 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       }
     }
   };
+  // FOLD (fp16 weights, tiles of 32 rows and more): the norm of the lane's weight row is
+  // multiplied into the dequantized fp16 operand, so the MFMAs accumulate straight into the
+  // running sums.  This drops the per-group accumulators (32 registers at TT = 2, which is
+  // what lets a third workgroup fit a CU) at the price of one fp16 rounding per weight.
+  constexpr bool FOLD = (MODE == DMQ_MODE_A16) && STAGE && (TT >= DMQ_FOLD_MIN_TT);
   auto compute = [&](int g, const uint32_t (&pk)[NT][WW], const uint2_t (&nr)[NT],
                      const uint32_t (&xa)[TT][AW], const float (&xs)[TT], const int (&xsb)[TT]) {
     uint32_t wqb[2][WQ];
     dequant_tile(pk[0], wqb[0]);
+#if DMQ_SCHED
+    if constexpr (FOLD) {
+      // Explicit software pipeline, one fence per MFMA step: scale this step's operand, issue a
+      // quarter of the next tile's look-ups, then the TT matrix instructions of the step.  The
+      // vector ALU work of a step does not depend on its MFMAs, so the two pipes overlap.
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        uint32_t (&wn)[WQ] = wqb[(j + 1) & 1];
+        const uint32_t (&wq)[WQ] = wqb[j & 1];
+        const _Float16 n = __builtin_bit_cast(half2_t, nr[j].x)[0];
+        const half8_t n8 = {n, n, n, n, n, n, n, n};
+        auto step = [&](auto sc) {
+          constexpr int s = decltype(sc)::value;
+          if (j + 1 < NT) dmq_dequant_step<MODE, BIT, s>(tbl, lane_base, pk[j + 1 < NT ? j + 1 : j], wn + s * OPW);
+          const half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[4 * s], wq[4 * s + 1],
+                                                                    wq[4 * s + 2], wq[4 * s + 3]}) * n8;
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            const half8_t b = __builtin_bit_cast(half8_t, (uint4_t){xa[t][4 * s], xa[t][4 * s + 1],
+                                                                    xa[t][4 * s + 2], xa[t][4 * s + 3]});
+            total_acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, total_acc[j][t], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
+        step(std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{});
+      }
+      return;
+    }
+#endif
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       if (j + 1 < NT) dequant_tile(pk[j + 1], wqb[(j + 1) & 1]);
@@ -291,11 +348,16 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         if constexpr (MODE == DMQ_MODE_A16) {
           half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[4 * s], wq[4 * s + 1], wq[4 * s + 2],
                                                             wq[4 * s + 3]});
+          if constexpr (FOLD) {
+            const _Float16 n = __builtin_bit_cast(half2_t, nr[j].x)[0];
+            a = a * (half8_t){n, n, n, n, n, n, n, n};
+          }
 #pragma unroll
           for (int t = 0; t < TT; ++t) {
             half8_t b = __builtin_bit_cast(half8_t, (uint4_t){xa[t][4 * s], xa[t][4 * s + 1],
                                                               xa[t][4 * s + 2], xa[t][4 * s + 3]});
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[t], 0, 0, 0);
+            if constexpr (FOLD) total_acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, total_acc[j][t], 0, 0, 0);
+            else acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[t], 0, 0, 0);
           }
         } else if constexpr (MODE == DMQ_MODE_A8) {
           int4_t a = {(int)wq[4 * s], (int)wq[4 * s + 1], (int)wq[4 * s + 2], (int)wq[4 * s + 3]};
@@ -326,16 +388,47 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       const float nrm[4] = {(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
+        if constexpr (!FOLD) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v = (float)acc[t][r];
-          if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) v = v * xs[t];
-          total_acc[j][t][r] += v * nrm[r];
+          for (int r = 0; r < 4; ++r) {
+            float v = (float)acc[t][r];
+            if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) v = v * xs[t];
+            total_acc[j][t][r] += v * nrm[r];
+          }
         }
         if (DBG && MODE == DMQ_MODE_A8 && avalid[t] && wave_active) {
           int4_t* d = (int4_t*)(p.dbg_acc + ((long)rlog[t] * p.groups + g) * p.n_out +
-                                feat0 + j * 16 + 4 * q);
+                                feat_k + j * 16 + 4 * q);
           *d = __builtin_bit_cast(int4_t, acc[t]);
+        }
+      }
+    }
+  };
+
+  // ---- store the finished sums of one n-block (features feat_k ...)
+  auto epilogue = [&]() {
+    if (!wave_active) return;
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      if (!avalid[t]) continue;
+#pragma unroll
+      for (int j = 0; j < NT; j += UNIT) {
+        if (KS > 1 && kpart != ((j / UNIT) * KS) / UNITS) continue;
+        if (EPI == DMQ_EPI_STORE) {
+          half4_t h = {(_Float16)total_acc[j][t][0], (_Float16)total_acc[j][t][1],
+                       (_Float16)total_acc[j][t][2], (_Float16)total_acc[j][t][3]};
+          *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat_k + j * 16 + 4 * q) = h;
+        } else if (EPI == DMQ_EPI_SILU) {
+          half4_t h;
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
+          *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat_k + (j >> 1) * 16 + 4 * q) = h;
+        } else {
+          const float rw = p.row_weight[rlog[t]];
+          const float4_t v = total_acc[j][t] * rw;
+          const half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+          *(half4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat_k + j * 16 + 4 * q) = h;
         }
       }
     }
@@ -418,12 +511,12 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     const uint8_t* const w_p = pw.w;
     const long group_rows = pw.n_total;
     auto lane_off = [](uint32_t o) { asm volatile("" : "+v"(o)); return o; };
-    auto stage_load = [&](int g, Staged& sr) {
+    auto stage_load = [&](int k, int g, Staged& sr) {
       const uint8_t* abase = act_p + (long)g * AB;
 #pragma unroll
       for (int c = 0; c < CPT; ++c)
         sr.a[c] = s_valid ? *(const uint4_t*)(abase + lane_off(s_off) + c * 16) : (uint4_t){0u, 0u, 0u, 0u};
-      const uint8_t* nbase = norms_p + (long)(g_base + g) * group_rows * 2;
+      const uint8_t* nbase = norms_p + ((long)(g_base + g) * group_rows + (long)k * FPB) * 2;
       sr.nrm = n_active ? *(const uint16_t*)(nbase + lane_off(n_off)) : 0u;
       sr.sc = 0u;
       if constexpr (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
@@ -467,33 +560,47 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         }
       }
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        nr[j] = *(const uint2_t*)(slot + NORM_OFF + ((wave * NT + j) * 16 + 4 * q) * 2);
+      for (int j = 0; j < NT; ++j) {
+        if constexpr (FOLD) {     // the norm of the lane's own weight row, in both halves of a word
+          const uint32_t n = *(const uint16_t*)(slot + NORM_OFF + ((wave * NT + j) * 16 + l16) * 2);
+          nr[j] = (uint2_t){n | (n << 16), 0u};
+        } else {
+          nr[j] = *(const uint2_t*)(slot + NORM_OFF + ((wave * NT + j) * 16 + 4 * q) * 2);
+        }
+      }
     };
-    auto load_packed = [&](int g, uint32_t (&pk)[NT][WW]) {
-      const uint8_t* wbase = w_p + (long)(g_base + g) * group_rows * PPG;
+    auto load_packed = [&](int k, int g, uint32_t (&pk)[NT][WW]) {
+      const uint8_t* wbase = w_p + ((long)(g_base + g) * group_rows + (long)k * FPB) * PPG;
 #pragma unroll
       for (int j = 0; j < NT; ++j) dmq_load_words<WW>(wbase + lane_off(w_off[j]), pk[j]);
     };
 
-    // Every load below is unconditional (group indices past the end are clamped to the last
-    // group, whose data is simply fetched again) and ring entry u is refilled only after its
-    // last use in program order: the loaded registers then carry straight across the loop's
-    // back edge, with no copy that would have to wait for loads still in flight.
+    // A workgroup walks nbc consecutive n-blocks of its item as one stream of nbc * G steps
+    // (step = one group of one n-block), so the loads of the next n-block are in flight while
+    // the current one finishes; the sums are stored and cleared at each n-block boundary.
+    // Every load is unconditional (positions past the last step repeat the last step) and ring
+    // entry u is refilled only after its last use in program order: the loaded registers then
+    // carry straight across the loop's back edge, with no copy that would have to wait for
+    // loads still in flight.
     constexpr int D = dmq_ring_depth<WW, TT>();
     static_assert(D % 2 == 0, "the LDS slot of a ring entry is fixed by its parity");
     uint32_t pkb[D][NT][WW];
     Staged srb[D];
-    const int g_last = g_hi - 1;
+    const int G = g_hi;
+    const int steps = nbc * G;
+    int lk = 0, lg = 0;                                // load position: n-block, group
+    auto next_load = [&]() {
+      if (lk * G + lg < steps - 1) { if (++lg == G) { lg = 0; ++lk; } }
+    };
     // the codebook entries of this thread's table row are requested first: they arrive while
     // the weights are still in flight and the table is ready one memory latency after launch
     uint32_t lutw[4];
     if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_fetch<BIT, T::ES>(pw.lut, threadIdx.x, lutw);
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      const int gl = (g_lo + u < g_last) ? g_lo + u : g_last;
-      stage_load(gl, srb[u]);
-      load_packed(gl, pkb[u]);
+      stage_load(lk, lg, srb[u]);
+      load_packed(lk, lg, pkb[u]);
+      next_load();
     }
     DMQ_MARK(1);
     if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_store_wave<BIT, T::ES>(tbl, wave, lutw);
@@ -501,24 +608,35 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     stage_store(0, srb[0]);
     __syncthreads();
     DMQ_MARK(3);
-    for (int gb = g_lo; gb < g_hi; gb += D) {
+    DMQ_WG_MARK(1);
+    int cg = 0;                                        // group of the step being computed
+    for (int sb = 0; sb < steps; sb += D) {
 #pragma unroll
       for (int u = 0; u < D; ++u) {
-        const int g = gb + u;
-        const int gl = (g + D < g_last) ? g + D : g_last;
-        stage_load(gl, srb[u]);                        // entry u went to LDS one step ago
-        if (g < g_hi) {                                // uniform over the workgroup
+        const bool live = sb + u < steps;              // uniform over the workgroup
+        stage_load(lk, lg, srb[u]);                    // entry u went to LDS one step ago
+        if (live) {
           uint32_t xa[TT][AW];
           uint2_t nr[NT];
           float xs[TT];
           int xsb[TT];
           stage_read(u & 1, xa, nr, xs, xsb);
-          compute(g, pkb[u], nr, xa, xs, xsb);
+          compute(cg, pkb[u], nr, xa, xs, xsb);
         }
-        load_packed(gl, pkb[u]);
+        load_packed(lk, lg, pkb[u]);
+        next_load();
         stage_store((u & 1) ^ 1, srb[(u + 1) % D]);
+        if (live && ++cg == G) {                       // n-block finished
+          epilogue();
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int t = 0; t < TT; ++t) total_acc[j][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+          cg = 0;
+          feat_k += FPB;
+        }
         __syncthreads();
-        DMQ_MARK(4 + g);
+        DMQ_MARK(4 + sb + u);
       }
     }
   }
@@ -555,51 +673,40 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       }
     }
   }
-  if (!wave_active) return;
-
-  // ------------------------------------------------------------------ epilogue
-#pragma unroll
-  for (int t = 0; t < TT; ++t) {
-    if (!avalid[t]) continue;
-#pragma unroll
-    for (int j = 0; j < NT; j += UNIT) {
-      if (KS > 1 && kpart != ((j / UNIT) * KS) / UNITS) continue;
-      if (EPI == DMQ_EPI_STORE) {
-        half4_t h = {(_Float16)total_acc[j][t][0], (_Float16)total_acc[j][t][1],
-                     (_Float16)total_acc[j][t][2], (_Float16)total_acc[j][t][3]};
-        *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + j * 16 + 4 * q) = h;
-      } else if (EPI == DMQ_EPI_SILU) {
-        half4_t h;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
-        *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat0 + (j >> 1) * 16 + 4 * q) = h;
-      } else {
-        const float rw = p.row_weight[rlog[t]];
-        const float4_t v = total_acc[j][t] * rw;
-        const half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-        *(half4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat0 + j * 16 + 4 * q) = h;
-      }
-    }
-  }
-  DMQ_MARK(60);
+  if constexpr (!STAGE) epilogue();
+  DMQ_MARK(120);
+  DMQ_WG_MARK(2);
 }
 
+// Waves per SIMD the register allocation aims for: three for tiles up to 32 rows (the 32-row
+// fp16 kernel sits a few registers above that limit otherwise), two for 64-row tiles.
 template <int MODE, int TT, int EPI, int KS, bool DBG>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((KS == 1 && TT <= 2) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
   constexpr int NT = 4;
   __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
-  __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2];
+#ifndef DMQ_LDS_PAD
+#define DMQ_LDS_PAD 0
+#endif
+  __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2 + DMQ_LDS_PAD];
 
   DMQ_MARK(0);
-  const int item = blockIdx.x / p.n_blocks;
-  const int nb = blockIdx.x - item * p.n_blocks;
-  // the record is fetched together with the item count; it is only trusted below the count
+  DMQ_WG_MARK(0);
+  // Workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD gets a contiguous range of
+  // the work list, so the workgroups that share an activation tile (the feature blocks of an
+  // item) and those that share weights (the row tiles of an expert) meet in one L2.
+  const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl;      // workgroups per item
+  const int total = p.n_items[0] * nbg;
+  const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
+  const int slot = blockIdx.x / DMQ_XCDS;
+  const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
+  if (slot >= per_xcd || unit >= total) return;
+  const int item = unit / nbg;
+  const int nb = (unit - item * nbg) * p.nbl;
+  const int nbc = min(p.nbl, p.n_blocks - nb);
   const int4_t* rec = (const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * item);
   const int4_t r0 = rec[0];
   const int4_t r1 = rec[1];
-  if (item >= p.n_items[0]) return;
   const int pool = r0[0];
   const int ttile = r0[2];
   const int token_start = r0[3];
@@ -608,12 +715,12 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE) return;
   if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb);
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc);
   } else {
     switch (pw.bit) {
-      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb); break;
-      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb); break;
-      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb); break;
+      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;
+      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;
+      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;
     }
   }
 }

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 3
+ABI_VERSION = 4
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER = 0, 1, 2
@@ -36,7 +36,8 @@ class GemmPool(Structure):
 
 class GemmArgs(Structure):
     _fields_ = [
-        ("mode", c_int), ("epi", c_int), ("tt", c_int), ("ks", c_int), ("n_pools", c_int),
+        ("mode", c_int), ("epi", c_int), ("tt", c_int), ("ks", c_int), ("nbl", c_int),
+        ("n_pools", c_int),
         ("pool", GemmPool * MAX_POOLS),
         ("act_row_bytes", c_long), ("act_scale_stride", c_int),
         ("groups", c_int), ("n_out", c_int), ("half_width", c_int), ("slice_is_groups", c_int),
@@ -93,10 +94,10 @@ PROTOTYPES = {
     "dmq_fill_zero": (c_int, [c_void_p, c_long, c_void_p]),
     "dmq_moe_workspace_bytes": (c_size_t, [POINTER(LayerDesc), c_int]),
     "dmq_moe_ffn_forward": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                    c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p]),
+                                    c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p]),
     "dmq_moe_ffn_forward_staged": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int,
                                            c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int,
-                                           POINTER(c_void_p), POINTER(c_long), c_void_p]),
+                                           c_int, POINTER(c_void_p), POINTER(c_long), c_void_p]),
 }
 
 _lib = None

@@ -121,6 +121,7 @@ class WxA16BitPartitionedGroupMoE:
         self._workspace = None
         self.tt_override = 0        # activation tiles of 16 rows per wave (0 = pick from tokens)
         self.ks_override = 0        # waves splitting K inside a workgroup (0 = pick from tt)
+        self.nbl_override = 0       # feature blocks per workgroup of the GEMMs (0 = pick from tokens)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -253,7 +254,7 @@ class WxA16BitPartitionedGroupMoE:
         check(load().dmq_moe_ffn_forward(
             ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens,
             None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-            int(self.tt_override), int(self.ks_override), stream), "moe_ffn_forward")
+            int(self.tt_override), int(self.ks_override), int(self.nbl_override), stream), "moe_ffn_forward")
         if orig_dtype != torch.float16:
             out = out.to(orig_dtype)
         return out.reshape(shape)
@@ -344,7 +345,8 @@ STAGE_NAMES = ("sort_prep", "rotation", "merged_gate_up", "act_quant_down", "mer
 
 @torch.no_grad()
 def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: torch.Tensor,
-                   topk_w: torch.Tensor, tt: int = 0, ks: int = 0, profile: bool = True):
+                   topk_w: torch.Tensor, tt: int = 0, ks: int = 0, nbl: int = 0,
+                   profile: bool = True):
     """dmq_moe_ffn_forward_staged: the production forward with an event recorded on the launch
     stream after every stage.  Returns (out fp16 [T, H], {stage: ms}, aux) where aux carries the
     per-expert routed-row counts (for byte accounting) and the tiling that was used.  Stage names
@@ -369,7 +371,7 @@ def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: 
     check(load().dmq_moe_ffn_forward_staged(
         ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens, None,
         out.data_ptr(), ws.data_ptr(), ws.numel(), int(tt or moe.tt_override),
-        int(ks or moe.ks_override), handles if profile else None, aux,
+        int(ks or moe.ks_override), int(nbl or moe.nbl_override), handles if profile else None, aux,
         ctypes.c_void_p(stream.cuda_stream)), "moe_ffn_forward_staged")
     torch.cuda.synchronize(x.device)
     stats = {}
@@ -378,4 +380,5 @@ def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: 
             stats[name] = events[i].elapsed_time(events[i + 1])
     counts = ws[aux[2]:aux[2] + 4 * moe.num_experts].view(torch.int32).clone()
     n_items = int(ws[aux[4]:aux[4] + 4].view(torch.int32).item())
-    return out, stats, {"counts": counts, "tt": int(aux[0]), "ks": int(aux[1]), "n_items": n_items}
+    return out, stats, {"counts": counts, "tt": int(aux[0]), "ks": int(aux[1]), "nbl": int(aux[5]),
+                        "n_items": n_items}

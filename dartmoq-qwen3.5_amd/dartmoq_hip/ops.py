@@ -238,7 +238,7 @@ def quantize_act(mode: int, x_rot: torch.Tensor, extra_scale: float = 1.0, scale
 
 def pick_tt(rows_total: int, n_experts: int) -> int:
     avg = rows_total / max(n_experts, 1)
-    return 1 if avg <= 8 else 2
+    return 1 if avg <= 8 else (2 if avg <= 160 else 4)
 
 
 def pick_ks(tt: int, rows_total: int) -> int:
@@ -252,11 +252,11 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 
 
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
-                 tt, ks=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
+                 tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list."""
     a = GemmArgs()
-    a.mode, a.epi, a.tt, a.ks, a.n_pools = mode, epi, tt, ks, len(pools)
+    a.mode, a.epi, a.tt, a.ks, a.nbl, a.n_pools = mode, epi, tt, ks, nbl, len(pools)
     dev = None
     for i, p in enumerate(pools):
         _need_cuda(p["act"], p["w"], p["norms"], p["expert_info"])
@@ -288,7 +288,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
 
 def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *, groups, n_out,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
-                  row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0,
+                  row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
                   tiling=None, dbg_acc=None):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
@@ -306,7 +306,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
         out_stride = n_out
     pool = gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index, w_scale_byte)
     return matmul_pools(mode, epi, [pool], items, n_items, max_items, groups=groups, n_out=n_out,
-                        slice_is_groups=slice_is_groups, tt=tt, ks=ks, out=out,
+                        slice_is_groups=slice_is_groups, tt=tt, ks=ks, nbl=nbl, out=out,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
                         dbg_acc=dbg_acc)

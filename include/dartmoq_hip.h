@@ -48,7 +48,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 3). */
+/* Library / build identification: returns the ABI version (currently 4). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -168,6 +168,8 @@ typedef struct {
   int epi;                  /* DMQ_EPI_* */
   int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4 */
   int ks;                   /* waves of a workgroup splitting K: 0 = 1; 4 or 1 for tt == 1, else 1 */
+  int nbl;                  /* blocks of output features one workgroup walks back to back (its
+                               loads stay in flight across blocks): 0 = 1; used when ks == 1 */
   int n_pools;
   dmq_gemm_pool pool[DMQ_MAX_POOLS];
   long act_row_bytes;
@@ -235,20 +237,22 @@ size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens);
  * and its WxA8 / WxFP8 / WxFP4 subclasses, routed experts only:
  *   x fp16 [tokens, hidden]; topk_idx int32 / topk_w fp32 [tokens, top_k];
  *   out fp16 [tokens, hidden] = sum_k w * down_e(silu(gate_e(x)) * up_e(x)) (+ add_f16).
- * Every expert must belong to exactly one pool.  tt <= 0 / ks <= 0 pick the tiling from tokens. */
+ * Every expert must belong to exactly one pool.  tt <= 0 / ks <= 0 / nbl <= 0 pick the tiling
+ * (rows per tile, K split, feature blocks per workgroup) from tokens. */
 int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                         const void* topk_w, int tokens, const void* add_f16, void* out,
-                        void* workspace, size_t workspace_bytes, int tt, int ks, void* stream);
+                        void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
+                        void* stream);
 
 /* Same forward with instrumentation, the role of the reference's CudaStageProfiler
  * (turboquant_utils/cuda_profiler.py:51-174): stage_events (optional) is a host array of 7
  * hipEvent_t recorded on `stream` before the first launch and after each stage (sort_prep,
  * rotation, merged_gate_up, act_quant_down, merged_down, combine); aux_out (optional) is a host
  * long[8] that receives tt, ks, the byte offset of counts[experts] inside the workspace,
- * max_items and the byte offset of n_items. */
+ * max_items, the byte offset of n_items and nbl. */
 int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                                const void* topk_w, int tokens, const void* add_f16, void* out,
-                               void* workspace, size_t workspace_bytes, int tt, int ks,
+                               void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
                                void* const* stage_events, void* aux_out, void* stream);
 
 #ifdef __cplusplus

@@ -206,6 +206,48 @@ def test_k_split_variants_agree(tt, ks):
     torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
 
 
+@pytest.mark.parametrize("tt", [1, 2, 4])
+@pytest.mark.parametrize("epi", ["silu", "store", "scatter"])
+def test_blocks_per_workgroup_identical(tt, epi):
+    """A workgroup walking 2, 3 or all feature blocks stores exactly what one block per
+    workgroup stores (same arithmetic, only the schedule differs)."""
+    from dartmoq_hip import ops
+    bit, k = 2, 512
+    counts = [5, 70, 0, 33]
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(900 + tt)
+    x = (torch.randn(rows_total, k, generator=g) * 0.5).half().cuda()
+    if epi == "silu":
+        inter = 512                                            # 4 blocks of 128 features
+        idx_gf, norms_gf, cb = _pool(bit, 2 * inter * len(counts), k, 91)
+        info = [(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(len(counts))]
+        kw = dict(n_out=inter, half_width=inter, slice_is_groups=False)
+        mode_epi = SILU
+    else:
+        n_slice = 1024                                         # 4 blocks of 256 features
+        idx_gf, norms_gf, cb = _pool(bit, n_slice * len(counts), k, 92)
+        info = [(starts[e], counts[e], e * n_slice, n_slice) for e in range(len(counts))]
+        kw = dict(n_out=n_slice, slice_is_groups=False)
+        mode_epi = STORE if epi == "store" else SCATTER
+    info_dev = torch.tensor(info, dtype=torch.int32).cuda()
+    slot = torch.randperm(rows_total, generator=g).int().cuda()
+    wts = torch.rand(rows_total, generator=g).cuda()
+    outs = []
+    for nbl in (1, 2, 3, 4):
+        extra = {}
+        if mode_epi == SCATTER:
+            extra = dict(out=torch.zeros(rows_total, kw["n_out"], dtype=torch.float16, device="cuda"),
+                         out_stride=kw["n_out"], row_weight=wts, row_slot=slot)
+        out = ops.matmul_merged(A16, bit, mode_epi, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(),
+                                info_dev, groups=k // 128, rows_total=rows_total, tt=tt, ks=1, nbl=nbl,
+                                **kw, **extra)
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    assert outs[0].abs().max() > 0
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
 def test_gemm_argument_errors():
     from dartmoq_hip import ops
     x = torch.zeros(16, 256, dtype=torch.float16, device="cuda")

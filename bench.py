@@ -112,7 +112,8 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
                 "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
-    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={aux['ks']},SILU> merged gate_up",
+    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={aux['ks']},SILU> merged gate_up, "
+                       f"nbl={aux['nbl']}",
                 launch_ms=gu_ms,
                 algorithmic_bytes=gu_bytes, algorithmic_flops=gu_flops,
                 distinct_experts=distinct, routed_rows=rows)
@@ -124,8 +125,24 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
         "layer_algorithmic_bytes": bytes_total,
         "gpu_stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
         "gpu_stage_sum_ms": round(sum(stage_ms.values()), 4),
-        "tt": aux["tt"], "ks": aux["ks"], "work_items": aux["n_items"],
+        "tt": aux["tt"], "ks": aux["ks"], "nbl": aux["nbl"], "work_items": aux["n_items"],
     }, roof
+
+
+def measured_traffic(config, mode, tokens):
+    """HBM bytes per launch of the dominant kernel from the committed counter runs
+    (profiles/gate_up_hbm_traffic.json: FETCH_SIZE + WRITE_SIZE, calibrated on a copy of known
+    size), or None when no run covers this workload."""
+    path = os.path.join(ROOT, "profiles", "gate_up_hbm_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    for r in rec.get("runs", []):
+        if r.get("config") == config and r.get("mode") == mode and r.get("tokens") == tokens:
+            return r.get("hbm_bytes_per_launch")
+    return None
 
 
 def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf):
@@ -161,6 +178,10 @@ def main():
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--cpu-tokens", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also launch dmq_finalize_kernel on 64 Mi fp32 elements (256 MiB read, "
+                         "128 MiB written): the known-size kernel that calibrates FETCH_SIZE / "
+                         "WRITE_SIZE counter runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -183,8 +204,17 @@ def main():
             pools, spec["experts"], spec["hidden"], spec["inter"], spec["top_k"], device="cuda")
         mods.append(dartmoq_hip.convert_moe(m, args.mode))
 
+    if args.traffic_probe:
+        from dartmoq_hip import ops
+        probe = torch.ones(64 << 20, dtype=torch.float32, device="cuda")
+        for _ in range(3):
+            ops.finalize_f16(probe)
+        torch.cuda.synchronize()
+        del probe
+
     main_res, roof = measure(mods, args.tokens, args.steps, args.warmup, args.seed, spec["zipf"],
                              args.mode)
+    roof["traffic"] = measured_traffic(args.config, args.mode, args.tokens)
     sweep = []
     for t in [int(v) for v in args.sweep.split(",") if v]:
         if t == args.tokens:

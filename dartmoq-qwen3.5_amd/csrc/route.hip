@@ -119,13 +119,18 @@ __device__ __forceinline__ int block_scan_incl(int v, int* wave_tot) {
 
 __global__ __launch_bounds__(1024)
 void dmq_plan_kernel(PlanParams p) {
+  // counts and offsets live in LDS between the phases; global memory is only written, so the
+  // kernel pays one round trip for the histogram and one for the slice tables
   __shared__ int wave_tot[16];
   __shared__ int carry;
   __shared__ int partial[1024];
+  __shared__ int s_cnt[DMQ_SORT_MAX_EXPERTS];
+  __shared__ int s_off[DMQ_SORT_MAX_EXPERTS + 1];
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
   // The chunk axis of the histogram is split over `parts` threads per expert so that all 1024
-  // threads load; a thread keeps at most 16 loads in flight.
+  // threads load; a thread keeps at most 16 loads in flight and its values stay in registers
+  // when its share of the chunks fits (16 per thread: up to 64 chunks at <= 256 experts).
   int epad = 64;
   while (epad < p.experts && epad < 1024) epad <<= 1;
   const int parts = 1024 / epad;
@@ -134,16 +139,19 @@ void dmq_plan_kernel(PlanParams p) {
   const int cpp = (p.n_chunks + parts - 1) / parts;
   const int c_lo = part * cpp;
   const int c_hi = min(p.n_chunks, c_lo + cpp);
+  const bool one_pass = p.experts <= epad && cpp <= 16;
+  int h[16];
+  auto load16 = [&](int e, int c0) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      h[i] = (e < p.experts && c0 + i < c_hi) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
+  };
   auto chunk_sum = [&](int e) {
     int sum = 0;
-    if (e < p.experts) {
-      for (int c0 = c_lo; c0 < c_hi; c0 += 16) {
-        int h[16];
+    for (int c0 = c_lo; c0 < c_hi; c0 += 16) {
+      load16(e, c0);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) h[i] = (c0 + i < c_hi) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sum += h[i];
-      }
+      for (int i = 0; i < 16; ++i) sum += h[i];
     }
     return sum;
   };
@@ -155,34 +163,36 @@ void dmq_plan_kernel(PlanParams p) {
     if (part == 0 && e < p.experts) {
       int total = 0;
       for (int q = 0; q < parts; ++q) total += partial[q * epad + el];
+      s_cnt[e] = total;
       p.counts[e] = total;
     }
-    __syncthreads();
+    if (!one_pass) __syncthreads();                    // partial[] is reused by the next pass
   }
+  __syncthreads();
   // expert offsets: exclusive scan of counts, 1024 experts per pass
   for (int base = 0; base < p.experts; base += 1024) {
     const int e = base + tid;
-    const int c = (e < p.experts) ? p.counts[e] : 0;
+    const int c = (e < p.experts) ? s_cnt[e] : 0;
     const int incl = block_scan_incl(c, wave_tot) + carry;
-    if (e < p.experts) p.offsets[e + 1] = incl;
+    if (e < p.experts) { s_off[e + 1] = incl; p.offsets[e + 1] = incl; }
     __syncthreads();
     if (tid == 1023) carry = incl;
     __syncthreads();
   }
-  if (tid == 0) p.offsets[0] = 0;
+  if (tid == 0) { s_off[0] = 0; p.offsets[0] = 0; }
   __syncthreads();
   // hist[c, e] <- position of the first row of chunk c routed to expert e
   for (int ebase = 0; ebase < p.experts; ebase += epad) {
     const int e = ebase + el;
-    partial[tid] = chunk_sum(e);
-    __syncthreads();
+    if (!one_pass) {
+      partial[tid] = chunk_sum(e);
+      __syncthreads();
+    }
     if (e < p.experts) {
-      int at = p.offsets[e + 1] - p.counts[e];
+      int at = s_off[e];
       for (int q = 0; q < part; ++q) at += partial[q * epad + el];
       for (int c0 = c_lo; c0 < c_hi; c0 += 16) {
-        int h[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) h[i] = (c0 + i < c_hi) ? p.hist[(long)(c0 + i) * p.experts + e] : 0;
+        if (!one_pass) load16(e, c0);                  // one_pass: h[] still holds this thread's chunks
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           if (c0 + i < c_hi) p.hist[(long)(c0 + i) * p.experts + e] = at;
@@ -190,21 +200,32 @@ void dmq_plan_kernel(PlanParams p) {
         }
       }
     }
-    __syncthreads();
+    if (!one_pass) __syncthreads();
   }
 
   // per-pool expert_info and the work-item list, pools in caller order, experts ascending
   if (tid == 0) carry = 0;
+  // the slice tables of all pools are requested at once when one pass covers the experts
+  int ss_pre[DMQ_MAX_POOLS], sc_pre[DMQ_MAX_POOLS];
+  const bool pre = p.experts <= 1024;
+#pragma unroll
+  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+    const bool ok = pre && pool < p.pools && tid < p.experts;
+    ss_pre[pool] = ok ? p.slice_start_rows[pool * p.experts + tid] : -1;
+    sc_pre[pool] = ok ? p.slice_count_rows[pool * p.experts + tid] : 0;
+  }
   __syncthreads();
-  for (int pool = 0; pool < p.pools; ++pool) {
+#pragma unroll
+  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+    if (pool >= p.pools) break;
     for (int base = 0; base < p.experts; base += 1024) {
       const int e = base + tid;
       int ntile = 0, ts = 0, tc = 0, gu_ss = 0, dn_ss = 0;
       if (e < p.experts) {
-        const int ss = p.slice_start_rows[pool * p.experts + e];
-        const int sc = p.slice_count_rows[pool * p.experts + e];
-        tc = (ss >= 0) ? p.counts[e] : 0;
-        ts = p.offsets[e + 1] - p.counts[e];
+        const int ss = pre ? ss_pre[pool] : p.slice_start_rows[pool * p.experts + e];
+        const int sc = pre ? sc_pre[pool] : p.slice_count_rows[pool * p.experts + e];
+        tc = (ss >= 0) ? s_cnt[e] : 0;
+        ts = s_off[e];
         gu_ss = ss >= 0 ? ss : 0;
         dn_ss = ss >= 0 ? ss / (2 * DMQ_GS) : 0;
         ntile = (tc + p.tile_rows - 1) / p.tile_rows;

@@ -154,6 +154,25 @@ class WxA16BitPartitionedGroupMoE:
         return moe
 
     @classmethod
+    def from_reference_module(cls, ref, gate_weight=None, renormalize=False, device="cuda"):
+        """Build from a loaded module of the reference (duck-typed, nothing is imported):
+        ``ref.bit_weights[bit_str]`` must offer ``gate_up_packed`` / ``down_packed`` dictionaries
+        (indices_packed, norms, codebook, seed, group_size, shape — the WxA16Weights properties,
+        quantization/wxa16/bit_partitioned_moe.py:78-150), ``ref.expert_offsets[bit_str]`` the
+        E+1 neuron offsets (:324), plus num_experts / hidden_size / intermediate_size / top_k
+        (:290-293).  Tensors are copied to ``device`` once; the reference module is not modified."""
+        pools = {}
+        for bit_str in ref.bit_weights.keys():
+            w = ref.bit_weights[bit_str]
+            offs = ref.expert_offsets[bit_str]
+            offs = offs.cpu().tolist() if torch.is_tensor(offs) else list(offs)
+            pools[str(bit_str)] = {"gate_up": dict(w.gate_up_packed), "down": dict(w.down_packed),
+                                   "expert_offsets": offs}
+        return cls.from_packed(pools, int(ref.num_experts), int(ref.hidden_size),
+                               int(ref.intermediate_size), int(ref.top_k), gate_weight, renormalize,
+                               device)
+
+    @classmethod
     def from_wxa16(cls, moe: "WxA16BitPartitionedGroupMoE"):
         """Switch an already loaded layer to this precision mode in place (no tensor copies),
         like WxA8BitPartitionedGroupMoE.from_wxa16 (wxa8/bit_partitioned_moe.py:47-61)."""

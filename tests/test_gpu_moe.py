@@ -101,3 +101,25 @@ def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):
         mod.forward(torch.zeros(4, small_layer.hidden, dtype=torch.float16))
+
+
+def test_from_reference_module_duck_typing():
+    """A stand-in with the attribute names of the reference module (bit_weights[bit].gate_up_packed /
+    down_packed, expert_offsets, sizes) loads into the same layer as from_packed."""
+    import types
+    import dartmoq_hip
+    layer = moe.build_layer(256, 128, 8, 2, [2, 4, 2, 4, 1, 4, 2, 2], seed=11)
+    ref = types.SimpleNamespace(
+        num_experts=layer.num_experts, hidden_size=layer.hidden, intermediate_size=layer.inter,
+        top_k=layer.top_k,
+        bit_weights={str(b): types.SimpleNamespace(gate_up_packed=p.gate_up, down_packed=p.down)
+                     for b, p in layer.pools.items()},
+        expert_offsets={str(b): torch.tensor(p.expert_offsets) for b, p in layer.pools.items()})
+    m1 = dartmoq_hip.WxA16BitPartitionedGroupMoE.from_reference_module(ref)
+    m2 = make_module(layer)
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(12, layer.hidden, generator=g) * 0.5).half().cuda()
+    logits = torch.randn(12, layer.num_experts, generator=g).cuda()
+    y1 = m1.forward(x, router_logits=logits)
+    y2 = m2.forward(x, router_logits=logits)
+    assert torch.equal(y1, y2)

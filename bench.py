@@ -39,12 +39,13 @@ def layer_bytes(mod, counts):
     h, i = mod.hidden_size, mod.intermediate_size
     total = 0
     per_pool = {}
+    n_exp = mod.num_experts + mod.n_shared      # the shared expert counts as n_shared slices
     for bit_str, bw in mod.bit_weights.items():
-        distinct = sum(1 for e in range(mod.num_experts)
+        distinct = sum(1 for e in range(n_exp)
                        if counts[e] > 0 and bw.expert_offsets[e + 1] > bw.expert_offsets[e])
-        rows = sum(int(counts[e]) for e in range(mod.num_experts)
+        rows = sum(int(counts[e]) for e in range(n_exp)
                    if bw.expert_offsets[e + 1] > bw.expert_offsets[e])
-        per_pool[bit_str] = (distinct, rows)
+        per_pool[bit_str] = (distinct, rows, bw.bit)
         total += distinct * mod.weight_bytes_per_expert(bw.bit)
     return total, per_pool
 
@@ -96,8 +97,8 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     gu_bytes = 0
     rows = 0
     distinct = 0
-    for b, (d_b, r_b) in per_pool.items():
-        gu_bytes += d_b * (2 * h * i * int(b) // 8 + 4 * h * i // 128)
+    for _key, (d_b, r_b, bit_b) in per_pool.items():
+        gu_bytes += d_b * (2 * h * i * bit_b // 8 + 4 * h * i // 128)
         gu_bytes += (tokens if r_b else 0) * h * 2 + r_b * i * 2
         rows += r_b
         distinct += d_b
@@ -145,7 +146,7 @@ def measured_traffic(config, mode, tokens):
     return None
 
 
-def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf):
+def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf, shared_cpu=None):
     """The CPU oracle (dequantize per call, fp32 matmuls) on a bounded sample of the workload."""
     import torch
     from oracle import moe as omoe, routing
@@ -153,6 +154,7 @@ def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf):
                           expert_bit=expert_bit)
     for b, p in pools_cpu.items():
         layer.pools[b] = omoe.BitPool(int(b), p["gate_up"], p["down"], p["expert_offsets"])
+    layer.shared = shared_cpu
     torch.set_num_threads(os.cpu_count() or 1)
     x = torch.randn(tokens, spec["hidden"], generator=torch.Generator().manual_seed(seed)).half()
     w, idx = routing.route_topk(routing.zipf_logits(tokens, spec["experts"], seed, skew=zipf),
@@ -198,10 +200,15 @@ def main():
     expert_bit = synthetic.assign_bits(spec["experts"], spec["fractions"], args.seed)
     pools = synthetic.build_pools(spec["hidden"], spec["inter"], spec["experts"], expert_bit,
                                   seed=args.seed, device="cuda")
+    shared = None
+    if spec.get("shared_inter"):
+        shared = synthetic.build_shared_expert(spec["hidden"], spec["shared_inter"], args.seed,
+                                               spec.get("shared_bit", 4), device="cuda")
     mods = []
     for _ in range(N_COPIES):
         m = dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
-            pools, spec["experts"], spec["hidden"], spec["inter"], spec["top_k"], device="cuda")
+            pools, spec["experts"], spec["hidden"], spec["inter"], spec["top_k"], device="cuda",
+            shared_expert=shared)
         mods.append(dartmoq_hip.convert_moe(m, args.mode))
 
     if args.traffic_probe:
@@ -230,7 +237,11 @@ def main():
                          "down": {k: (v.cpu() if torch.is_tensor(v) else v)
                                   for k, v in p["down"].items()},
                          "expert_offsets": p["expert_offsets"]} for b, p in pools.items()}
-        cpu = cpu_baseline(pools_cpu, spec, expert_bit, args.cpu_tokens, args.seed, spec["zipf"])
+        shared_cpu = None if shared is None else {
+            k: ({kk: (vv.cpu() if torch.is_tensor(vv) else vv) for kk, vv in v.items()}
+                if isinstance(v, dict) else v.cpu()) for k, v in shared.items()}
+        cpu = cpu_baseline(pools_cpu, spec, expert_bit, args.cpu_tokens, args.seed, spec["zipf"],
+                           shared_cpu)
 
     bits = {b: sum(1 for e in expert_bit if e == int(b)) for b in pools}
     line = {
@@ -241,7 +252,10 @@ def main():
         "config": {
             "workload": f"configs[{args.config}]: single MoE FFN layer, {args.mode}, H={spec['hidden']} "
                         f"E={spec['experts']} top-{spec['top_k']} I={spec['inter']} SwiGLU, "
-                        f"experts per bit {bits}, group 128, T={args.tokens} tokens, "
+                        f"experts per bit {bits}, "
+                        + (f"shared expert I_s={spec['shared_inter']} bit{spec.get('shared_bit', 4)}, "
+                           if shared is not None else "") +
+                        f"group 128, T={args.tokens} tokens, "
                         f"{'Zipf(1.1)-skewed' if spec['zipf'] else 'uniform'} randn router logits",
             "tokens": args.tokens, "mode": args.mode, "weight_copies_rotated": N_COPIES,
         },

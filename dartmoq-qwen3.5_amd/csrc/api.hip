@@ -34,7 +34,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 4; }
+int dmq_abi_version(void) { return 5; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -87,8 +87,24 @@ int dmq_fold_indices_to_e2m1(const void* idx_gf, const void* nib_lut, long rows,
 int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts, int k, int renorm,
                    void* out_w, void* out_idx, void* stream) {
   if (!logits || !out_w || !out_idx) return DMQ_ERR_NULL;
-  return dmq_route_topk_launch(logits, logits_fp16, tokens, experts, k, renorm, (float*)out_w,
-                               (int*)out_idx, (hipStream_t)stream);
+  return dmq_route_topk_launch(logits, logits_fp16, nullptr, nullptr, tokens, experts, k, renorm,
+                               (float*)out_w, (int*)out_idx, SharedGate{nullptr, nullptr, 0, 0},
+                               (hipStream_t)stream);
+}
+
+int dmq_route_topk_shared(const void* logits, int logits_fp16, const void* topk_idx_in,
+                          const void* topk_w_in, int tokens, int experts, int k, int renorm,
+                          const void* x_f16, const void* gate_row_f16, int hidden, int n_shared,
+                          void* out_w, void* out_idx, void* stream) {
+  if (!out_w || !out_idx) return DMQ_ERR_NULL;
+  if (!logits && (!topk_idx_in || !topk_w_in)) return DMQ_ERR_NULL;
+  if (n_shared < 0) return DMQ_ERR_SHAPE;
+  if (n_shared > 0 && (!x_f16 || !gate_row_f16 || hidden <= 0)) return DMQ_ERR_NULL;
+  return dmq_route_topk_launch(logits, logits_fp16, (const int*)topk_idx_in, (const float*)topk_w_in,
+                               tokens, experts, k, renorm, (float*)out_w, (int*)out_idx,
+                               SharedGate{(const __half*)x_f16, (const __half*)gate_row_f16, hidden,
+                                          n_shared},
+                               (hipStream_t)stream);
 }
 
 size_t dmq_route_scratch_bytes(int tokens, int k, int experts) {

@@ -59,6 +59,14 @@ static inline void dmq_sort_chunks(long rows, int* chunk_rows, int* n_chunks) {
   *n_chunks = (int)((rows + cr - 1) / cr);
 }
 
+// Sigmoid gate of the always-on shared experts (n_shared == 0: none).
+struct SharedGate {
+  const __half* x;               // [tokens, hidden]
+  const __half* gate_row;        // [hidden]
+  int hidden;
+  int n_shared;
+};
+
 struct PlanParams {
   int* counts;                   // [experts] rows per expert (written by the plan kernel)
   int* hist;                     // [n_chunks, experts] chunk histogram, then chunk start positions
@@ -79,8 +87,9 @@ struct PlanParams {
 
 int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream);
 int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
-int dmq_route_topk_launch(const void* logits, int logits_fp16, int tokens, int experts, int k,
-                          int renorm, float* out_w, int* out_idx, hipStream_t stream);
+int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx, const float* in_w,
+                          int tokens, int experts, int k, int renorm, float* out_w, int* out_idx,
+                          const SharedGate& sg, hipStream_t stream);
 int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int tokens, int k,
                              const PlanParams& plan, int* sorted_tokens,
                              float* sorted_weights, int* sorted_rows, hipStream_t stream);

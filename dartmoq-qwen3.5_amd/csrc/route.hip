@@ -16,10 +16,50 @@ template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
 
+// Always-on shared experts ride the routed path as n_shared extra columns of the top-k arrays:
+// column k + j names expert `experts + j` with weight sigmoid(x . gate_row), rounded to fp16 after
+// the dot and after the sigmoid like an fp16 Linear followed by torch.sigmoid.
+__device__ __forceinline__ void dmq_shared_columns(const SharedGate& sg, int tok, int experts, int k,
+                                                   int lane, float* out_w, int* out_idx) {
+  if (sg.n_shared <= 0) return;
+  const __half* xr = sg.x + (long)tok * sg.hidden;
+  float dot = 0.f;
+  for (int h = lane * 8; h < sg.hidden; h += 512) {
+    const half8_t a = *(const half8_t*)(xr + h);
+    const half8_t b = *(const half8_t*)(sg.gate_row + h);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) dot += (float)a[c] * (float)b[c];
+  }
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) dot += __shfl_xor(dot, m, 64);
+  const float z = (float)(_Float16)dot;
+  const float g = (float)(_Float16)(1.f / (1.f + expf(-z)));
+  const int stride = k + sg.n_shared;
+  if (lane < sg.n_shared) {
+    out_w[(long)tok * stride + k + lane] = g;
+    out_idx[(long)tok * stride + k + lane] = experts + lane;
+  }
+}
+
+// Widen caller-made top-k arrays [tokens, k] by the shared columns.
+__global__ __launch_bounds__(256)
+void dmq_topk_widen_kernel(const int* in_idx, const float* in_w, int tokens, int experts, int k,
+                           float* out_w, int* out_idx, SharedGate sg) {
+  const int lane = threadIdx.x & 63;
+  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tok >= tokens) return;
+  const int stride = k + sg.n_shared;
+  for (int j = lane; j < k; j += 64) {
+    out_w[(long)tok * stride + j] = in_w[(long)tok * k + j];
+    out_idx[(long)tok * stride + j] = in_idx[(long)tok * k + j];
+  }
+  dmq_shared_columns(sg, tok, experts, k, lane, out_w, out_idx);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256)
 void dmq_topk_kernel(const T* logits, int tokens, int experts, int k, int renorm,
-                     float* out_w, int* out_idx) {
+                     float* out_w, int* out_idx, SharedGate sg) {
   const int lane = threadIdx.x & 63;
   const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (tok >= tokens) return;
@@ -68,10 +108,12 @@ void dmq_topk_kernel(const T* logits, int tokens, int experts, int k, int renorm
         if (i == (be >> 6)) v[i] = -INFINITY;
     }
   }
+  const int stride = k + sg.n_shared;
   if (lane < k) {
-    out_w[(long)tok * k + lane] = renorm ? my_w / wsum : my_w;
-    out_idx[(long)tok * k + lane] = my_e;
+    out_w[(long)tok * stride + lane] = renorm ? my_w / wsum : my_w;
+    out_idx[(long)tok * stride + lane] = my_e;
   }
+  dmq_shared_columns(sg, tok, experts, k, lane, out_w, out_idx);
 }
 
 // ------------------------------------------------------------------------------ counting
@@ -353,17 +395,22 @@ void dmq_combine_kernel(const __half* slots, int k, const __half* add, long toke
 }
 
 // ------------------------------------------------------------------------------ host
-int dmq_route_topk_launch(const void* logits, int logits_fp16, int tokens, int experts, int k,
-                          int renorm, float* out_w, int* out_idx, hipStream_t stream) {
+int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx, const float* in_w,
+                          int tokens, int experts, int k, int renorm, float* out_w, int* out_idx,
+                          const SharedGate& sg, hipStream_t stream) {
   if (tokens <= 0) return DMQ_OK;
-  if (experts > 1024 || k > 64 || k > experts || k <= 0) return DMQ_ERR_LIMIT;
+  if (experts > 1024 || k > 64 || k > experts || k <= 0 || sg.n_shared > 64) return DMQ_ERR_LIMIT;
+  if (sg.n_shared > 0 && sg.hidden % 8) return DMQ_ERR_ALIGN;
   const int grid = (tokens + 3) / 4;
-  if (logits_fp16)
+  if (!logits)
+    hipLaunchKernelGGL(dmq_topk_widen_kernel, dim3(grid), dim3(256), 0, stream, in_idx, in_w, tokens,
+                       experts, k, out_w, out_idx, sg);
+  else if (logits_fp16)
     hipLaunchKernelGGL(dmq_topk_kernel<__half>, dim3(grid), dim3(256), 0, stream,
-                       (const __half*)logits, tokens, experts, k, renorm, out_w, out_idx);
+                       (const __half*)logits, tokens, experts, k, renorm, out_w, out_idx, sg);
   else
     hipLaunchKernelGGL(dmq_topk_kernel<float>, dim3(grid), dim3(256), 0, stream,
-                       (const float*)logits, tokens, experts, k, renorm, out_w, out_idx);
+                       (const float*)logits, tokens, experts, k, renorm, out_w, out_idx, sg);
   return dmq_check_launch();
 }
 

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 4
+ABI_VERSION = 5
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER = 0, 1, 2
@@ -77,6 +77,8 @@ PROTOTYPES = {
     "dmq_fold_indices_to_e2m1": (c_int, [c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p]),
     "dmq_route_topk": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                c_void_p]),
+    "dmq_route_topk_shared": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                      c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "dmq_route_permute": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                   c_int, c_int] + [c_void_p] * 10 + [c_size_t, c_void_p]),
     "dmq_route_scratch_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -104,6 +104,7 @@ class WxA16BitPartitionedGroupMoE:
 
     MODE = "wxa16"
     rotation_hoist_threshold = 1.5
+    SHARED_KEY = "shared"
 
     def __init__(self, num_experts: int, hidden_size: int, intermediate_size: int, top_k: int,
                  gate_weight: torch.Tensor | None = None, renormalize: bool = False, device="cuda"):
@@ -117,6 +118,11 @@ class WxA16BitPartitionedGroupMoE:
         self.bit_weights: dict[str, BitPoolWeights] = {}
         self.expert_offsets: dict[str, list] = {}
         self.bit_list: list[int] = []
+        # always-on shared expert, run as n_shared extra experts of the routed path (see
+        # attach_shared_expert); its pool sits in bit_weights under SHARED_KEY
+        self.n_shared = 0
+        self.shared_intermediate_size = 0
+        self.shared_gate_row = None
         self._desc = None
         self._workspace = None
         self.tt_override = 0        # activation tiles of 16 rows per wave (0 = pick from tokens)
@@ -126,9 +132,11 @@ class WxA16BitPartitionedGroupMoE:
     # ------------------------------------------------------------------ construction
     @classmethod
     def from_packed(cls, pools: dict, num_experts: int, hidden_size: int, intermediate_size: int,
-                    top_k: int, gate_weight=None, renormalize=False, device="cuda"):
+                    top_k: int, gate_weight=None, renormalize=False, device="cuda",
+                    shared_expert: dict | None = None):
         """pools: {bit_str: {"gate_up": packed, "down": packed, "expert_offsets": [E+1]}} in
-        processing order (the ModuleDict order of the reference)."""
+        processing order (the ModuleDict order of the reference).  shared_expert (optional):
+        see attach_shared_expert."""
         moe = cls(num_experts, hidden_size, intermediate_size, top_k, gate_weight, renormalize, device)
         for bit_str, p in pools.items():
             bit = int(bit_str)
@@ -151,7 +159,69 @@ class WxA16BitPartitionedGroupMoE:
             if homes != 1:
                 raise ValueError(f"expert {ex} belongs to {homes} bit pools; this build handles "
                                  "layers whose experts live in exactly one pool")
+        if shared_expert is not None:
+            moe.attach_shared_expert(shared_expert)
         return moe
+
+    def attach_shared_expert(self, shared: dict):
+        """Add the always-on shared expert of the reference layer
+        (``final += shared_expert(x) * sigmoid(shared_expert_gate(x))``,
+        quantization/wxa16/bit_partitioned_moe.py:1101-1106).
+
+        shared = {"gate": packed, "up": packed, "down": packed, "gate_row": fp16 [1, H] or [H]}:
+        the three quantized Linears of the shared MLP in the row-major packed format of
+        WxA16Linear (quantization/wxa16/linear.py:27-80; all three share bit width, codebook and
+        seed, dartmoq_utils.py:884) and the weight of the sigmoid gate.  The shared width must be a
+        multiple of the routed experts' width I: the neurons are cut into I_s / I slices which
+        join the routed path as extra experts E, E+1, ... that every token selects with the gate
+        value as its routing weight, so the shared expert costs no extra launches."""
+        if self.n_shared:
+            raise ValueError("shared expert already attached")
+        if len(self.bit_weights) + 1 > _lib_max_pools():
+            raise ValueError(f"at most {_lib_max_pools()} pools per layer including the shared expert")
+        gate, up, down = shared["gate"], shared["up"], shared["down"]
+        inter = self.intermediate_size
+        i_s, h = (int(v) for v in gate["shape"])
+        if h != self.hidden_size or tuple(up["shape"]) != (i_s, h) or tuple(down["shape"]) != (h, i_s):
+            raise ValueError("shared expert shapes must be gate/up [I_s, H], down [H, I_s]")
+        if i_s % inter:
+            raise ValueError(f"shared intermediate size {i_s} must be a multiple of {inter}")
+        bit = int(gate["bit_width"])
+        if bit not in (1, 2, 4) or int(up["bit_width"]) != bit or int(down["bit_width"]) != bit:
+            raise ValueError(f"shared expert bit_width must be 1/2/4 and equal for gate/up/down, got {bit}")
+        if int(up["seed"]) != int(gate["seed"]):
+            raise ValueError("gate and up of the shared expert must share the rotation seed")
+        if not torch.equal(gate["codebook"].cpu().half(), up["codebook"].cpu().half()):
+            raise ValueError("gate and up of the shared expert must share the codebook")
+        m = i_s // inter
+        # rows of slice v: gate[v*I:(v+1)*I] then up[v*I:(v+1)*I], the layout of a routed expert
+        def interleave(a, b):
+            a = a.reshape(m, inter, -1)
+            b = b.reshape(m, inter, -1)
+            return torch.cat([a, b], dim=1).reshape(2 * i_s, -1).contiguous()
+        gu = dict(gate)
+        gu["indices_packed"] = interleave(gate["indices_packed"], up["indices_packed"])
+        gn, un = gate["norms"], up["norms"]
+        if gn.dim() == 1:
+            gn, un = gn.unsqueeze(1), un.unsqueeze(1)
+        gu["norms"] = interleave(gn, un)
+        gu["shape"] = (2 * i_s, h)
+        e = self.num_experts
+        offs = [0] * (e + 1) + [inter * (v + 1) for v in range(m)]
+        for key, o in self.expert_offsets.items():
+            o.extend([o[-1]] * m)
+            self.bit_weights[key].expert_offsets = list(o)
+        self.bit_weights[self.SHARED_KEY] = BitPoolWeights(bit, gu, dict(down), offs, self.device)
+        self.expert_offsets[self.SHARED_KEY] = offs
+        self.bit_list.append(bit)
+        self.n_shared = m
+        self.shared_intermediate_size = i_s
+        self.shared_gate_row = shared["gate_row"].reshape(-1).to(self.device, torch.float16).contiguous()
+        if self.shared_gate_row.numel() != h:
+            raise ValueError("gate_row must hold hidden_size values")
+        self._desc = None
+        self._workspace = None
+        return self
 
     @classmethod
     def from_reference_module(cls, ref, gate_weight=None, renormalize=False, device="cuda"):
@@ -160,7 +230,9 @@ class WxA16BitPartitionedGroupMoE:
         (indices_packed, norms, codebook, seed, group_size, shape — the WxA16Weights properties,
         quantization/wxa16/bit_partitioned_moe.py:78-150), ``ref.expert_offsets[bit_str]`` the
         E+1 neuron offsets (:324), plus num_experts / hidden_size / intermediate_size / top_k
-        (:290-293).  Tensors are copied to ``device`` once; the reference module is not modified."""
+        (:290-293).  ``ref.shared_expert`` (gate_proj / up_proj / down_proj as WxA16Linear) and
+        ``ref.shared_expert_gate`` (:294-295) are attached when present.  Tensors are copied to
+        ``device`` once; the reference module is not modified."""
         pools = {}
         for bit_str in ref.bit_weights.keys():
             w = ref.bit_weights[bit_str]
@@ -168,9 +240,20 @@ class WxA16BitPartitionedGroupMoE:
             offs = offs.cpu().tolist() if torch.is_tensor(offs) else list(offs)
             pools[str(bit_str)] = {"gate_up": dict(w.gate_up_packed), "down": dict(w.down_packed),
                                    "expert_offsets": offs}
+        shared = None
+        sh, sh_gate = getattr(ref, "shared_expert", None), getattr(ref, "shared_expert_gate", None)
+        if sh is not None and sh_gate is not None:
+            # WxA16Linear buffers (quantization/wxa16/linear.py:66-69) of the shared MLP
+            def packed(lin):
+                return {"indices_packed": lin.packed_indices, "norms": lin.norms,
+                        "codebook": lin.codebook, "seed": int(lin.seed),
+                        "group_size": int(lin.group_size), "bit_width": int(lin.bit_width),
+                        "shape": (int(lin.out_features), int(lin.in_features))}
+            shared = {"gate": packed(sh.gate_proj), "up": packed(sh.up_proj),
+                      "down": packed(sh.down_proj), "gate_row": sh_gate.weight}
         return cls.from_packed(pools, int(ref.num_experts), int(ref.hidden_size),
                                int(ref.intermediate_size), int(ref.top_k), gate_weight, renormalize,
-                               device)
+                               device, shared_expert=shared)
 
     @classmethod
     def from_wxa16(cls, moe: "WxA16BitPartitionedGroupMoE"):
@@ -192,7 +275,8 @@ class WxA16BitPartitionedGroupMoE:
     def _descriptor(self):
         if self._desc is not None:
             return self._desc
-        e = self.num_experts
+        e = self.num_experts + self.n_shared
+        top_k = self.top_k + self.n_shared
         n_pools = len(self.bit_weights)
         start = torch.full((n_pools, e), -1, dtype=torch.int32)
         count = torch.zeros((n_pools, e), dtype=torch.int32)
@@ -212,7 +296,9 @@ class WxA16BitPartitionedGroupMoE:
             d = pool_arr[pi]
             d.bit, d.mode = bw.bit, mode
             # expected routed rows of the pool exceed threshold * T  <=>  share * top_k > threshold
-            d.major = int(members * self.top_k > self.rotation_hoist_threshold * e)
+            # (the shared pool sees every token: rotating by token never does more work)
+            d.major = int(bit_str == self.SHARED_KEY or
+                          members * self.top_k > self.rotation_hoist_threshold * self.num_experts)
             d.n_gate_up, d.down_groups = bw.n_gate_up, bw.down_in // GROUP_SIZE
             d.gu_w, d.gu_norms = ctx["gu_w"].data_ptr(), ctx["gu_norms"].data_ptr()
             d.gu_lut = ctx["gu_lut"].data_ptr() if ctx["gu_lut"] is not None else None
@@ -226,7 +312,7 @@ class WxA16BitPartitionedGroupMoE:
         slice_count = count.to(self.device)
         desc = LayerDesc()
         desc.hidden, desc.inter = self.hidden_size, self.intermediate_size
-        desc.experts, desc.top_k, desc.pools = e, self.top_k, n_pools
+        desc.experts, desc.top_k, desc.pools = e, top_k, n_pools
         desc.pool = ctypes.cast(pool_arr, ctypes.POINTER(PoolDesc))
         desc.slice_start, desc.slice_count = slice_start.data_ptr(), slice_count.data_ptr()
         self._desc = (desc, pool_arr, slice_start, slice_count, keep)
@@ -246,7 +332,18 @@ class WxA16BitPartitionedGroupMoE:
             if self.gate_weight is None:
                 raise ValueError("no gate weight: pass router_logits or topk_idx/topk_w")
             router_logits = torch.matmul(x, self.gate_weight.t().to(x.dtype))
+        if self.n_shared:
+            return ops.route_topk_shared(router_logits, None, None, self.top_k, self.renormalize,
+                                         x, self.shared_gate_row, self.num_experts, self.n_shared)
         return ops.route_topk(router_logits, self.top_k, self.renormalize)
+
+    def widen_topk(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_w: torch.Tensor):
+        """Append the shared-expert columns to a router's own top-k: (weights, indices) of shape
+        [T, top_k + n_shared] (unchanged when the layer has no shared expert)."""
+        if not self.n_shared or topk_idx.shape[-1] == self.top_k + self.n_shared:
+            return topk_w, topk_idx
+        return ops.route_topk_shared(None, topk_idx, topk_w, self.top_k, False, x,
+                                     self.shared_gate_row, self.num_experts, self.n_shared)
 
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None,
@@ -263,6 +360,8 @@ class WxA16BitPartitionedGroupMoE:
         tokens = x.shape[0]
         if topk_idx is None:
             topk_w, topk_idx = self.route(x, router_logits)
+        else:
+            topk_w, topk_idx = self.widen_topk(x, topk_idx, topk_w)
         topk_idx = topk_idx.to(torch.int32).contiguous()
         topk_w = topk_w.float().contiguous()
         desc = self._descriptor()[0]
@@ -287,7 +386,7 @@ class WxA16BitPartitionedGroupMoE:
         return 3 * h * i * bit // 8 + 6 * h * i // GROUP_SIZE
 
     def flops_per_token(self) -> int:
-        return self.top_k * 6 * self.hidden_size * self.intermediate_size
+        return 6 * self.hidden_size * (self.top_k * self.intermediate_size + self.shared_intermediate_size)
 
 
 class WxA8BitPartitionedGroupMoE(WxA16BitPartitionedGroupMoE):
@@ -374,6 +473,7 @@ def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: 
     fused), combine (the add of the scattered rows)."""
     x = x.half().contiguous()
     tokens = x.shape[0]
+    topk_w, topk_idx = moe.widen_topk(x, topk_idx.to(torch.int32).contiguous(), topk_w.float().contiguous())
     topk_idx = topk_idx.to(torch.int32).contiguous()
     topk_w = topk_w.float().contiguous()
     desc = moe._descriptor()[0]
@@ -397,7 +497,7 @@ def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: 
     if profile:
         for i, name in enumerate(STAGE_NAMES):
             stats[name] = events[i].elapsed_time(events[i + 1])
-    counts = ws[aux[2]:aux[2] + 4 * moe.num_experts].view(torch.int32).clone()
+    counts = ws[aux[2]:aux[2] + 4 * (moe.num_experts + moe.n_shared)].view(torch.int32).clone()
     n_items = int(ws[aux[4]:aux[4] + 4].view(torch.int32).item())
     return out, stats, {"counts": counts, "tt": int(aux[0]), "ks": int(aux[1]), "nbl": int(aux[5]),
                         "n_items": n_items}

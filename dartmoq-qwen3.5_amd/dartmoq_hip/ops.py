@@ -114,6 +114,41 @@ def route_topk(logits: torch.Tensor, top_k: int, renormalize: bool = False):
     return w, idx
 
 
+def route_topk_shared(logits, topk_idx, topk_w, top_k: int, renormalize: bool, x: torch.Tensor,
+                      gate_row: torch.Tensor, num_experts: int, n_shared: int):
+    """Top-k (from ``logits``, or copied from ``topk_idx`` / ``topk_w`` when logits is None) widened
+    by ``n_shared`` always-on columns: index num_experts + j, weight sigmoid(x . gate_row)."""
+    _need_cuda(x, gate_row)
+    if x.dtype != torch.float16 or gate_row.dtype != torch.float16:
+        raise TypeError("x and gate_row must be fp16")
+    x = x.contiguous()
+    gate_row = gate_row.contiguous().reshape(-1)
+    t, h = x.shape
+    if gate_row.numel() != h:
+        raise ValueError("gate_row must hold hidden values")
+    w = torch.empty((t, top_k + n_shared), dtype=torch.float32, device=x.device)
+    idx = torch.empty((t, top_k + n_shared), dtype=torch.int32, device=x.device)
+    if logits is not None:
+        _need_cuda(logits)
+        if logits.dtype not in (torch.float32, torch.float16):
+            logits = logits.float()
+        logits = logits.contiguous()
+        if logits.shape != (t, num_experts):
+            raise ValueError("logits must be [tokens, num_experts]")
+        args = (_ptr(logits), int(logits.dtype == torch.float16), None, None)
+    else:
+        _need_cuda(topk_idx, topk_w)
+        topk_idx = topk_idx.to(torch.int32).contiguous()
+        topk_w = topk_w.float().contiguous()
+        if topk_idx.shape != (t, top_k) or topk_w.shape != (t, top_k):
+            raise ValueError("topk_idx / topk_w must be [tokens, top_k]")
+        args = (None, 0, _ptr(topk_idx), _ptr(topk_w))
+    check(load().dmq_route_topk_shared(*args, t, num_experts, top_k, int(renormalize), _ptr(x),
+                                       _ptr(gate_row), h, n_shared, _ptr(w), _ptr(idx),
+                                       _stream(x.device)), "route_topk_shared")
+    return w, idx
+
+
 def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_rows=16):
     """Device-side sort + pool partition.  Returns a dict of int32/fp32 device tensors."""
     _need_cuda(topk_idx, topk_w, slice_start, slice_count)

@@ -48,7 +48,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 4). */
+/* Library / build identification: returns the ABI version (currently 5). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -89,6 +89,20 @@ int dmq_fold_indices_to_e2m1(const void* idx_gf, const void* nib_lut, long rows,
  * out_idx int32 [tokens, k].  experts <= 1024, k <= 64. */
 int dmq_route_topk(const void* logits, int logits_fp16, int tokens, int experts, int k,
                    int renorm, void* out_w, void* out_idx, void* stream);
+
+/* The same top-k widened by the always-on shared expert of
+ * quantization/wxa16/bit_partitioned_moe.py:1101-1106: the shared expert is handed to the routed
+ * path as n_shared extra experts that every token selects (its intermediate neurons cut into
+ * n_shared slices of the routed experts' width), so out_w / out_idx are [tokens, k + n_shared]
+ * with out_idx[t, k + j] = experts + j and out_w[t, k + j] = sigmoid(x[t] . gate_row) -- the
+ * torch.sigmoid(self.shared_expert_gate(x)) factor, rounded to fp16 after the dot product and
+ * after the sigmoid.  With logits == NULL the first k columns are copied from topk_idx_in int32 /
+ * topk_w_in fp32 [tokens, k] (a router that already returned its top-k).  x fp16 [tokens, hidden],
+ * gate_row fp16 [hidden], hidden % 8 == 0, n_shared <= 64. */
+int dmq_route_topk_shared(const void* logits, int logits_fp16, const void* topk_idx_in,
+                          const void* topk_w_in, int tokens, int experts, int k, int renorm,
+                          const void* x_f16, const void* gate_row_f16, int hidden, int n_shared,
+                          void* out_w, void* out_idx, void* stream);
 
 /* Sort / bincount / pool partition of bit_partitioned_moe.py:1125-1138 and
  * _merged_pools / _merged_expert_info_rows / _merged_expert_info_groups (:1014-1057) and

@@ -12,7 +12,8 @@ def pools_dict(layer):
 def make_module(layer, mode="wxa16", device="cuda"):
     import dartmoq_hip
     moe = dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
-        pools_dict(layer), layer.num_experts, layer.hidden, layer.inter, layer.top_k, device=device)
+        pools_dict(layer), layer.num_experts, layer.hidden, layer.inter, layer.top_k, device=device,
+        shared_expert=layer.shared)
     return dartmoq_hip.convert_moe(moe, mode) if mode != "wxa16" else moe
 
 

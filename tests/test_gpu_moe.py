@@ -97,6 +97,74 @@ def test_layer_routes_from_logits(small_layer):
     assert relerr(out, ideal) < 3e-3
 
 
+@pytest.fixture(scope="module")
+def shared_layer(small_layer):
+    """small_layer plus an always-on shared expert twice as wide as a routed expert (bit 4)."""
+    import dataclasses
+    return moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), 2 * small_layer.inter,
+                                 seed=77)
+
+
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
+@pytest.mark.parametrize("tokens,tt", [(1, 0), (50, 0), (200, 2)])
+def test_layer_with_shared_expert(shared_layer, mode, tokens, tt):
+    """Routed experts + shared_expert(x) * sigmoid(shared_expert_gate(x)): the shared expert runs
+    as two always-on slices inside the routed launches."""
+    layer = shared_layer
+    x, idx, w, out = _run(layer, mode, tokens, seed=5 + tokens, tt=tt)
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    ref = moe.reference_forward(layer, x, idx, w)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+    assert relerr(out, ref) < MODE_BOUND[mode], (mode, relerr(out, ref))
+    # the shared expert is a visible part of the output
+    routed_only = moe.quantized_forward(dataclasses_replace_shared(layer), x, idx, w, mode)
+    assert relerr(routed_only, ideal) > 0.1
+
+
+def dataclasses_replace_shared(layer):
+    import dataclasses
+    return dataclasses.replace(layer, shared=None)
+
+
+def test_shared_expert_from_logits_and_gate_columns(shared_layer):
+    """Widened top-k: columns k.. name experts E, E+1 with the fp16 sigmoid gate as weight; the
+    forward from logits equals the forward from the router's own top-k."""
+    import dartmoq_hip
+    from dartmoq_hip import ops
+    layer = shared_layer
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(37, layer.hidden, generator=g).half()
+    logits = routing.zipf_logits(37, layer.num_experts, 12)
+    w, idx = routing.route_topk(logits, layer.top_k)
+    mod = make_module(layer, "wxa16")
+    assert mod.n_shared == 2
+    ww, wi = ops.route_topk_shared(logits.cuda(), None, None, layer.top_k, False, x.cuda(),
+                                   mod.shared_gate_row, layer.num_experts, mod.n_shared)
+    k = layer.top_k
+    assert torch.equal(wi[:, :k].cpu().long(), idx.long())
+    torch.testing.assert_close(ww[:, :k].cpu(), w.float(), rtol=1e-5, atol=1e-7)
+    assert torch.equal(wi[:, k:].cpu(), torch.tensor([[layer.num_experts, layer.num_experts + 1]] * 37,
+                                                     dtype=torch.int32))
+    gate = moe.shared_gate_value(layer, x)
+    # one fp16 ulp of slack: the dot product is summed in another order
+    torch.testing.assert_close(ww[:, k:].cpu(), gate.expand(37, 2), rtol=2e-3, atol=0)
+    ww2, wi2 = ops.route_topk_shared(None, idx.cuda().int(), w.cuda(), k, False, x.cuda(),
+                                     mod.shared_gate_row, layer.num_experts, mod.n_shared)
+    assert torch.equal(wi2, wi) and torch.equal(ww2[:, k:], ww[:, k:])
+    a = mod.forward(x.cuda(), router_logits=logits.cuda())
+    b = mod.forward(x.cuda(), topk_idx=wi[:, :k].contiguous(), topk_w=ww[:, :k].contiguous())
+    assert torch.equal(a, b)
+
+
+def test_shared_expert_shape_errors(small_layer):
+    import dataclasses
+    bad = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter + 128,
+                                seed=3)
+    with pytest.raises(ValueError):
+        make_module(bad, "wxa16")
+
+
 def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):

@@ -16,6 +16,7 @@ E2M1_GRID = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
 FP4_BITS = (1, 4)            # pools that run on the MX fp4 path in wxfp4 mode (bit 2 stays int8)
 
 _ROT_CACHE: dict[tuple[int, int], torch.Tensor] = {}
+_BATCH_CACHE: dict[tuple, torch.Tensor] = {}
 
 
 def generate_rotation_matrix(d: int, seed: int = 42) -> torch.Tensor:
@@ -37,10 +38,22 @@ def generate_rotation_matrix(d: int, seed: int = 42) -> torch.Tensor:
 
 def generate_batch_rotation_matrices(d: int, seed_base: int, num_groups: int, stride: int,
                                      device=None, dtype=torch.float16) -> torch.Tensor:
-    """[num_groups, d, d], group i seeded seed_base + i*stride (rotation.py:127-173)."""
+    """[num_groups, d, d], group i seeded seed_base + i*stride (rotation.py:127-173).  Batches of
+    up to 64 matrices (the per-call rotations of the Linear path) are kept per device like the
+    reference's batch cache; the large per-pool batches are owned by their modules instead."""
+    key = (int(d), int(seed_base), int(num_groups), int(stride), str(device), str(dtype))
+    hit = _BATCH_CACHE.get(key)
+    if hit is not None:
+        return hit
     mats = torch.stack([generate_rotation_matrix(d, seed_base + i * stride).to(dtype)
                         for i in range(num_groups)], 0).contiguous()
-    return mats if device is None else mats.to(device)
+    if device is not None:
+        mats = mats.to(device)
+    if num_groups <= 64:
+        if len(_BATCH_CACHE) >= 512:
+            _BATCH_CACHE.pop(next(iter(_BATCH_CACHE)))
+        _BATCH_CACHE[key] = mats
+    return mats
 
 
 def build_int8_codebook(codebook: torch.Tensor):

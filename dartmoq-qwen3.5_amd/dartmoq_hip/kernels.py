@@ -183,6 +183,72 @@ def triton_fused_matmul_merged_in_features_gf(x_rot, indices_packed_gf, codebook
     return out if orig == torch.float16 else out.to(orig)
 
 
+# Row-major (checkpoint layout) callables of the Linear path.  The kernels read the group-first
+# layout only, so these convert on first sight of a weight tensor and keep the converted copy while
+# the source tensor is alive and unmodified; modules that own their weights (dartmoq_hip.linear)
+# convert once at load and do not come through here.
+_GF_CACHE: dict[tuple, tuple] = {}
+
+
+def _group_first_cached(indices_packed, norms, group_size, bit_width):
+    if norms.dim() == 1:
+        norms = norms.unsqueeze(1)
+    key = (indices_packed.data_ptr(), norms.data_ptr(), tuple(indices_packed.shape), int(bit_width),
+           indices_packed._version, norms._version, str(indices_packed.device))
+    hit = _GF_CACHE.get(key)
+    if hit is None:
+        nh = norms if norms.dtype == torch.float16 else norms.half()
+        hit = ops.convert_to_group_first(indices_packed.contiguous(), nh.contiguous(), group_size,
+                                         bit_width, prescale=True)
+        if len(_GF_CACHE) >= 64:
+            _GF_CACHE.pop(next(iter(_GF_CACHE)))
+        _GF_CACHE[key] = hit
+    return hit
+
+
+def triton_fused_matmul_grouped(x, indices_packed, codebook, norms, seed, group_size, in_features,
+                                bit_width: int = 4):
+    """triton_kernels.py:600-684, the kernel of WxA16Linear.forward: x[B, K] times the whole packed
+    matrix [N, K*bit/8] (row-major), group g rotated with seed + g*group_size.  in_features must
+    be a multiple of the group size (the reference's per-group fallback for ragged K is not built)."""
+    _check_bit(bit_width, {1, 2, 4}, "matmul_grouped")
+    _check_gs(group_size)
+    if in_features % group_size:
+        raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
+    idx_gf, norms_gf = _group_first_cached(indices_packed, norms, group_size, bit_width)
+    return triton_fused_matmul_grouped_slice_rows_gf(
+        x, idx_gf, codebook, norms_gf, seed, group_size, in_features, 0, indices_packed.shape[0],
+        bit_width, norms_prescaled=True)
+
+
+def triton_fused_matmul_grouped_slice_rows(x, indices_packed, codebook, norms, seed, group_size,
+                                           in_features, row_start, row_end, bit_width: int = 4):
+    """triton_kernels.py:686-771: output rows [row_start, row_end) of a row-major packed matrix."""
+    _check_bit(bit_width, {1, 2, 4}, "slice_rows")
+    _check_gs(group_size)
+    if in_features % group_size:
+        raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
+    idx_gf, norms_gf = _group_first_cached(indices_packed, norms, group_size, bit_width)
+    return triton_fused_matmul_grouped_slice_rows_gf(
+        x, idx_gf, codebook, norms_gf, seed, group_size, in_features, row_start, row_end, bit_width,
+        norms_prescaled=True)
+
+
+def triton_fused_matmul_grouped_slice_in_features(x, indices_packed, codebook, norms, seed,
+                                                  group_size, original_start, original_end,
+                                                  full_in_features, bit_width: int = 4):
+    """triton_kernels.py:774-860: input features [original_start, original_end) of a row-major
+    packed matrix; x[B, end-start] is rotated with seed + original_start."""
+    _check_bit(bit_width, {1, 2, 4}, "slice_in_features")
+    _check_gs(group_size)
+    if original_start % group_size:
+        raise ValueError(f"original_start ({original_start}) must be aligned to group_size ({group_size})")
+    idx_gf, norms_gf = _group_first_cached(indices_packed, norms, group_size, bit_width)
+    return triton_fused_matmul_grouped_slice_in_features_gf(
+        x, idx_gf, codebook, norms_gf, seed, group_size, original_start, original_end,
+        full_in_features, bit_width, norms_prescaled=True)
+
+
 # ----------------------------------------------------------------------------- activation quantizers
 
 def rotate_quantize_fused(x, rot, group_size, num_groups, extra_scale: float = 1.0):
@@ -299,6 +365,27 @@ def wxa8_matmul_merged_in_features_gf(x_i8, x_scale, indices_packed_gf, codebook
     return _qa_merged(MODE_A8, "wxa8 merged_in_features", False, x_i8, x_scale.half(),
                       indices_packed_gf, codebook_i8, norms_gf, expert_info, group_size, 0, bit_width,
                       norms_prescaled, cfg)
+
+
+def wxa8_matmul_grouped_gf(x_i8, x_scale, indices_packed_gf, codebook_i8, norms_gf, group_size,
+                           num_groups, bit_width: int = 8, identity_cb: bool = False, cfg=None):
+    """triton_kernels_a8.py:769-799, the kernel of WxA8Linear.forward: the whole matrix, norms_gf
+    already divided by sqrt(group_size).  The 8-bit uniform codebook (identity_cb) of the attention
+    Linears is not built: bit widths 1/2/4 with an int8 look-up table only."""
+    if identity_cb or bit_width == 8:
+        raise ValueError("wxa8_matmul_grouped_gf: the 8-bit identity codebook is not built; "
+                         "bit_width must be 1/2/4")
+    return _qa_slice_rows(MODE_A8, "wxa8 grouped", x_i8, x_scale.half(), indices_packed_gf,
+                          codebook_i8, norms_gf, group_size, num_groups * group_size, 0,
+                          indices_packed_gf.shape[1], bit_width, True)
+
+
+def wxfp8_matmul_grouped_gf(x_f8, x_scale, indices_packed_gf, cb_f8, norms_gf, group_size,
+                            num_groups, bit_width: int, cfg=None):
+    """triton_kernels_fp8.py:407-428: the whole matrix (WxFP8Linear.forward); bit widths 1/2/4."""
+    return _qa_slice_rows(MODE_FP8, "wxfp8 grouped", x_f8, x_scale.half(), indices_packed_gf, cb_f8,
+                          norms_gf, group_size, num_groups * group_size, 0,
+                          indices_packed_gf.shape[1], bit_width, True)
 
 
 def wxfp8_matmul_grouped_slice_rows_gf(x_f8, x_scale, indices_packed_gf, cb_f8, norms_gf, group_size,

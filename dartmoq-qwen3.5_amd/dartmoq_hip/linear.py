@@ -1,0 +1,156 @@
+"""Quantized Linear layers on MI355X: WxA16Linear and its WxA8 / WxFP8 variants.
+
+Host-side mirror of quantization/wxa16/linear.py:27-260 (WxA16Linear: row-major packed indices,
+fp16 norms [N, G], fp16 codebook, one rotation seed; forward = triton_fused_matmul_grouped),
+quantization/wxa8/linear.py:79-159 (fused rotate + int8 quantize, integer GEMM) and
+quantization/wxfp8/linear.py:37-100 (e4m3 activations and look-up table).  These are the Linears
+of the shared expert of the MoE layer.  Like the reference's WxA8Linear._ensure_gf the module
+converts the checkpoint layout to group-first once (norms divided by sqrt(128)) and keeps the
+rotation matrices and the per-mode look-up table resident; a forward is two launches (rotate
+(+quantize), dequant GEMM) on the current stream.
+
+Bit widths 1, 2 and 4 with a codebook look-up are built.  The 8-bit uniform codebook of the
+attention Linears (bit_width 8, codebook_type "uniform") is not: constructing such a layer raises
+ValueError.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import hostprep, ops
+from ._lib import EPI_STORE, MODE_A16, MODE_A8, MODE_FP8
+
+GROUP_SIZE = ops.GROUP_SIZE
+
+
+class WxA16Linear:
+    MODE = MODE_A16
+
+    def __init__(self, in_features: int, out_features: int, bit_width: int, group_size: int,
+                 packed_indices: torch.Tensor, codebook: torch.Tensor, norms: torch.Tensor, seed: int,
+                 rotation: str = "qr", bias=None, orig_dtype: torch.dtype = torch.float16,
+                 codebook_type: str = "lloydmax", device="cuda"):
+        if bit_width not in (1, 2, 4):
+            raise ValueError(f"bit_width must be 1/2/4, got {bit_width}")
+        if group_size != GROUP_SIZE:
+            raise ValueError(f"group_size must be {GROUP_SIZE}, got {group_size}")
+        if in_features % group_size:
+            raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
+        if rotation != "qr":
+            raise ValueError(f"rotation must be 'qr', got {rotation!r}")
+        self.in_features, self.out_features = int(in_features), int(out_features)
+        self.bit_width, self.group_size = int(bit_width), int(group_size)
+        self.seed = int(seed.item()) if isinstance(seed, torch.Tensor) else int(seed)
+        self.rotation, self.orig_dtype, self.codebook_type = rotation, orig_dtype, codebook_type
+        self.device = torch.device(device)
+        self.n_groups = self.in_features // self.group_size
+        ppg = self.group_size * self.bit_width // 8
+        if tuple(packed_indices.shape) != (self.out_features, self.n_groups * ppg):
+            raise ValueError(f"packed_indices must be {(self.out_features, self.n_groups * ppg)}, "
+                             f"got {tuple(packed_indices.shape)}")
+        if norms.dim() == 1:
+            norms = norms.unsqueeze(1)
+        if tuple(norms.shape) != (self.out_features, self.n_groups):
+            raise ValueError(f"norms must be {(self.out_features, self.n_groups)}, got {tuple(norms.shape)}")
+        self.codebook = codebook.to(self.device, torch.float16).contiguous()
+        self.bias = None if bias is None else bias.to(self.device)
+        # group-first relayout, norms / sqrt(gs): the row-major originals are not kept on the device
+        self.indices_gf, self.norms_gf = ops.convert_to_group_first(
+            packed_indices.to(self.device).contiguous(), norms.to(self.device).half().contiguous(),
+            self.group_size, self.bit_width, prescale=True)
+        self.rot = hostprep.generate_batch_rotation_matrices(self.group_size, self.seed, self.n_groups,
+                                                             self.group_size, self.device)
+        self._ctx: dict[int, tuple] = {}
+        self._info: dict[int, torch.Tensor] = {}
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_packed(cls, packed: dict, bias=None, device="cuda"):
+        """packed: the dictionary turboquant_quantize_packed_full returns (quantize.py:350-474):
+        indices_packed, norms, codebook, seed, group_size, shape, bit_width."""
+        n, k = (int(v) for v in packed["shape"])
+        return cls(k, n, int(packed["bit_width"]), int(packed["group_size"]), packed["indices_packed"],
+                   packed["codebook"], packed["norms"], packed["seed"],
+                   rotation=packed.get("rotation", "qr"), bias=bias,
+                   codebook_type=packed.get("codebook_type", "lloydmax"), device=device)
+
+    @classmethod
+    def from_reference_module(cls, lin, device="cuda"):
+        """Build from a loaded WxA16Linear of the reference (duck-typed buffers and attributes,
+        quantization/wxa16/linear.py:54-80); the module is not modified."""
+        return cls(lin.in_features, lin.out_features, lin.bit_width, lin.group_size, lin.packed_indices,
+                   lin.codebook, lin.norms, lin.seed, rotation=getattr(lin, "rotation", "qr"),
+                   bias=getattr(lin, "bias", None),
+                   orig_dtype=getattr(lin, "orig_dtype", torch.float16),
+                   codebook_type=getattr(lin, "codebook_type", "lloydmax"), device=device)
+
+    @classmethod
+    def from_wxa16(cls, linear: "WxA16Linear"):
+        """Switch a loaded layer to this precision mode in place (no tensor copies), like
+        WxA8Linear.from_wxa16 (quantization/wxa8/linear.py:79-98)."""
+        if not isinstance(linear, WxA16Linear):
+            raise TypeError(f"expected WxA16Linear, got {type(linear)}")
+        linear.__class__ = cls
+        return linear
+
+    # ------------------------------------------------------------------ forward
+    def _mode_ctx(self):
+        """(look-up table, activation extra scale) of this precision mode, built on first use."""
+        ctx = self._ctx.get(self.MODE)
+        if ctx is None:
+            if self.MODE == MODE_A16:
+                ctx = (self.codebook, 1.0)
+            elif self.MODE == MODE_A8:
+                q, step = hostprep.build_int8_codebook(self.codebook)
+                ctx = (q.to(self.device), step)
+            else:
+                q, scale = hostprep.build_fp8_codebook(self.codebook)
+                ctx = (q.to(self.device), scale)
+            self._ctx[self.MODE] = ctx
+        return ctx
+
+    def _expert_info(self, rows: int) -> torch.Tensor:
+        info = self._info.get(rows)
+        if info is None:
+            if len(self._info) >= 64:
+                self._info.pop(next(iter(self._info)))
+            info = torch.tensor([[0, rows, 0, self.out_features]], dtype=torch.int32, device=self.device)
+            self._info[rows] = info
+        return info
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if not x.is_cuda:
+            raise RuntimeError("dartmoq_hip layers run on the GPU only (no CPU fallback)")
+        shape = x.shape
+        if shape[-1] != self.in_features:
+            raise ValueError(f"expected {self.in_features} input features, got {shape[-1]}")
+        x2 = x.reshape(-1, self.in_features)
+        src = x2 if x2.dtype == torch.float16 else x2.half()
+        rows = src.shape[0]
+        lut, extra = self._mode_ctx()
+        codes, scale = ops.rotate(self.MODE, src, self.rot, extra_scale=extra, scale_fp32=False)
+        out = ops.matmul_merged(self.MODE, self.bit_width, EPI_STORE, codes,
+                                None if self.MODE == MODE_A16 else scale, self.indices_gf,
+                                self.norms_gf, lut, self._expert_info(rows), groups=self.n_groups,
+                                n_out=self.out_features, slice_is_groups=False, rows_total=rows)
+        if self.bias is not None:
+            out = out + self.bias.to(out.dtype)
+        return out.reshape(*shape[:-1], self.out_features).to(x.dtype)
+
+    __call__ = forward
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, "
+                f"bit_width={self.bit_width}, group_size={self.group_size}, rotation={self.rotation}")
+
+
+class WxA8Linear(WxA16Linear):
+    """int8 activations per token and group, int8 codebook look-up, i32 accumulation."""
+    MODE = MODE_A8
+
+
+class WxFP8Linear(WxA16Linear):
+    """e4m3 activations per token and group, e4m3 codebook look-up, fp32 accumulation."""
+    MODE = MODE_FP8

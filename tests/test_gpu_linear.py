@@ -1,0 +1,149 @@
+"""GPU parity: quantized Linear layers (the Linears of the shared expert) and the un-sliced
+callables of the reference's Linear path, against the CPU oracle.
+
+fp32 reference: x @ dequantize(W)^T (WxA16Linear.dequantize, quantization/wxa16/linear.py:160-221).
+WxA16 is held to the north-star bound (max relative error <= 1e-2, cosine >= 0.9999); the
+activation-quantized modes are compared with the oracle's restatement of their dataflow.
+"""
+
+import pytest
+import torch
+
+from oracle import moe, turboquant
+from oracle.rotation import batch_rotation_matrices, rotate_with
+from tests.helpers import cosine, max_rel, relerr
+
+pytestmark = pytest.mark.gpu
+
+
+def _packed(n, k, bit, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(n, k, generator=g) * 0.02).half()
+    return turboquant.quantize_packed(w, bit, 128, seed=seed + 5)
+
+
+def _dataflow(packed, x, mode):
+    gs = packed["group_size"]
+    n, k = packed["shape"]
+    w_lut, norms, extra, wbs = moe._lut_weights(packed, mode)
+    rot = batch_rotation_matrices(gs, packed["seed"], k // gs, gs, torch.float16)
+    codes, scale = moe.quantize_activation(rotate_with(x.half(), rot, torch.float32), mode, gs, extra)
+    return moe.lut_gemm(codes, scale, w_lut, norms, gs, wbs)
+
+
+@pytest.mark.parametrize("bit", [1, 2, 4])
+@pytest.mark.parametrize("rows", [1, 33, 300])
+def test_wxa16_linear_matches_dequantized_matmul(bit, rows):
+    import dartmoq_hip
+    packed = _packed(384, 512, bit, seed=bit)
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed)
+    x = torch.randn(rows, 512, generator=torch.Generator().manual_seed(rows)).half()
+    out = lin(x.cuda()).float().cpu()
+    ref = x.float() @ turboquant.dequantize_packed(packed).T
+    assert out.shape == (rows, 384)
+    assert relerr(out, ref) < 2e-3
+    assert max_rel(out, ref) <= 1e-2 and cosine(out, ref) >= 0.9999
+    assert relerr(out, _dataflow(packed, x, "wxa16")) < 1.5e-3
+
+
+@pytest.mark.parametrize("mode,cls,tight", [("wxa8", "WxA8Linear", 6e-3), ("wxfp8", "WxFP8Linear", 2e-2)])
+def test_quantized_activation_linears(mode, cls, tight):
+    import dartmoq_hip
+    packed = _packed(256, 640, 4, seed=9)
+    lin = getattr(dartmoq_hip, cls).from_wxa16(dartmoq_hip.WxA16Linear.from_packed(packed))
+    x = torch.randn(70, 640, generator=torch.Generator().manual_seed(4)).half()
+    out = lin(x.cuda()).float().cpu()
+    assert relerr(out, _dataflow(packed, x, mode)) < tight
+    ref = x.float() @ turboquant.dequantize_packed(packed).T
+    assert relerr(out, ref) < {"wxa8": 0.02, "wxfp8": 0.075}[mode]
+
+
+def test_linear_bias_shapes_and_dtypes():
+    import dartmoq_hip
+    packed = _packed(128, 256, 2, seed=3)
+    bias = torch.linspace(-1, 1, 128).half()
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed, bias=bias)
+    x = torch.randn(2, 5, 256, generator=torch.Generator().manual_seed(8))
+    ref = x.reshape(-1, 256).half().float() @ turboquant.dequantize_packed(packed).T + bias.float()
+    out = lin(x.cuda().bfloat16())
+    assert out.dtype == torch.bfloat16 and out.shape == (2, 5, 128)
+    assert relerr(out.float().cpu().reshape(-1, 128), ref) < 1e-2       # bf16 in and out
+    out16 = lin(x.cuda().half())
+    assert relerr(out16.float().cpu().reshape(-1, 128), ref) < 2e-3
+    with pytest.raises(ValueError):
+        lin(torch.zeros(3, 128, dtype=torch.float16, device="cuda"))
+    with pytest.raises(RuntimeError):
+        lin(torch.zeros(3, 256, dtype=torch.float16))
+
+
+def test_linear_constructor_errors():
+    import dartmoq_hip
+    packed = _packed(128, 256, 2, seed=3)
+    with pytest.raises(ValueError):
+        dartmoq_hip.WxA16Linear(256, 128, 8, 128, packed["indices_packed"], packed["codebook"],
+                                packed["norms"], 1)
+    with pytest.raises(ValueError):
+        dartmoq_hip.WxA16Linear(256, 128, 2, 64, packed["indices_packed"], packed["codebook"],
+                                packed["norms"], 1)
+    with pytest.raises(ValueError):
+        dartmoq_hip.WxA16Linear(256, 64, 2, 128, packed["indices_packed"], packed["codebook"],
+                                packed["norms"], 1)
+    with pytest.raises(TypeError):
+        dartmoq_hip.WxA8Linear.from_wxa16(object())
+
+
+def test_reference_module_duck_typing():
+    import types
+    import dartmoq_hip
+    packed = _packed(128, 256, 4, seed=6)
+    ref_lin = types.SimpleNamespace(
+        in_features=256, out_features=128, bit_width=4, group_size=128,
+        packed_indices=packed["indices_packed"], codebook=packed["codebook"], norms=packed["norms"],
+        seed=torch.tensor(packed["seed"]), rotation="qr", bias=None, orig_dtype=torch.float16,
+        codebook_type="lloydmax")
+    a = dartmoq_hip.WxA16Linear.from_reference_module(ref_lin)
+    b = dartmoq_hip.WxA16Linear.from_packed(packed)
+    x = torch.randn(9, 256, generator=torch.Generator().manual_seed(1)).half().cuda()
+    assert torch.equal(a(x), b(x))
+
+
+def test_unsliced_callables_by_reference_names():
+    """triton_fused_matmul_grouped and its row-major slice variants; wxa8 / wxfp8 grouped_gf."""
+    from dartmoq_hip import kernels as K
+    packed = _packed(256, 512, 2, seed=11)
+    w = turboquant.dequantize_packed(packed)
+    x = torch.randn(40, 512, generator=torch.Generator().manual_seed(3)).half()
+    dev = lambda t: t.cuda()
+    ip, cb, nm = dev(packed["indices_packed"]), dev(packed["codebook"]), dev(packed["norms"])
+    out = K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, 512, 2)
+    assert relerr(out.float().cpu(), x.float() @ w.T) < 2e-3
+    # second call hits the converted-layout cache and gives the same bits
+    assert torch.equal(out, K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, torch.tensor(packed["seed"]),
+                                                          128, 512, 2))
+    rows = K.triton_fused_matmul_grouped_slice_rows(x.cuda(), ip, cb, nm, packed["seed"], 128, 512, 64, 192, 2)
+    assert torch.equal(rows, out[:, 64:192])
+    xs = x[:, 128:384].contiguous()
+    part = K.triton_fused_matmul_grouped_slice_in_features(xs.cuda(), ip, cb, nm, packed["seed"], 128,
+                                                           128, 384, 512, 2)
+    assert relerr(part.float().cpu(), xs.float() @ w[:, 128:384].T) < 2e-3
+    with pytest.raises(ValueError):
+        K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, 512, 8)
+    with pytest.raises(ValueError):
+        K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, 500, 2)
+    with pytest.raises(ValueError):
+        K.triton_fused_matmul_grouped_slice_in_features(xs.cuda(), ip, cb, nm, packed["seed"], 128, 64, 320,
+                                                        512, 2)
+
+    idx_gf, norms_gf = K.convert_to_group_first(ip, nm, 128, 2)
+    norms_pre = (norms_gf.float() / 128 ** 0.5).half()
+    rot = K.generate_batch_rotation_matrices(128, packed["seed"], 4, 128, device="cuda")
+    cb_i8, step = K.build_int8_codebook(packed["codebook"])
+    x_i8, x_s = K.rotate_quantize_fused(x.cuda(), rot, 128, 4, extra_scale=step)
+    o8 = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, cb_i8.cuda(), norms_pre, 128, 4, 2)
+    assert relerr(o8.float().cpu(), _dataflow(packed, x, "wxa8")) < 6e-3
+    with pytest.raises(ValueError):
+        K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, cb_i8.cuda(), norms_pre, 128, 4, 8, identity_cb=True)
+    cb_f8, sc = K.build_fp8_codebook(packed["codebook"])
+    x_f8, x_s8 = K.rotate_quantize_fused_fp8(x.cuda(), rot, 128, 4, extra_scale=sc)
+    of8 = K.wxfp8_matmul_grouped_gf(x_f8, x_s8, idx_gf, cb_f8.cuda(), norms_pre, 128, 4, 2)
+    assert relerr(of8.float().cpu(), _dataflow(packed, x, "wxfp8")) < 2e-2

@@ -66,7 +66,7 @@ def time_steps(mods, x, logits, steps, warmup):
 def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     """Throughput of the full layer plus the live timing of its dominant kernel."""
     import torch
-    from dartmoq_hip import ops, synthetic
+    from dartmoq_hip import synthetic
     from dartmoq_hip.moe import forward_staged
     mod = mods[0]
     h, i, k = mod.hidden_size, mod.intermediate_size, mod.top_k
@@ -75,12 +75,11 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     sec = time_steps(mods, x, logits, steps, warmup)
 
     # stage timing (events on the launch stream), rotating the copies like the timed loop
-    topk_w, topk_idx = ops.route_topk(logits, k)
     reps = max(3, min(steps, 20))
     acc = {}
     aux = None
     for r in range(reps + 1):
-        _out, stats, aux = forward_staged(mods[r % len(mods)], x, topk_idx, topk_w)
+        _out, stats, aux = forward_staged(mods[r % len(mods)], x, router_logits=logits)
         if r == 0:
             continue                                   # first pass warms the allocator
         for name, ms in stats.items():

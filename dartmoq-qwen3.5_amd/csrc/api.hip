@@ -34,7 +34,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 5; }
+int dmq_abi_version(void) { return 6; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -135,6 +135,15 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
   plan.slice_start_rows = (const int*)slice_start; plan.slice_count_rows = (const int*)slice_count;
   plan.offsets = (int*)offsets; plan.gu_info = (int*)gu_info; plan.dn_info = (int*)dn_info;
   plan.n_items = (int*)n_items; plan.items = (int*)items;
+  if ((long)tokens * k <= DMQ_ROUTE_SMALL_ROWS && experts <= DMQ_ROUTE_SMALL_EXPERTS && k <= 64) {
+    RouteSmallParams sp{};                   // one launch instead of three
+    sp.in_idx = (const int*)topk_idx; sp.in_w = (const float*)topk_w;
+    sp.tokens = tokens; sp.router_experts = experts; sp.k = k;
+    sp.plan = plan;
+    sp.sorted_tokens = (int*)sorted_tokens; sp.sorted_weights = (float*)sorted_weights;
+    sp.sorted_rows = (int*)sorted_rows;
+    return dmq_route_small_launch(sp, (hipStream_t)stream);
+  }
   return dmq_route_permute_launch((const int*)topk_idx, (const float*)topk_w, tokens, k, plan,
                                   (int*)sorted_tokens, (float*)sorted_weights, (int*)sorted_rows,
                                   (hipStream_t)stream);
@@ -311,6 +320,8 @@ int dmq_fill_zero(void* ptr, long n_bytes, void* stream) {
 // ------------------------------------------------------------------------------- whole layer
 struct MoeWorkspace {
   int *counts, *offsets, *sorted_tokens, *sorted_rows, *gu_info, *dn_info, *n_items, *items;
+  int* topk_idx;                     // [tokens, top_k] incl. the shared columns (routed entry point)
+  float* topk_w;
   float* sorted_weights;
   uint8_t* slots;                    // fp16 [tokens * top_k, hidden]
   uint8_t* xq[DMQ_MAX_POOLS];        // hoisted pools: codes by token; others share xq_rows
@@ -344,6 +355,8 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.sorted_tokens = (int*)take(R * 4);
   w.sorted_rows = (int*)take(R * 4);
   w.sorted_weights = (float*)take(R * 4);
+  w.topk_idx = (int*)take(R * 4);
+  w.topk_w = (float*)take(R * 4);
   w.gu_info = (int*)take(P * E * 16);
   w.dn_info = (int*)take(P * E * 16);
   w.n_items = (int*)take(16);
@@ -383,7 +396,22 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
                                const void* topk_w, int tokens, const void* add_f16, void* out,
                                void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
                                void* const* stage_events, void* aux_out, void* stream) {
-  if (!layer || !x || !topk_idx || !topk_w || !out || !workspace || !layer->pool) return DMQ_ERR_NULL;
+  if (!topk_idx || !topk_w) return DMQ_ERR_NULL;
+  dmq_router_args r{};
+  r.topk_idx = topk_idx; r.topk_w = topk_w;
+  return dmq_moe_ffn_forward_routed(layer, &r, x, tokens, add_f16, out, workspace, workspace_bytes,
+                                    tt, ks, nbl, stage_events, aux_out, stream);
+}
+
+int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_args* router,
+                               const void* x, int tokens, const void* add_f16, void* out,
+                               void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
+                               void* const* stage_events, void* aux_out, void* stream) {
+  if (!layer || !router || !x || !out || !workspace || !layer->pool) return DMQ_ERR_NULL;
+  if (!router->logits && (!router->topk_idx || !router->topk_w)) return DMQ_ERR_NULL;
+  const int n_shared = router->n_shared;
+  if (n_shared < 0 || n_shared >= layer->top_k || n_shared >= layer->experts) return DMQ_ERR_SHAPE;
+  if (n_shared > 0 && !router->shared_gate_row) return DMQ_ERR_NULL;
   auto mark = [&](int i) {
     if (stage_events && stage_events[i]) (void)hipEventRecord((hipEvent_t)stage_events[i], (hipStream_t)stream);
   };
@@ -422,11 +450,46 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
     if (!seen) modes[n_modes++] = m;
   }
 
-  // 1. sort by expert, per-pool expert_info, work items
-  rc = dmq_route_permute(topk_idx, topk_w, tokens, K, E, P, layer->slice_start, layer->slice_count,
-                         w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
-                         w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items, w.items,
-                         w.sort_scratch, w.sort_scratch_bytes, stream);
+  // 1. top-k (when the router hands over logits), shared columns, sort by expert, per-pool
+  //    expert_info, work items: one launch for small batches
+  {
+    const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
+    const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
+    const bool small = (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
+                       K <= 64 && (!router->logits || tokens <= DMQ_ROUTE_SMALL_TOKENS);
+    if (small) {
+      RouteSmallParams sp{};
+      sp.logits = router->logits; sp.logits_fp16 = router->logits_fp16;
+      sp.in_idx = (const int*)router->topk_idx; sp.in_w = (const float*)router->topk_w;
+      sp.tokens = tokens; sp.router_experts = re; sp.k = rk; sp.renorm = router->renorm;
+      sp.sg = sg;
+      sp.out_w = w.topk_w; sp.out_idx = w.topk_idx;
+      PlanParams& plan = sp.plan;
+      plan.counts = w.counts; plan.experts = E; plan.pools = P; plan.tile_rows = w.tile_rows;
+      plan.max_items = w.max_items;
+      plan.slice_start_rows = (const int*)layer->slice_start;
+      plan.slice_count_rows = (const int*)layer->slice_count;
+      plan.offsets = w.offsets; plan.gu_info = w.gu_info; plan.dn_info = w.dn_info;
+      plan.n_items = w.n_items; plan.items = w.items;
+      sp.sorted_tokens = w.sorted_tokens; sp.sorted_weights = w.sorted_weights;
+      sp.sorted_rows = w.sorted_rows;
+      rc = dmq_route_small_launch(sp, st);
+    } else {
+      const void* tk_idx = router->topk_idx;
+      const void* tk_w = router->topk_w;
+      if (router->logits || n_shared > 0) {
+        rc = dmq_route_topk_launch(router->logits, router->logits_fp16, (const int*)router->topk_idx,
+                                   (const float*)router->topk_w, tokens, re, rk, router->renorm,
+                                   w.topk_w, w.topk_idx, sg, st);
+        if (rc) return rc;
+        tk_idx = w.topk_idx; tk_w = w.topk_w;
+      }
+      rc = dmq_route_permute(tk_idx, tk_w, tokens, K, E, P, layer->slice_start, layer->slice_count,
+                             w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
+                             w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items,
+                             w.items, w.sort_scratch, w.sort_scratch_bytes, stream);
+    }
+  }
   if (rc) return rc;
   mark(1);
 

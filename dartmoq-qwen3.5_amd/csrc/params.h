@@ -85,6 +85,28 @@ struct PlanParams {
   int* items;                    // [max_items, DMQ_ITEM_WORDS]
 };
 
+// One-workgroup routing for small batches: top-k (or a copy of the caller's top-k), the shared
+// columns, the stable sort by expert and the work-item list in a single launch.
+#define DMQ_ROUTE_SMALL_ROWS 1024       // routed rows (tokens * (k + n_shared)) it handles
+#define DMQ_ROUTE_SMALL_EXPERTS 512     // experts including the shared slices
+#define DMQ_ROUTE_SMALL_TOKENS 16       // tokens when the top-k is computed inside (one per wave:
+                                        // more would serialize on the one compute unit)
+struct RouteSmallParams {
+  const void* logits;            // [tokens, router_experts] fp32 / fp16, or NULL
+  int logits_fp16;
+  const int* in_idx;             // logits == NULL: top-k of the router [tokens, k]
+  const float* in_w;
+  int tokens, router_experts, k, renorm;
+  SharedGate sg;
+  float* out_w;                  // optional [tokens, k + n_shared]: the widened top-k
+  int* out_idx;
+  PlanParams plan;               // experts = router_experts + n_shared; hist / chunk fields unused
+  int* sorted_tokens;
+  float* sorted_weights;
+  int* sorted_rows;
+};
+int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream);
+
 int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream);
 int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
 int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx, const float* in_w,

@@ -10,18 +10,40 @@
 //   4. dmq_chunk_fill_kernel  one wave per chunk: write its rows to their sorted positions
 //   5. dmq_combine_kernel     out[t] = sum over the k slot rows of token t (fixed order)
 #include "params.h"
+#include <type_traits>
 
 // ------------------------------------------------------------------------------ top-k
+// Wave-wide max / min through data-parallel lane moves: xor 1, xor 2, mirror within 8 and within
+// 16 lanes leave every lane with the result of its row of 16; the four rows are then combined
+// through scalar registers.  The result is uniform over the wave.
+template <typename F>
+__device__ __forceinline__ int wave_reduce_i32(int v, F op) {
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, true));   // row_mirror
+  const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+  const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+  return op(op(a, b), op(c, d));
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+  // finite floats and -inf order like their bit patterns after this monotone map
+  auto key = [](float f) { int b = __builtin_bit_cast(int, f); return b >= 0 ? b : (int)(0x80000000u - (unsigned)b); };
+  const int k = wave_reduce_i32(key(v), [](int x, int y) { return x > y ? x : y; });
+  return __builtin_bit_cast(float, k >= 0 ? k : (int)(0x80000000u - (unsigned)k));
+}
+__device__ __forceinline__ int wave_min_i32(int v) {
+  return wave_reduce_i32(v, [](int x, int y) { return x < y ? x : y; });
+}
+
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
 
 // Always-on shared experts ride the routed path as n_shared extra columns of the top-k arrays:
 // column k + j names expert `experts + j` with weight sigmoid(x . gate_row), rounded to fp16 after
-// the dot and after the sigmoid like an fp16 Linear followed by torch.sigmoid.
-__device__ __forceinline__ void dmq_shared_columns(const SharedGate& sg, int tok, int experts, int k,
-                                                   int lane, float* out_w, int* out_idx) {
-  if (sg.n_shared <= 0) return;
+// the dot and after the sigmoid like an fp16 Linear followed by torch.sigmoid.  Wave-uniform result.
+__device__ __forceinline__ float dmq_shared_gate_value(const SharedGate& sg, int tok, int lane) {
   const __half* xr = sg.x + (long)tok * sg.hidden;
   float dot = 0.f;
   for (int h = lane * 8; h < sg.hidden; h += 512) {
@@ -33,11 +55,88 @@ __device__ __forceinline__ void dmq_shared_columns(const SharedGate& sg, int tok
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) dot += __shfl_xor(dot, m, 64);
   const float z = (float)(_Float16)dot;
-  const float g = (float)(_Float16)(1.f / (1.f + expf(-z)));
+  return (float)(_Float16)(1.f / (1.f + expf(-z)));
+}
+
+__device__ __forceinline__ void dmq_shared_columns(const SharedGate& sg, int tok, int experts, int k,
+                                                   int lane, float* out_w, int* out_idx) {
+  if (sg.n_shared <= 0) return;
+  const float g = dmq_shared_gate_value(sg, tok, lane);
   const int stride = k + sg.n_shared;
   if (lane < sg.n_shared) {
     out_w[(long)tok * stride + k + lane] = g;
     out_idx[(long)tok * stride + k + lane] = experts + lane;
+  }
+}
+
+// softmax + top-k of one token by one wave: lane j < k returns the j-th largest probability and
+// its expert (lowest expert index wins ties).  NV values per lane cover up to 64 * NV experts;
+// the loads are a call of their own so that a caller can request the next token's row early.
+template <typename T, int NV>
+__device__ __forceinline__ void dmq_topk_load(const T* row, int experts, int lane, float (&v)[NV]) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    int e = lane + 64 * i;
+    v[i] = (e < experts) ? to_f32<T>(row[e]) : -INFINITY;
+  }
+}
+
+template <int NV>
+__device__ __forceinline__ void dmq_topk_select(float (&v)[NV], int experts, int k, int renorm, int lane,
+                                                float& my_w, int& my_e) {
+  float vmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) vmax = fmaxf(vmax, v[i]);
+  vmax = wave_max_f32(vmax);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) sum += (lane + 64 * i < experts) ? expf(v[i] - vmax) : 0.f;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) sum += __shfl_xor(sum, m, 64);
+
+  float my_v = -INFINITY;
+  my_e = 0;
+  for (int round = 0; round < k; ++round) {
+    float bv = -INFINITY;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      int e = lane + 64 * i;
+      if (v[i] > bv) { bv = v[i]; be = e; }
+    }
+    // wave arg-max in two reductions: the largest value, then the lowest expert index holding it
+    const float top = wave_max_f32(bv);
+    be = wave_min_i32(bv == top ? be : 0x7fffffff);
+    if (lane == round) { my_v = top; my_e = be; }
+    if ((be & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+        if (i == (be >> 6)) v[i] = -INFINITY;
+    }
+  }
+  // lane j turns the j-th logit into its probability; the kept mass is summed in round order
+  my_w = (lane < k) ? expf(my_v - vmax) / sum : 0.f;
+  if (renorm) {
+    float wsum = 0.f;
+    for (int j = 0; j < k; ++j) wsum += __shfl(my_w, j, 64);
+    my_w = my_w / wsum;
+  }
+}
+
+// The sum of exponentials runs over the same values in the same order for every NV, so the
+// weights do not depend on which instance serves a layer.
+template <typename T>
+__device__ __forceinline__ void dmq_topk_token(const T* row, int experts, int k, int renorm, int lane,
+                                               float& my_w, int& my_e) {
+  if (experts <= 256) {
+    float v[4]; dmq_topk_load<T, 4>(row, experts, lane, v);
+    dmq_topk_select<4>(v, experts, k, renorm, lane, my_w, my_e);
+  } else if (experts <= 512) {
+    float v[8]; dmq_topk_load<T, 8>(row, experts, lane, v);
+    dmq_topk_select<8>(v, experts, k, renorm, lane, my_w, my_e);
+  } else {
+    float v[16]; dmq_topk_load<T, 16>(row, experts, lane, v);
+    dmq_topk_select<16>(v, experts, k, renorm, lane, my_w, my_e);
   }
 }
 
@@ -63,54 +162,12 @@ void dmq_topk_kernel(const T* logits, int tokens, int experts, int k, int renorm
   const int lane = threadIdx.x & 63;
   const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (tok >= tokens) return;
-  const T* row = logits + (long)tok * experts;
-  // up to 16 experts per lane (experts <= 1024), strided so lane l owns l, l+64, ...
-  float v[16];
-  float vmax = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    int e = lane + 64 * i;
-    v[i] = (e < experts) ? to_f32<T>(row[e]) : -INFINITY;
-    vmax = fmaxf(vmax, v[i]);
-  }
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, m, 64));
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) sum += (lane + 64 * i < experts) ? expf(v[i] - vmax) : 0.f;
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) sum += __shfl_xor(sum, m, 64);
-
-  float wsum = 0.f;
-  float my_w = 0.f;
-  int my_e = 0;
-  for (int round = 0; round < k; ++round) {
-    // lane-local best (lowest expert index wins ties), then wave arg-max
-    float bv = -INFINITY;
-    int be = 0x7fffffff;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      int e = lane + 64 * i;
-      if (v[i] > bv) { bv = v[i]; be = e; }
-    }
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) {
-      float ov = __shfl_xor(bv, m, 64);
-      int oe = __shfl_xor(be, m, 64);
-      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
-    }
-    const float w = expf(bv - vmax) / sum;
-    wsum += w;
-    if (lane == round) { my_w = w; my_e = be; }
-    if ((be & 63) == lane) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (i == (be >> 6)) v[i] = -INFINITY;
-    }
-  }
+  float my_w;
+  int my_e;
+  dmq_topk_token<T>(logits + (long)tok * experts, experts, k, renorm, lane, my_w, my_e);
   const int stride = k + sg.n_shared;
   if (lane < k) {
-    out_w[(long)tok * stride + lane] = renorm ? my_w / wsum : my_w;
+    out_w[(long)tok * stride + lane] = my_w;
     out_idx[(long)tok * stride + lane] = my_e;
   }
   dmq_shared_columns(sg, tok, experts, k, lane, out_w, out_idx);
@@ -157,6 +214,58 @@ __device__ __forceinline__ int block_scan_incl(int v, int* wave_tot) {
   for (int w = 0; w < wave; ++w) add += wave_tot[w];
   __syncthreads();
   return v + add;
+}
+
+// Per-pool expert_info and the work-item list from the per-expert counts and offsets in LDS
+// (pools in caller order, experts ascending).  Called by all 1024 threads of the workgroup.
+__device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* s_cnt, const int* s_off,
+                                                int* wave_tot, int* carry_p) {
+  const int tid = threadIdx.x;
+  if (tid == 0) *carry_p = 0;
+  // the slice tables of all pools are requested at once when one pass covers the experts
+  int ss_pre[DMQ_MAX_POOLS], sc_pre[DMQ_MAX_POOLS];
+  const bool pre = p.experts <= 1024;
+#pragma unroll
+  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+    const bool ok = pre && pool < p.pools && tid < p.experts;
+    ss_pre[pool] = ok ? p.slice_start_rows[pool * p.experts + tid] : -1;
+    sc_pre[pool] = ok ? p.slice_count_rows[pool * p.experts + tid] : 0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+    if (pool >= p.pools) break;
+    for (int base = 0; base < p.experts; base += 1024) {
+      const int e = base + tid;
+      int ntile = 0, ts = 0, tc = 0, gu_ss = 0, dn_ss = 0;
+      if (e < p.experts) {
+        const int ss = pre ? ss_pre[pool] : p.slice_start_rows[pool * p.experts + e];
+        const int sc = pre ? sc_pre[pool] : p.slice_count_rows[pool * p.experts + e];
+        tc = (ss >= 0) ? s_cnt[e] : 0;
+        ts = s_off[e];
+        gu_ss = ss >= 0 ? ss : 0;
+        dn_ss = ss >= 0 ? ss / (2 * DMQ_GS) : 0;
+        ntile = (tc + p.tile_rows - 1) / p.tile_rows;
+        int* gi = p.gu_info + ((long)pool * p.experts + e) * 4;
+        gi[0] = ts; gi[1] = tc; gi[2] = gu_ss; gi[3] = sc;
+        int* di = p.dn_info + ((long)pool * p.experts + e) * 4;
+        di[0] = ts; di[1] = tc; di[2] = dn_ss; di[3] = sc / (2 * DMQ_GS);
+      }
+      const int incl = block_scan_incl(ntile, wave_tot);
+      const int first = incl - ntile + *carry_p;
+      for (int i = 0; i < ntile; ++i) {
+        if (first + i < p.max_items) {
+          int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * (first + i));
+          it[0] = (int4_t){pool, e, i, ts};
+          it[1] = (int4_t){tc, gu_ss, dn_ss, 0};
+        }
+      }
+      __syncthreads();
+      if (tid == 1023) *carry_p = incl + *carry_p;
+      __syncthreads();
+    }
+  }
+  if (tid == 0) p.n_items[0] = min(*carry_p, p.max_items);
 }
 
 __global__ __launch_bounds__(1024)
@@ -245,52 +354,7 @@ void dmq_plan_kernel(PlanParams p) {
     if (!one_pass) __syncthreads();
   }
 
-  // per-pool expert_info and the work-item list, pools in caller order, experts ascending
-  if (tid == 0) carry = 0;
-  // the slice tables of all pools are requested at once when one pass covers the experts
-  int ss_pre[DMQ_MAX_POOLS], sc_pre[DMQ_MAX_POOLS];
-  const bool pre = p.experts <= 1024;
-#pragma unroll
-  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
-    const bool ok = pre && pool < p.pools && tid < p.experts;
-    ss_pre[pool] = ok ? p.slice_start_rows[pool * p.experts + tid] : -1;
-    sc_pre[pool] = ok ? p.slice_count_rows[pool * p.experts + tid] : 0;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
-    if (pool >= p.pools) break;
-    for (int base = 0; base < p.experts; base += 1024) {
-      const int e = base + tid;
-      int ntile = 0, ts = 0, tc = 0, gu_ss = 0, dn_ss = 0;
-      if (e < p.experts) {
-        const int ss = pre ? ss_pre[pool] : p.slice_start_rows[pool * p.experts + e];
-        const int sc = pre ? sc_pre[pool] : p.slice_count_rows[pool * p.experts + e];
-        tc = (ss >= 0) ? s_cnt[e] : 0;
-        ts = s_off[e];
-        gu_ss = ss >= 0 ? ss : 0;
-        dn_ss = ss >= 0 ? ss / (2 * DMQ_GS) : 0;
-        ntile = (tc + p.tile_rows - 1) / p.tile_rows;
-        int* gi = p.gu_info + ((long)pool * p.experts + e) * 4;
-        gi[0] = ts; gi[1] = tc; gi[2] = gu_ss; gi[3] = sc;
-        int* di = p.dn_info + ((long)pool * p.experts + e) * 4;
-        di[0] = ts; di[1] = tc; di[2] = dn_ss; di[3] = sc / (2 * DMQ_GS);
-      }
-      const int incl = block_scan_incl(ntile, wave_tot);
-      const int first = incl - ntile + carry;
-      for (int i = 0; i < ntile; ++i) {
-        if (first + i < p.max_items) {
-          int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * (first + i));
-          it[0] = (int4_t){pool, e, i, ts};
-          it[1] = (int4_t){tc, gu_ss, dn_ss, 0};
-        }
-      }
-      __syncthreads();
-      if (tid == 1023) carry = incl + carry;
-      __syncthreads();
-    }
-  }
-  if (tid == 0) p.n_items[0] = min(carry, p.max_items);
+  plan_emit_items(p, s_cnt, s_off, wave_tot, &carry);
 }
 
 // Stable scatter of one chunk.  The rows of one token name distinct experts, so the lanes of a
@@ -327,6 +391,117 @@ void dmq_chunk_fill_kernel(const int* topk_idx, const float* topk_w, int rows, i
       sorted_tokens[at] = tok;
       sorted_weights[at] = w;
       sorted_rows[at] = r;
+    }
+  }
+}
+
+// Small batches: the whole routing step in one workgroup of 16 waves.  Wave w computes the top-k
+// of tokens w, w + 16, ... (or copies the caller's), appends the shared columns and keeps the
+// rows in LDS; the sort is the chunked counting sort above with one chunk of 64 rows per wave and
+// every table in LDS.
+template <typename T>
+__global__ __launch_bounds__(1024)
+void dmq_route_small_kernel(RouteSmallParams p) {
+  __shared__ int wave_tot[16];
+  __shared__ int carry;
+  __shared__ int s_cnt[DMQ_ROUTE_SMALL_EXPERTS];
+  __shared__ int s_off[DMQ_ROUTE_SMALL_EXPERTS + 1];
+  __shared__ int s_hist[16 * DMQ_ROUTE_SMALL_EXPERTS];
+  __shared__ int s_idx[DMQ_ROUTE_SMALL_ROWS];
+  __shared__ float s_w[DMQ_ROUTE_SMALL_ROWS];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int k = p.k;
+  const int kt = k + p.sg.n_shared;
+  const int rows = p.tokens * kt;
+  const int experts = p.plan.experts;
+  for (int i = tid; i < 16 * experts; i += 1024) s_hist[i] = 0;
+  // top-k (or the caller's), shared columns: the rows of the next token of the wave are requested
+  // before the current token is worked on
+  auto tokens_of_wave = [&](auto nv_tag) {
+    constexpr int NV = decltype(nv_tag)::value;
+    float v_next[NV];
+    if (p.logits && wave < p.tokens)
+      dmq_topk_load<T, NV>((const T*)p.logits + (long)wave * p.router_experts, p.router_experts, lane, v_next);
+    for (int tok = wave; tok < p.tokens; tok += 16) {
+      float w = 0.f;
+      int e = -1;
+      float g = 0.f;
+      if (p.sg.n_shared > 0) g = dmq_shared_gate_value(p.sg, tok, lane);
+      if (p.logits) {
+        float v[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) v[i] = v_next[i];
+        if (tok + 16 < p.tokens)
+          dmq_topk_load<T, NV>((const T*)p.logits + (long)(tok + 16) * p.router_experts,
+                               p.router_experts, lane, v_next);
+        dmq_topk_select<NV>(v, p.router_experts, k, p.renorm, lane, w, e);
+      } else if (lane < k) {
+        w = p.in_w[(long)tok * k + lane];
+        e = p.in_idx[(long)tok * k + lane];
+      }
+      if (lane >= k && lane < kt) { w = g; e = p.router_experts + (lane - k); }
+      if (lane < kt) {
+        s_idx[tok * kt + lane] = e;
+        s_w[tok * kt + lane] = w;
+        if (p.out_w) { p.out_w[(long)tok * kt + lane] = w; p.out_idx[(long)tok * kt + lane] = e; }
+      }
+    }
+  };
+  if (!p.logits || p.router_experts <= 256) tokens_of_wave(std::integral_constant<int, 4>{});
+  else if (p.router_experts <= 512) tokens_of_wave(std::integral_constant<int, 8>{});
+  else tokens_of_wave(std::integral_constant<int, 16>{});
+  __syncthreads();
+  // rows per (wave chunk, expert)
+  const int r = tid;
+  const int e_r = (r < rows) ? s_idx[r] : -1;
+  const bool hit = e_r >= 0 && e_r < experts;
+  int* my_hist = s_hist + wave * experts;
+  if (hit) atomicAdd(&my_hist[e_r], 1);
+  __syncthreads();
+  if (tid < experts) {
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) total += s_hist[w * experts + tid];
+    s_cnt[tid] = total;
+    p.plan.counts[tid] = total;
+  }
+  __syncthreads();
+  {
+    const int c = (tid < experts) ? s_cnt[tid] : 0;
+    const int incl = block_scan_incl(c, wave_tot);
+    if (tid < experts) { s_off[tid + 1] = incl; p.plan.offsets[tid + 1] = incl; }
+    if (tid == 0) { s_off[0] = 0; p.plan.offsets[0] = 0; }
+  }
+  __syncthreads();
+  // s_hist[w, e] <- sorted position of the first row of wave chunk w routed to expert e
+  if (tid < experts) {
+    int at = s_off[tid];
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int n = s_hist[w * experts + tid];
+      s_hist[w * experts + tid] = at;
+      at += n;
+    }
+  }
+  __syncthreads();
+  plan_emit_items(p.plan, s_cnt, s_off, wave_tot, &carry);
+  // stable scatter of the wave's chunk: tokens one after the other, the rows of a token name
+  // distinct experts
+  const int base = wave * 64;
+  if (base < rows) {
+    const int tok = r / kt;
+    const int tok_first = base / kt;
+    const int tok_last = (min(base + 64, rows) - 1) / kt;
+    int at = -1;
+    for (int t = tok_first; t <= tok_last; ++t) {
+      if (hit && tok == t) at = atomicAdd(&my_hist[e_r], 1);
+    }
+    if (at >= 0) {
+      p.sorted_tokens[at] = tok;
+      p.sorted_weights[at] = s_w[r];
+      p.sorted_rows[at] = r;
     }
   }
 }
@@ -427,6 +602,19 @@ int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int token
   hipLaunchKernelGGL(dmq_chunk_fill_kernel, dim3(grid_c), dim3(256), 0, stream, topk_idx, topk_w,
                      rows, k, experts, plan.chunk_rows, plan.n_chunks, plan.hist, sorted_tokens,
                      sorted_weights, sorted_rows);
+  return dmq_check_launch();
+}
+
+int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream) {
+  const int kt = p.k + p.sg.n_shared;
+  if ((long)p.tokens * kt > DMQ_ROUTE_SMALL_ROWS || p.plan.experts > DMQ_ROUTE_SMALL_EXPERTS || kt > 64)
+    return DMQ_ERR_LIMIT;
+  if (p.logits && (p.router_experts > 1024 || p.k > p.router_experts)) return DMQ_ERR_LIMIT;
+  if (p.sg.n_shared > 0 && p.sg.hidden % 8) return DMQ_ERR_ALIGN;
+  if (p.logits && p.logits_fp16)
+    hipLaunchKernelGGL(dmq_route_small_kernel<__half>, dim3(1), dim3(1024), 0, stream, p);
+  else
+    hipLaunchKernelGGL(dmq_route_small_kernel<float>, dim3(1), dim3(1024), 0, stream, p);
   return dmq_check_launch();
 }
 

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 5
+ABI_VERSION = 6
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER = 0, 1, 2
@@ -65,6 +65,14 @@ class LayerDesc(Structure):
     ]
 
 
+class RouterArgs(Structure):
+    _fields_ = [
+        ("logits", c_void_p), ("logits_fp16", c_int), ("renorm", c_int),
+        ("topk_idx", c_void_p), ("topk_w", c_void_p),
+        ("shared_gate_row", c_void_p), ("n_shared", c_int),
+    ]
+
+
 # name -> (restype, argtypes); the single source for the symbol-export test as well
 PROTOTYPES = {
     "dmq_abi_version": (c_int, []),
@@ -98,6 +106,9 @@ PROTOTYPES = {
     "dmq_moe_ffn_forward": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                     c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p]),
     "dmq_moe_ffn_forward_staged": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int,
+                                           c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int,
+                                           c_int, POINTER(c_void_p), POINTER(c_long), c_void_p]),
+    "dmq_moe_ffn_forward_routed": (c_int, [POINTER(LayerDesc), POINTER(RouterArgs), c_void_p, c_int,
                                            c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int,
                                            c_int, POINTER(c_void_p), POINTER(c_long), c_void_p]),
 }

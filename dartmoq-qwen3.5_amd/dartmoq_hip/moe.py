@@ -17,8 +17,8 @@ import math
 import torch
 
 from . import hostprep, ops
-from ._lib import (MODE_A16, MODE_A8, MODE_BY_NAME, MODE_FP4, MODE_FP8, LayerDesc, PoolDesc, check,
-                   load)
+from ._lib import (MODE_A16, MODE_A8, MODE_BY_NAME, MODE_FP4, MODE_FP8, LayerDesc, PoolDesc,
+                   RouterArgs, check, load)
 
 GROUP_SIZE = 128
 
@@ -345,6 +345,39 @@ class WxA16BitPartitionedGroupMoE:
         return ops.route_topk_shared(None, topk_idx, topk_w, self.top_k, False, x,
                                      self.shared_gate_row, self.num_experts, self.n_shared)
 
+    def _router_args(self, x, router_logits, topk_idx, topk_w):
+        """dmq_router_args for this call plus the tensors it points into (kept alive by the caller)."""
+        r = RouterArgs()
+        keep = []
+        if topk_idx is None:
+            if router_logits is None:
+                if self.gate_weight is None:
+                    raise ValueError("no gate weight: pass router_logits or topk_idx/topk_w")
+                router_logits = torch.matmul(x, self.gate_weight.t().to(x.dtype))
+            if router_logits.dtype not in (torch.float32, torch.float16):
+                router_logits = router_logits.float()
+            router_logits = router_logits.contiguous()
+            if tuple(router_logits.shape) != (x.shape[0], self.num_experts):
+                raise ValueError("router_logits must be [tokens, num_experts]")
+            keep.append(router_logits)
+            r.logits = router_logits.data_ptr()
+            r.logits_fp16 = int(router_logits.dtype == torch.float16)
+            r.renorm = int(self.renormalize)
+        else:
+            if topk_idx.shape[-1] == self.top_k + self.n_shared and self.n_shared:
+                # already widened by widen_topk: hand the router's own columns over
+                topk_idx, topk_w = topk_idx[:, :self.top_k], topk_w[:, :self.top_k]
+            topk_idx = topk_idx.to(torch.int32).contiguous()
+            topk_w = topk_w.float().contiguous()
+            if tuple(topk_idx.shape) != (x.shape[0], self.top_k) or topk_w.shape != topk_idx.shape:
+                raise ValueError("topk_idx / topk_w must be [tokens, top_k]")
+            keep += [topk_idx, topk_w]
+            r.topk_idx, r.topk_w = topk_idx.data_ptr(), topk_w.data_ptr()
+        if self.n_shared:
+            r.shared_gate_row = self.shared_gate_row.data_ptr()
+            r.n_shared = self.n_shared
+        return r, keep
+
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None,
                 topk_idx: torch.Tensor | None = None, topk_w: torch.Tensor | None = None,
@@ -358,21 +391,18 @@ class WxA16BitPartitionedGroupMoE:
             x = x.half()
         x = x.contiguous()
         tokens = x.shape[0]
-        if topk_idx is None:
-            topk_w, topk_idx = self.route(x, router_logits)
-        else:
-            topk_w, topk_idx = self.widen_topk(x, topk_idx, topk_w)
-        topk_idx = topk_idx.to(torch.int32).contiguous()
-        topk_w = topk_w.float().contiguous()
+        router, keep = self._router_args(x, router_logits, topk_idx, topk_w)
         desc = self._descriptor()[0]
         ws = self._get_workspace(tokens)
         out = torch.empty_like(x)
         add = None if residual is None else residual.reshape(-1, shape[-1]).half().contiguous()
         stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
-        check(load().dmq_moe_ffn_forward(
-            ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens,
+        check(load().dmq_moe_ffn_forward_routed(
+            ctypes.byref(desc), ctypes.byref(router), x.data_ptr(), tokens,
             None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-            int(self.tt_override), int(self.ks_override), int(self.nbl_override), stream), "moe_ffn_forward")
+            int(self.tt_override), int(self.ks_override), int(self.nbl_override), None, None, stream),
+            "moe_ffn_forward_routed")
+        del keep
         if orig_dtype != torch.float16:
             out = out.to(orig_dtype)
         return out.reshape(shape)
@@ -462,20 +492,20 @@ STAGE_NAMES = ("sort_prep", "rotation", "merged_gate_up", "act_quant_down", "mer
 
 
 @torch.no_grad()
-def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: torch.Tensor,
-                   topk_w: torch.Tensor, tt: int = 0, ks: int = 0, nbl: int = 0,
-                   profile: bool = True):
-    """dmq_moe_ffn_forward_staged: the production forward with an event recorded on the launch
-    stream after every stage.  Returns (out fp16 [T, H], {stage: ms}, aux) where aux carries the
+def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor,
+                   topk_idx: torch.Tensor | None = None, topk_w: torch.Tensor | None = None,
+                   tt: int = 0, ks: int = 0, nbl: int = 0, profile: bool = True,
+                   router_logits: torch.Tensor | None = None):
+    """dmq_moe_ffn_forward_routed with instrumentation: the production forward with an event
+    recorded on the launch stream after every stage (sort_prep includes the top-k when
+    ``router_logits`` are given instead of ``topk_idx`` / ``topk_w``).  Returns (out fp16 [T, H], {stage: ms}, aux) where aux carries the
     per-expert routed-row counts (for byte accounting) and the tiling that was used.  Stage names
     follow the reference's profiler: sort_prep, rotation (rotation_hoisted / act_quant),
     merged_gate_up (with silu_mul fused), act_quant_down, merged_down (routing weight and scatter
     fused), combine (the add of the scattered rows)."""
     x = x.half().contiguous()
     tokens = x.shape[0]
-    topk_w, topk_idx = moe.widen_topk(x, topk_idx.to(torch.int32).contiguous(), topk_w.float().contiguous())
-    topk_idx = topk_idx.to(torch.int32).contiguous()
-    topk_w = topk_w.float().contiguous()
+    router, keep = moe._router_args(x, router_logits, topk_idx, topk_w)
     desc = moe._descriptor()[0]
     ws = moe._get_workspace(tokens)
     out = torch.empty_like(x)
@@ -487,11 +517,11 @@ def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor, topk_idx: 
             ev.record(stream)                       # materialise the HIP event behind the object
             handles[i] = ev.cuda_event
     aux = (ctypes.c_long * 8)()
-    check(load().dmq_moe_ffn_forward_staged(
-        ctypes.byref(desc), x.data_ptr(), topk_idx.data_ptr(), topk_w.data_ptr(), tokens, None,
+    check(load().dmq_moe_ffn_forward_routed(
+        ctypes.byref(desc), ctypes.byref(router), x.data_ptr(), tokens, None,
         out.data_ptr(), ws.data_ptr(), ws.numel(), int(tt or moe.tt_override),
         int(ks or moe.ks_override), int(nbl or moe.nbl_override), handles if profile else None, aux,
-        ctypes.c_void_p(stream.cuda_stream)), "moe_ffn_forward_staged")
+        ctypes.c_void_p(stream.cuda_stream)), "moe_ffn_forward_routed")
     torch.cuda.synchronize(x.device)
     stats = {}
     if profile:

@@ -48,7 +48,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 5). */
+/* Library / build identification: returns the ABI version (currently 6). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -266,6 +266,31 @@ int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* 
  * max_items, the byte offset of n_items and nbl. */
 int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                                const void* topk_w, int tokens, const void* add_f16, void* out,
+                               void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
+                               void* const* stage_events, void* aux_out, void* stream);
+
+/* The router's output as the layer forward takes it: either its logits (softmax + top-k run
+ * inside, quantization/wxa16/bit_partitioned_moe.py:1112-1120) or its own top-k (the HF tuple
+ * form), plus the sigmoid gate of the always-on shared expert (:1101-1106, see
+ * dmq_route_topk_shared). */
+typedef struct {
+  const void* logits;           /* [tokens, experts - n_shared] fp32 / fp16, or NULL */
+  int logits_fp16;
+  int renorm;                   /* divide the kept weights by their sum */
+  const void* topk_idx;         /* logits == NULL: int32 [tokens, top_k - n_shared] */
+  const void* topk_w;           /* logits == NULL: fp32  [tokens, top_k - n_shared] */
+  const void* shared_gate_row;  /* fp16 [hidden] (n_shared > 0) */
+  int n_shared;                 /* slices of the shared expert among layer->experts / top_k */
+} dmq_router_args;
+
+/* The whole layer from the router's output: dmq_moe_ffn_forward_staged plus the routing step.
+ * layer->experts and layer->top_k count the n_shared always-on slices (experts E .. E+n_shared-1,
+ * selected by every token with the gate value as routing weight).  For up to 1024 routed rows
+ * and 512 experts (16 tokens when the top-k is computed here) top-k, shared columns, sort and
+ * work-item list are a single one-workgroup launch.  stage_events / aux_out as in
+ * dmq_moe_ffn_forward_staged (the first stage then includes the top-k); both may be NULL. */
+int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_args* router,
+                               const void* x, int tokens, const void* add_f16, void* out,
                                void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
                                void* const* stage_events, void* aux_out, void* stream);
 

@@ -191,3 +191,22 @@ def test_from_reference_module_duck_typing():
     y1 = m1.forward(x, router_logits=logits)
     y2 = m2.forward(x, router_logits=logits)
     assert torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("tokens", [1, 64, 65, 128, 300])
+def test_forward_from_logits_equals_forward_from_topk(small_layer, tokens):
+    """The routing step has three shapes (one fused launch with the top-k inside, fused launch
+    after a separate top-k, chunked sort): all must give the bits of the forward that is handed
+    the same top-k."""
+    from dartmoq_hip import ops
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(tokens, small_layer.hidden, generator=g).half().cuda()
+    logits = routing.zipf_logits(tokens, small_layer.num_experts, tokens).cuda()
+    mod = make_module(small_layer, "wxa16")
+    w, idx = ops.route_topk(logits, small_layer.top_k)
+    a = mod.forward(x, router_logits=logits)
+    b = mod.forward(x, topk_idx=idx, topk_w=w)
+    assert torch.equal(a, b)
+    c = mod.forward(x, router_logits=logits.half())
+    w16, idx16 = ops.route_topk(logits.half(), small_layer.top_k)
+    assert torch.equal(c, mod.forward(x, topk_idx=idx16, topk_w=w16))

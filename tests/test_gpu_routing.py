@@ -85,7 +85,8 @@ def test_permute_matches_oracle(tokens, tile_rows):
     assert [tuple(r) for r in res["items"][:n].cpu().tolist()] == exp_items
 
 
-@pytest.mark.parametrize("tokens,experts,k", [(700, 100, 3), (1000, 37, 1), (333, 300, 5), (5000, 256, 8)])
+@pytest.mark.parametrize("tokens,experts,k", [(700, 100, 3), (1000, 37, 1), (333, 300, 5), (5000, 256, 8),
+                                                   (113, 257, 9), (128, 512, 8), (60, 513, 8), (129, 512, 8)])
 def test_permute_odd_shapes(tokens, experts, k):
     """Tokens whose k rows straddle the 64-row steps of the sort, expert counts off the wave size."""
     from dartmoq_hip import ops

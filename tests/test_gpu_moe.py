@@ -210,3 +210,33 @@ def test_forward_from_logits_equals_forward_from_topk(small_layer, tokens):
     c = mod.forward(x, router_logits=logits.half())
     w16, idx16 = ops.route_topk(logits.half(), small_layer.top_k)
     assert torch.equal(c, mod.forward(x, topk_idx=idx16, topk_w=w16))
+
+
+@pytest.mark.parametrize("tokens", [4, 150])
+def test_forward_is_graph_capturable(small_layer, tokens):
+    """The forward allocates nothing and never synchronises, so a caller can capture it in a HIP
+    graph: every replay, with eager work and synchronisation in between, reproduces the eager
+    result bit for bit."""
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(tokens, small_layer.hidden, generator=g).half().cuda()
+    logits = routing.zipf_logits(tokens, small_layer.num_experts, tokens).cuda()
+    mod = make_module(small_layer, "wxa8")
+    ref = mod.forward(x, router_logits=logits).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            mod.forward(x, router_logits=logits)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = mod.forward(x, router_logits=logits)
+    for _ in range(4):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, ref)
+        other = mod.forward(x.flip(0).contiguous(), router_logits=logits.flip(0).contiguous())
+        torch.cuda.synchronize()
+        assert torch.equal(other.flip(0), ref)

@@ -68,7 +68,7 @@ int dmq_convert_to_group_first(const void* indices_packed, const void* norms, in
 
 int dmq_dequant_tile(const void* idx_gf, const void* codebook_f16, const void* norms_gf, int n_total,
                      int g0, int g_cnt, int n0, int n_cnt, int bit, void* out_f16, void* stream) {
-  if (!dmq_valid_bit(bit)) return DMQ_ERR_BIT;
+  if (!dmq_valid_bit_wide(bit)) return DMQ_ERR_BIT;
   if (!idx_gf || !codebook_f16 || !out_f16) return DMQ_ERR_NULL;
   if (g0 < 0 || n0 < 0 || g_cnt < 0 || n_cnt < 0 || n0 + n_cnt > n_total) return DMQ_ERR_SHAPE;
   return dmq_dequant_tile_launch((const uint8_t*)idx_gf, (const __half*)codebook_f16,
@@ -220,8 +220,14 @@ int dmq_quantize_act(int mode, const void* x, int x_fp32, long x_stride, int row
 int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (!a) return DMQ_ERR_NULL;
   if (a->n_pools <= 0 || a->n_pools > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
-  for (int i = 0; i < a->n_pools; ++i)
-    if (!dmq_valid_bit(a->pool[i].bit)) return DMQ_ERR_BIT;
+  bool any_wide = false, any_narrow = false;
+  for (int i = 0; i < a->n_pools; ++i) {
+    const int b = a->pool[i].bit;
+    if (!dmq_valid_bit_wide(b)) return DMQ_ERR_BIT;
+    if (a->pool[i].mode != a->mode) continue;
+    if (b == 8 && a->mode == DMQ_MODE_FP4) return DMQ_ERR_BIT;
+    (b == 8 ? any_wide : any_narrow) = true;
+  }
   if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
   if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SCATTER) return DMQ_ERR_MODE;
   const int ks = a->ks > 0 ? a->ks : 1;
@@ -258,13 +264,6 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.slice_is_groups = a->slice_is_groups;
   p.items = (const int*)a->items;
   p.n_items = (const int*)a->n_items;
-  const int feat_per_block = (4 / ks) * feat_per_wave;
-  p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
-  // several n-blocks per workgroup need every block complete and the waves on distinct features
-  int nbl = a->nbl > 0 ? a->nbl : 1;
-  if (ks > 1 || a->n_out % feat_per_block) nbl = 1;
-  if (nbl > p.n_blocks) nbl = p.n_blocks;
-  p.nbl = nbl;
   p.out = (__half*)a->out;
   p.out_stride = a->out_stride;
   p.out_slots = (__half*)a->out;
@@ -273,20 +272,37 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.dbg_acc = (int*)a->dbg_acc;
   L.epi = a->epi;
   L.tt = a->tt;
-  L.ks = ks;
   L.dbg = a->dbg_acc != nullptr;
   L.stream = (hipStream_t)stream;
-  long work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl);
-  work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;      // every XCD gets the same number of slots
-  if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
-  L.grid = (int)work;
-  switch (a->mode) {
-    case DMQ_MODE_A16: return dmq_gemm_launch_a16(L);
-    case DMQ_MODE_A8: return dmq_gemm_launch_a8(L);
-    case DMQ_MODE_FP8: return dmq_gemm_launch_fp8(L);
-    case DMQ_MODE_FP4: return dmq_gemm_launch_fp4(L);
+  // the 1/2/4-bit pools and the 8-bit pools of the mode are separate launches over the same work
+  // list (each skips the items of the other kind); 8-bit pools never split K over the waves
+  for (int wide = 0; wide < 2; ++wide) {
+    if (!(wide ? any_wide : any_narrow)) continue;
+    const int lks = wide ? 1 : ks;
+    const int feat_per_block = (4 / lks) * feat_per_wave;
+    p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
+    // several n-blocks per workgroup need every block complete and the waves on distinct features
+    int nbl = a->nbl > 0 ? a->nbl : 1;
+    if (lks > 1 || a->n_out % feat_per_block) nbl = 1;
+    if (nbl > p.n_blocks) nbl = p.n_blocks;
+    p.nbl = nbl;
+    L.p = p;
+    L.ks = lks;
+    L.wide = wide;
+    long work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl);
+    work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
+    if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
+    L.grid = (int)work;
+    int rc = DMQ_ERR_MODE;
+    switch (a->mode) {
+      case DMQ_MODE_A16: rc = dmq_gemm_launch_a16(L); break;
+      case DMQ_MODE_A8: rc = dmq_gemm_launch_a8(L); break;
+      case DMQ_MODE_FP8: rc = dmq_gemm_launch_fp8(L); break;
+      case DMQ_MODE_FP4: rc = dmq_gemm_launch_fp4(L); break;
+    }
+    if (rc) return rc;
   }
-  return DMQ_ERR_MODE;
+  return DMQ_OK;
 }
 
 int dmq_combine_slots(const void* slots_f16, int k, const void* add_f16, long tokens, int hidden,
@@ -444,7 +460,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   for (int i = 0; i < P; ++i) {
     const int m = layer->pool[i].mode;
     if (!valid_mode(m)) return DMQ_ERR_MODE;
-    if (!dmq_valid_bit(layer->pool[i].bit)) return DMQ_ERR_BIT;
+    if (!dmq_valid_bit_wide(layer->pool[i].bit)) return DMQ_ERR_BIT;
+    if (layer->pool[i].bit == 8 && m == DMQ_MODE_FP4) return DMQ_ERR_BIT;
     bool seen = false;
     for (int j = 0; j < n_modes; ++j) seen |= (modes[j] == m);
     if (!seen) modes[n_modes++] = m;

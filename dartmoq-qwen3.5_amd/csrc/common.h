@@ -25,6 +25,9 @@ static inline int dmq_check_launch() {
 }
 
 static inline bool dmq_valid_bit(int bit) { return bit == 1 || bit == 2 || bit == 4; }
+// 8-bit indices (256-entry codebooks of the Linear path) are served by the GEMM, the dequantized
+// tile and the layout kernels, not by the e2m1 fold
+static inline bool dmq_valid_bit_wide(int bit) { return dmq_valid_bit(bit) || bit == 8; }
 
 // ---------------------------------------------------------------- device helpers
 // silu(x) = x * sigmoid(x); the hardware reciprocal (1 ulp) replaces the IEEE division, the

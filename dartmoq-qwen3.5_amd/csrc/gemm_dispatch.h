@@ -9,6 +9,7 @@ struct GemmLaunch {
   int tt;          // activation tiles of 16 rows per wave: 1, 2 or 4
   int ks;          // waves splitting K: 1, 2 or 4
   int dbg;
+  int wide;        // 1: the pools of 8-bit indices (ks must be 1), 0: the 1/2/4-bit pools
   int grid;
   hipStream_t stream;
 };
@@ -21,7 +22,15 @@ static inline bool dmq_gemm_config_ok(int tt, int ks) {
 
 template <int MODE, int TT, int KS, int EPI, bool DBG>
 static int dmq_gemm_launch_one(const GemmLaunch& L) {
-  hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG>), dim3(L.grid), dim3(256), 0,
+  if constexpr (MODE != DMQ_MODE_FP4 && KS == 1 && !DBG) {
+    if (L.wide) {
+      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, true>), dim3(L.grid), dim3(256), 0,
+                         L.stream, L.p);
+      return dmq_check_launch();
+    }
+  }
+  if (L.wide) return DMQ_ERR_MODE;
+  hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false>), dim3(L.grid), dim3(256), 0,
                      L.stream, L.p);
   return dmq_check_launch();
 }

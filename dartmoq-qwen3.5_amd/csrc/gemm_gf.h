@@ -126,10 +126,14 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
     constexpr int bi = S * BYTES + b;
     if constexpr (G::EB >= 4) {
       dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], w + b * (G::EB / 4));
-    } else {                                            // two one-byte elements per look-up
+    } else if constexpr (G::EB == 2) {                  // two two-byte entries per operand word
       uint32_t v;
       dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], &v);
       if (b & 1) w[b >> 1] |= v << 16; else w[b >> 1] = v;
+    } else {                                            // four one-byte entries per operand word
+      uint32_t v;
+      dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], &v);
+      if (b & 3) w[b >> 2] |= v << (8 * (b & 3)); else w[b >> 2] = v;
     }
   };
   one(std::integral_constant<int, 0>{});
@@ -139,7 +143,13 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
     one(std::integral_constant<int, 4>{}); one(std::integral_constant<int, 5>{});
     one(std::integral_constant<int, 6>{}); one(std::integral_constant<int, 7>{});
   }
-  static_assert(BYTES <= 8, "at most eight packed bytes per MFMA step");
+  if constexpr (BYTES > 8) {
+    one(std::integral_constant<int, 8>{}); one(std::integral_constant<int, 9>{});
+    one(std::integral_constant<int, 10>{}); one(std::integral_constant<int, 11>{});
+    one(std::integral_constant<int, 12>{}); one(std::integral_constant<int, 13>{});
+    one(std::integral_constant<int, 14>{}); one(std::integral_constant<int, 15>{});
+  }
+  static_assert(BYTES <= 16, "at most sixteen packed bytes per MFMA step");
 }
 
 // Groups in flight per wave on the staged path.  WW registers hold one (group, n-tile) of packed
@@ -680,8 +690,11 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 
 // Waves per SIMD the register allocation aims for: three for tiles up to 32 rows (the 32-row
 // fp16 kernel sits a few registers above that limit otherwise), two for 64-row tiles.
-template <int MODE, int TT, int EPI, int KS, bool DBG>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((KS == 1 && TT <= 2) ? 3 : 2)))
+// WIDE kernels serve the pools of 8-bit indices (one byte per weight: twice the packed words per
+// lane of a 4-bit pool); they are separate instances so that their registers do not count against
+// the kernels of the 1/2/4-bit pools.  A launch skips the work items of the other kind.
+template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
   constexpr int NT = 4;
   __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
@@ -714,8 +727,11 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   const int slice_start = p.slice_is_groups ? r1[2] : r1[1];
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE) return;
+  if (WIDE != (pw.bit == 8)) return;
   if constexpr (MODE == DMQ_MODE_FP4) {
     dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc);
+  } else if constexpr (WIDE) {
+    dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc);
   } else {
     switch (pw.bit) {
       case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;

@@ -1,6 +1,7 @@
 // Byte-indexed codebook look-up table held in LDS.
 //
-// A packed weight byte carries 8/BIT codebook indices.  The table maps a byte
+// A packed weight byte carries 8/BIT codebook indices (one for the 8-bit codebooks of the Linear
+// path).  The table maps a byte
 // value straight to its 8/BIT dequantized elements (fp16 for WxA16, one byte
 // each for the int8 / e4m3 look-ups), so dequantizing costs one LDS read per
 // packed byte.  Every entry is replicated across a row of DMQ_LUT_ROW bytes; lane L
@@ -100,7 +101,9 @@ __device__ __forceinline__ void dmq_lut_read_word(const uint8_t* tbl, uint32_t l
     off = (((word >> (8 * K)) & 0xffu) * DMQ_LUT_ROW) + lane_base;
   }
   const uint8_t* p = tbl + off;
-  if (G::EB == 2) {
+  if (G::EB == 1) {
+    out[0] = *p;
+  } else if (G::EB == 2) {
     out[0] = *(const uint16_t*)p;
   } else if (G::EB == 4) {
     out[0] = *(const uint32_t*)p;

@@ -146,6 +146,7 @@ int dmq_dequant_tile_launch(const uint8_t* idx_gf, const __half* cb, const __hal
     case 1: hipLaunchKernelGGL(dmq_dequant_tile_kernel<1>, dim3(grid), dim3(256), 0, s, idx_gf, cb, norms, n_total, g0, g_cnt, n0, n_cnt, out); break;
     case 2: hipLaunchKernelGGL(dmq_dequant_tile_kernel<2>, dim3(grid), dim3(256), 0, s, idx_gf, cb, norms, n_total, g0, g_cnt, n0, n_cnt, out); break;
     case 4: hipLaunchKernelGGL(dmq_dequant_tile_kernel<4>, dim3(grid), dim3(256), 0, s, idx_gf, cb, norms, n_total, g0, g_cnt, n0, n_cnt, out); break;
+    case 8: hipLaunchKernelGGL(dmq_dequant_tile_kernel<8>, dim3(grid), dim3(256), 0, s, idx_gf, cb, norms, n_total, g0, g_cnt, n0, n_cnt, out); break;
     default: return DMQ_ERR_BIT;
   }
   return dmq_check_launch();

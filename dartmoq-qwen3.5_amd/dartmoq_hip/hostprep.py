@@ -66,6 +66,42 @@ def build_int8_codebook(codebook: torch.Tensor):
     return (cb / step).round().clamp_(-127, 127).to(torch.int8).contiguous(), step
 
 
+def uniform_codebook_step(codebook: torch.Tensor) -> float:
+    """Step of a uniform 256-level codebook cb[i] = (i - 128) * step, from its end points
+    (quantization/wxa8/linear.py:35-47)."""
+    cb = codebook.float()
+    if cb.numel() != 256:
+        raise ValueError(f"an 8-bit codebook has 256 levels, got {cb.numel()}")
+    step = float((cb[-1] - cb[0]) / 255.0)
+    if step <= 0:
+        raise ValueError(f"illegal codebook step {step}")
+    return step
+
+
+def is_uniform_codebook(codebook: torch.Tensor, rel_tol: float = 1e-2) -> bool:
+    """Constant spacing between neighbouring levels (quantization/wxa8/linear.py:50-62)."""
+    if codebook.numel() != 256:
+        return False
+    d = codebook.float()[1:] - codebook.float()[:-1]
+    mean = d.mean().abs()
+    if mean <= 0:
+        return False
+    return bool((d - d.mean()).abs().max() < rel_tol * mean)
+
+
+def build_int8_lut(codebook: torch.Tensor):
+    """int8 look-up table and step of a codebook for the int8 path: the rounded table of
+    build_int8_codebook for 1/2/4-bit codebooks; for 8-bit codebooks the identity w = idx - 128
+    with the uniform step, which is what the reference's IDENTITY_CB kernels compute
+    (quantization/wxa8/linear.py:130-159) and needs a uniform codebook (:79-98)."""
+    if codebook.numel() == 256:
+        if not is_uniform_codebook(codebook):
+            raise ValueError("the int8 path takes 8-bit weights only with a uniform codebook")
+        q = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8)
+        return q, uniform_codebook_step(codebook)
+    return build_int8_codebook(codebook)
+
+
 def build_fp8_codebook(codebook: torch.Tensor, n_coarse: int = 512):
     """(cb_e4m3, cb_scale) by the log-grid scale search of triton_kernels_fp8.py:35-87."""
     cb = codebook.detach().float().cpu()

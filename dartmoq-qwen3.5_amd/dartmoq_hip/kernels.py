@@ -18,7 +18,8 @@ import torch
 from . import hostprep, ops
 from ._lib import (EPI_STORE, MODE_A16, MODE_A8, MODE_FP4, MODE_FP8)
 from .hostprep import (build_e2m1_codebook, build_fp8_codebook, build_int8_codebook,  # noqa: F401
-                       generate_batch_rotation_matrices, generate_rotation_matrix)
+                       generate_batch_rotation_matrices, generate_rotation_matrix,
+                       is_uniform_codebook, uniform_codebook_step)
 from .moe import HipStageProfiler as CudaStageProfiler  # noqa: F401  (cuda_profiler.py:51-174)
 from .ops import fold_indices_to_e2m1  # noqa: F401  (triton_kernels_fp4.py:80-122)
 
@@ -110,7 +111,7 @@ def triton_fused_matmul_grouped_slice_rows_gf(x, indices_packed_gf, codebook, no
                                               bit_width: int = 4, x_is_rotated: bool = False,
                                               norms_prescaled: bool = False):
     """triton_kernels.py:1143-1251 (gate_up, one expert): rows [row_start, row_end) of the pool."""
-    _check_bit(bit_width, {1, 2, 4}, "slice_rows_gf")
+    _check_bit(bit_width, {1, 2, 4, 8}, "slice_rows_gf")
     _check_gs(group_size)
     if in_features % group_size:
         raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
@@ -131,7 +132,7 @@ def triton_fused_matmul_grouped_slice_in_features_gf(x, indices_packed_gf, codeb
                                                      norms_prescaled: bool = False):
     """triton_kernels.py:1254-1354 (down, one expert): groups [start/gs, end/gs) of the pool;
     rotates x with seed + original_start."""
-    _check_bit(bit_width, {1, 2, 4}, "slice_in_features_gf")
+    _check_bit(bit_width, {1, 2, 4, 8}, "slice_in_features_gf")
     _check_gs(group_size)
     if original_start % group_size or (original_end - original_start) % group_size:
         raise ValueError(f"slice [{original_start}, {original_end}) must align to group_size {group_size}")
@@ -151,7 +152,7 @@ def triton_fused_matmul_merged_rows_gf(x_rot, indices_packed_gf, codebook, norms
                                        group_size, in_features, bit_width: int = 4,
                                        norms_prescaled: bool = False, cfg=None):
     """triton_kernels.py:1482-1551: every expert of a bit pool in one launch (gate_up)."""
-    _check_bit(bit_width, {1, 2, 4}, "merged_rows_gf")
+    _check_bit(bit_width, {1, 2, 4, 8}, "merged_rows_gf")
     _check_gs(group_size)
     if in_features % group_size:
         raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
@@ -170,7 +171,7 @@ def triton_fused_matmul_merged_in_features_gf(x_rot, indices_packed_gf, codebook
                                               expert_info, group_size, bit_width: int = 4,
                                               norms_prescaled: bool = False, cfg=None):
     """triton_kernels.py:1554-1615: every expert of a bit pool in one launch (down)."""
-    _check_bit(bit_width, {1, 2, 4}, "merged_in_features_gf")
+    _check_bit(bit_width, {1, 2, 4, 8}, "merged_in_features_gf")
     _check_gs(group_size)
     info, g_slice, total = _info(expert_info, x_rot.device, "merged_in_features_gf")
     if g_slice < 2:
@@ -209,9 +210,10 @@ def _group_first_cached(indices_packed, norms, group_size, bit_width):
 def triton_fused_matmul_grouped(x, indices_packed, codebook, norms, seed, group_size, in_features,
                                 bit_width: int = 4):
     """triton_kernels.py:600-684, the kernel of WxA16Linear.forward: x[B, K] times the whole packed
-    matrix [N, K*bit/8] (row-major), group g rotated with seed + g*group_size.  in_features must
-    be a multiple of the group size (the reference's per-group fallback for ragged K is not built)."""
-    _check_bit(bit_width, {1, 2, 4}, "matmul_grouped")
+    matrix [N, K*bit/8] (row-major, bit 1/2/4/8), group g rotated with seed + g*group_size.
+    in_features must be a multiple of the group size (the reference's per-group fallback for ragged
+    K is not built)."""
+    _check_bit(bit_width, {1, 2, 4, 8}, "matmul_grouped")
     _check_gs(group_size)
     if in_features % group_size:
         raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
@@ -224,7 +226,7 @@ def triton_fused_matmul_grouped(x, indices_packed, codebook, norms, seed, group_
 def triton_fused_matmul_grouped_slice_rows(x, indices_packed, codebook, norms, seed, group_size,
                                            in_features, row_start, row_end, bit_width: int = 4):
     """triton_kernels.py:686-771: output rows [row_start, row_end) of a row-major packed matrix."""
-    _check_bit(bit_width, {1, 2, 4}, "slice_rows")
+    _check_bit(bit_width, {1, 2, 4, 8}, "slice_rows")
     _check_gs(group_size)
     if in_features % group_size:
         raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
@@ -239,7 +241,7 @@ def triton_fused_matmul_grouped_slice_in_features(x, indices_packed, codebook, n
                                                   full_in_features, bit_width: int = 4):
     """triton_kernels.py:774-860: input features [original_start, original_end) of a row-major
     packed matrix; x[B, end-start] is rotated with seed + original_start."""
-    _check_bit(bit_width, {1, 2, 4}, "slice_in_features")
+    _check_bit(bit_width, {1, 2, 4, 8}, "slice_in_features")
     _check_gs(group_size)
     if original_start % group_size:
         raise ValueError(f"original_start ({original_start}) must be aligned to group_size ({group_size})")
@@ -292,7 +294,7 @@ def quantize_act_e2m1_per32(x_rot):
 
 def _qa_slice_rows(mode, what, x_q, x_scale, idx_gf, lut, norms_gf, group_size, in_features, row_start,
                    row_end, bit_width, norms_prescaled, w_scale_byte=127):
-    _check_bit(bit_width, {1, 2, 4}, what)
+    _check_bit(bit_width, {1, 2, 4} if mode == MODE_FP4 else {1, 2, 4, 8}, what)
     _check_gs(group_size)
     b = x_q.shape[0]
     info = torch.tensor([[0, b, row_start, row_end - row_start]], dtype=torch.int32, device=x_q.device)
@@ -303,7 +305,7 @@ def _qa_slice_rows(mode, what, x_q, x_scale, idx_gf, lut, norms_gf, group_size, 
 
 def _qa_slice_in(mode, what, x_q, x_scale, idx_gf, lut, norms_gf, group_size, original_start,
                  original_end, bit_width, norms_prescaled, w_scale_byte=127):
-    _check_bit(bit_width, {1, 2, 4}, what)
+    _check_bit(bit_width, {1, 2, 4} if mode == MODE_FP4 else {1, 2, 4, 8}, what)
     _check_gs(group_size)
     if original_start % group_size or (original_end - original_start) % group_size:
         raise ValueError(f"slice [{original_start}, {original_end}) must align to group_size {group_size}")
@@ -317,7 +319,7 @@ def _qa_slice_in(mode, what, x_q, x_scale, idx_gf, lut, norms_gf, group_size, or
 
 def _qa_merged(mode, what, rows, x_q, x_scale, idx_gf, lut, norms_gf, expert_info, group_size,
                in_features, bit_width, norms_prescaled, cfg, w_scale_byte=127):
-    _check_bit(bit_width, {1, 2, 4}, what)
+    _check_bit(bit_width, {1, 2, 4} if mode == MODE_FP4 else {1, 2, 4, 8}, what)
     _check_gs(group_size)
     info, n_slice, total = _info(expert_info, x_q.device, what)
     if rows:
@@ -367,14 +369,27 @@ def wxa8_matmul_merged_in_features_gf(x_i8, x_scale, indices_packed_gf, codebook
                       norms_prescaled, cfg)
 
 
+_IDENTITY_CB: dict[str, torch.Tensor] = {}
+
+
+def _identity_cb(device) -> torch.Tensor:
+    """w = idx - 128 as a 256-entry int8 table: what the reference's IDENTITY_CB kernels compute
+    without a table (triton_kernels_a8.py:769-799)."""
+    key = str(device)
+    if key not in _IDENTITY_CB:
+        _IDENTITY_CB[key] = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8).to(device)
+    return _IDENTITY_CB[key]
+
+
 def wxa8_matmul_grouped_gf(x_i8, x_scale, indices_packed_gf, codebook_i8, norms_gf, group_size,
                            num_groups, bit_width: int = 8, identity_cb: bool = False, cfg=None):
     """triton_kernels_a8.py:769-799, the kernel of WxA8Linear.forward: the whole matrix, norms_gf
-    already divided by sqrt(group_size).  The 8-bit uniform codebook (identity_cb) of the attention
-    Linears is not built: bit widths 1/2/4 with an int8 look-up table only."""
-    if identity_cb or bit_width == 8:
-        raise ValueError("wxa8_matmul_grouped_gf: the 8-bit identity codebook is not built; "
-                         "bit_width must be 1/2/4")
+    already divided by sqrt(group_size).  With identity_cb (8-bit uniform codebook) codebook_i8 is
+    not read and the weights are idx - 128; the codebook step rides x_scale."""
+    if identity_cb:
+        if bit_width != 8:
+            raise ValueError("identity_cb needs bit_width 8")
+        codebook_i8 = _identity_cb(x_i8.device)
     return _qa_slice_rows(MODE_A8, "wxa8 grouped", x_i8, x_scale.half(), indices_packed_gf,
                           codebook_i8, norms_gf, group_size, num_groups * group_size, 0,
                           indices_packed_gf.shape[1], bit_width, True)
@@ -382,7 +397,7 @@ def wxa8_matmul_grouped_gf(x_i8, x_scale, indices_packed_gf, codebook_i8, norms_
 
 def wxfp8_matmul_grouped_gf(x_f8, x_scale, indices_packed_gf, cb_f8, norms_gf, group_size,
                             num_groups, bit_width: int, cfg=None):
-    """triton_kernels_fp8.py:407-428: the whole matrix (WxFP8Linear.forward); bit widths 1/2/4."""
+    """triton_kernels_fp8.py:407-428: the whole matrix (WxFP8Linear.forward)."""
     return _qa_slice_rows(MODE_FP8, "wxfp8 grouped", x_f8, x_scale.half(), indices_packed_gf, cb_f8,
                           norms_gf, group_size, num_groups * group_size, 0,
                           indices_packed_gf.shape[1], bit_width, True)

@@ -9,9 +9,9 @@ converts the checkpoint layout to group-first once (norms divided by sqrt(128)) 
 rotation matrices and the per-mode look-up table resident; a forward is two launches (rotate
 (+quantize), dequant GEMM) on the current stream.
 
-Bit widths 1, 2 and 4 with a codebook look-up are built.  The 8-bit uniform codebook of the
-attention Linears (bit_width 8, codebook_type "uniform") is not: constructing such a layer raises
-ValueError.
+Bit widths 1, 2, 4 and 8 are built, all through a codebook look-up.  8-bit weights run on the int8
+path only with a uniform codebook (then the table is the identity w = idx - 128 and the step rides
+the activation scale, the reference's IDENTITY_CB); the fp16 and e4m3 paths take any codebook.
 """
 
 from __future__ import annotations
@@ -31,8 +31,8 @@ class WxA16Linear:
                  packed_indices: torch.Tensor, codebook: torch.Tensor, norms: torch.Tensor, seed: int,
                  rotation: str = "qr", bias=None, orig_dtype: torch.dtype = torch.float16,
                  codebook_type: str = "lloydmax", device="cuda"):
-        if bit_width not in (1, 2, 4):
-            raise ValueError(f"bit_width must be 1/2/4, got {bit_width}")
+        if bit_width not in (1, 2, 4, 8):
+            raise ValueError(f"bit_width must be 1/2/4/8, got {bit_width}")
         if group_size != GROUP_SIZE:
             raise ValueError(f"group_size must be {GROUP_SIZE}, got {group_size}")
         if in_features % group_size:
@@ -91,6 +91,8 @@ class WxA16Linear:
         WxA8Linear.from_wxa16 (quantization/wxa8/linear.py:79-98)."""
         if not isinstance(linear, WxA16Linear):
             raise TypeError(f"expected WxA16Linear, got {type(linear)}")
+        if cls.MODE == MODE_A8 and linear.bit_width == 8 and not hostprep.is_uniform_codebook(linear.codebook):
+            raise ValueError("WxA8Linear takes 8-bit weights only with a uniform codebook")
         linear.__class__ = cls
         return linear
 
@@ -102,7 +104,7 @@ class WxA16Linear:
             if self.MODE == MODE_A16:
                 ctx = (self.codebook, 1.0)
             elif self.MODE == MODE_A8:
-                q, step = hostprep.build_int8_codebook(self.codebook)
+                q, step = hostprep.build_int8_lut(self.codebook)
                 ctx = (q.to(self.device), step)
             else:
                 q, scale = hostprep.build_fp8_codebook(self.codebook)

@@ -69,8 +69,8 @@ class BitPoolWeights:
         if mode == MODE_A16:
             ctx["gu_lut"], ctx["dn_lut"] = self.gu_codebook, self.dn_codebook
         elif mode == MODE_A8:
-            gq, gstep = hostprep.build_int8_codebook(self.gu_codebook)
-            dq, dstep = hostprep.build_int8_codebook(self.dn_codebook)
+            gq, gstep = hostprep.build_int8_lut(self.gu_codebook)
+            dq, dstep = hostprep.build_int8_lut(self.dn_codebook)
             ctx.update(gu_lut=gq.to(dev), dn_lut=dq.to(dev), gu_extra=gstep, dn_extra=dstep)
         elif mode == MODE_FP8:
             gq, gs_ = hostprep.build_fp8_codebook(self.gu_codebook)
@@ -140,8 +140,8 @@ class WxA16BitPartitionedGroupMoE:
         moe = cls(num_experts, hidden_size, intermediate_size, top_k, gate_weight, renormalize, device)
         for bit_str, p in pools.items():
             bit = int(bit_str)
-            if bit not in (1, 2, 4):
-                raise ValueError(f"bit_width must be 1/2/4, got {bit}")
+            if bit not in (1, 2, 4, 8):
+                raise ValueError(f"bit_width must be 1/2/4/8, got {bit}")
             offs = [int(v) for v in p["expert_offsets"]]
             if len(offs) != num_experts + 1:
                 raise ValueError("expert_offsets must have num_experts + 1 entries")
@@ -187,8 +187,8 @@ class WxA16BitPartitionedGroupMoE:
         if i_s % inter:
             raise ValueError(f"shared intermediate size {i_s} must be a multiple of {inter}")
         bit = int(gate["bit_width"])
-        if bit not in (1, 2, 4) or int(up["bit_width"]) != bit or int(down["bit_width"]) != bit:
-            raise ValueError(f"shared expert bit_width must be 1/2/4 and equal for gate/up/down, got {bit}")
+        if bit not in (1, 2, 4, 8) or int(up["bit_width"]) != bit or int(down["bit_width"]) != bit:
+            raise ValueError(f"shared expert bit_width must be 1/2/4/8 and equal for gate/up/down, got {bit}")
         if int(up["seed"]) != int(gate["seed"]):
             raise ValueError("gate and up of the shared expert must share the rotation seed")
         if not torch.equal(gate["codebook"].cpu().half(), up["codebook"].cpu().half()):
@@ -269,7 +269,9 @@ class WxA16BitPartitionedGroupMoE:
     def pool_mode(self, bit: int) -> int:
         mode = MODE_BY_NAME[self.MODE]
         if mode == MODE_FP4 and bit not in hostprep.FP4_BITS:
-            return MODE_A8                      # wxfp4/bit_partitioned_moe.py:50,296-299
+            # bit-2 pools (wxfp4/bit_partitioned_moe.py:50,296-299) and the 8-bit Linears of the
+            # shared expert (:8) stay on the int8 path
+            return MODE_A8
         return mode
 
     def _descriptor(self):

@@ -77,7 +77,7 @@ def convert_to_group_first(indices_packed, norms, group_size, bit_width, prescal
 
 
 def dequant_tile(idx_gf, codebook, norms_gf, g0, g_cnt, n0, n_cnt, bit_width):
-    _check_bit(bit_width)
+    _check_bit(bit_width, (1, 2, 4, 8))
     _need_cuda(idx_gf, codebook)
     out = torch.empty((g_cnt, n_cnt, GROUP_SIZE), dtype=torch.float16, device=idx_gf.device)
     check(load().dmq_dequant_tile(_ptr(idx_gf), _ptr(codebook.contiguous()), _ptr(norms_gf),
@@ -296,7 +296,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     for i, p in enumerate(pools):
         _need_cuda(p["act"], p["w"], p["norms"], p["expert_info"])
         dev = p["act"].device
-        _check_bit(p["bit"])
+        _check_bit(p["bit"], (1, 2, 4, 8))
         q = a.pool[i]
         q.w, q.norms = p["w"].data_ptr(), p["norms"].data_ptr()
         q.lut = p["lut"].data_ptr() if p["lut"] is not None else None
@@ -327,7 +327,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                   tiling=None, dbg_acc=None):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
-    _check_bit(bit)
+    _check_bit(bit, (1, 2, 4, 8))
     n_exp = expert_info.shape[0]
     if tt is None:
         tt = pick_tt(rows_total, n_exp)

@@ -14,7 +14,8 @@
  *
  * Conventions shared by all entry points
  *   group size            128 input features per quantization group
- *   bit                   1, 2 or 4 bits per codebook index (unpack also takes 8)
+ *   bit                   1, 2 or 4 bits per codebook index; 8 (the 256-entry codebooks of the
+ *                         quantized Linears) everywhere except the e2m1 fold and DMQ_MODE_FP4
  *   idx_gf                uint8 [G, N, 128*bit/8]  group-first packed indices
  *   norms_gf              fp16  [G, N]             per-(group,row) norms / sqrt(128)
  *   mode                  DMQ_MODE_A16 / A8 / FP8 / FP4
@@ -202,7 +203,8 @@ typedef struct {
   void* dbg_acc;            /* A8, tt == 1, ks == 1, STORE only: int32 [rows, groups, n_out] or NULL */
 } dmq_gemm_args;
 
-/* Merged dequant GEMM: one launch for all bit pools of a layer that share `mode`.  Stands in for
+/* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more
+ * for its 8-bit pools (never split over K).  Stands in for
  *   triton_fused_matmul_merged_rows_gf / _merged_in_features_gf   (triton_kernels.py:1482-1615)
  *   wxa8_matmul_merged_rows_gf / _merged_in_features_gf           (triton_kernels_a8.py:959-1068)
  *   wxfp8_matmul_merged_rows_gf / _merged_in_features_gf          (triton_kernels_fp8.py:641-750)

@@ -80,7 +80,7 @@ def test_linear_constructor_errors():
     import dartmoq_hip
     packed = _packed(128, 256, 2, seed=3)
     with pytest.raises(ValueError):
-        dartmoq_hip.WxA16Linear(256, 128, 8, 128, packed["indices_packed"], packed["codebook"],
+        dartmoq_hip.WxA16Linear(256, 128, 3, 128, packed["indices_packed"], packed["codebook"],
                                 packed["norms"], 1)
     with pytest.raises(ValueError):
         dartmoq_hip.WxA16Linear(256, 128, 2, 64, packed["indices_packed"], packed["codebook"],
@@ -127,7 +127,7 @@ def test_unsliced_callables_by_reference_names():
                                                            128, 384, 512, 2)
     assert relerr(part.float().cpu(), xs.float() @ w[:, 128:384].T) < 2e-3
     with pytest.raises(ValueError):
-        K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, 512, 8)
+        K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, 512, 3)
     with pytest.raises(ValueError):
         K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, 500, 2)
     with pytest.raises(ValueError):
@@ -142,8 +142,80 @@ def test_unsliced_callables_by_reference_names():
     o8 = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, cb_i8.cuda(), norms_pre, 128, 4, 2)
     assert relerr(o8.float().cpu(), _dataflow(packed, x, "wxa8")) < 6e-3
     with pytest.raises(ValueError):
-        K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, cb_i8.cuda(), norms_pre, 128, 4, 8, identity_cb=True)
+        K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, cb_i8.cuda(), norms_pre, 128, 4, 2, identity_cb=True)
     cb_f8, sc = K.build_fp8_codebook(packed["codebook"])
     x_f8, x_s8 = K.rotate_quantize_fused_fp8(x.cuda(), rot, 128, 4, extra_scale=sc)
     of8 = K.wxfp8_matmul_grouped_gf(x_f8, x_s8, idx_gf, cb_f8.cuda(), norms_pre, 128, 4, 2)
     assert relerr(of8.float().cpu(), _dataflow(packed, x, "wxfp8")) < 2e-2
+
+
+# ----------------------------------------------------------------------------- 8-bit codebooks
+
+def _packed8(n, k, seed, uniform):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(n, k, generator=g) * 0.02).half()
+    return turboquant.quantize_packed(w, 8, 128, seed=seed + 5, uniform_codebook=uniform)
+
+
+@pytest.mark.parametrize("uniform", [True, False])
+@pytest.mark.parametrize("rows", [3, 40, 200])
+def test_wxa16_linear_8bit(uniform, rows):
+    """8-bit indices (the attention / shared-expert Linears of a real checkpoint), uniform grid
+    and 256-level Lloyd-Max, through the 256-entry fp16 table."""
+    import dartmoq_hip
+    packed = _packed8(256, 384, seed=2, uniform=uniform)
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed)
+    x = torch.randn(rows, 384, generator=torch.Generator().manual_seed(rows)).half()
+    out = lin(x.cuda()).float().cpu()
+    ref = x.float() @ turboquant.dequantize_packed(packed).T
+    assert relerr(out, ref) < 2e-3
+    assert max_rel(out, ref) <= 1e-2 and cosine(out, ref) >= 0.9999
+
+
+def test_dequant_tile_8bit_is_exact():
+    from dartmoq_hip import ops
+    from oracle import packing
+    packed = _packed8(64, 256, seed=9, uniform=True)
+    idx_gf, norms_gf = packing.convert_to_group_first(packed["indices_packed"], packed["norms"], 128, 8)
+    tile = ops.dequant_tile(idx_gf.cuda(), packed["codebook"].cuda(), None, 0, 2, 0, 64, 8).cpu()
+    want = packed["codebook"][idx_gf.long()]                      # [G, N, 128] one index per byte
+    assert torch.equal(tile, want)
+
+
+def test_wxa8_linear_8bit_identity_codebook():
+    """int8 path on 8-bit uniform weights: w = idx - 128, step folded into the activation scale
+    (the reference's IDENTITY_CB); a Lloyd-Max 8-bit codebook is refused like the reference does."""
+    import dartmoq_hip
+    from dartmoq_hip import kernels as K
+    packed = _packed8(256, 512, seed=4, uniform=True)
+    lin = dartmoq_hip.WxA8Linear.from_wxa16(dartmoq_hip.WxA16Linear.from_packed(packed))
+    x = torch.randn(70, 512, generator=torch.Generator().manual_seed(1)).half()
+    out = lin(x.cuda()).float().cpu()
+    ideal = _dataflow(packed, x, "wxa8")
+    assert relerr(out, ideal) < 6e-3
+    ref = x.float() @ turboquant.dequantize_packed(packed).T
+    assert relerr(out, ref) < 0.02
+    # the reference-named kernel with identity_cb=True: same numbers from explicit pieces
+    idx_gf, norms_gf = K.convert_to_group_first(packed["indices_packed"].cuda(), packed["norms"].cuda(), 128, 8)
+    norms_pre = (norms_gf.float() / 128 ** 0.5).half()
+    rot = K.generate_batch_rotation_matrices(128, packed["seed"], 4, 128, device="cuda")
+    step = K.uniform_codebook_step(packed["codebook"])
+    assert step == pytest.approx(3.5 / 128, rel=1e-3) and K.is_uniform_codebook(packed["codebook"])
+    x_i8, x_s = K.rotate_quantize_fused(x.cuda(), rot, 128, 4, extra_scale=step)
+    dummy = torch.zeros(256, dtype=torch.int8, device="cuda")
+    o = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, dummy, norms_pre, 128, 4, 8, identity_cb=True)
+    assert torch.equal(o, lin(x.cuda()))
+    lloyd = _packed8(128, 256, seed=4, uniform=False)
+    with pytest.raises(ValueError):
+        dartmoq_hip.WxA8Linear.from_wxa16(dartmoq_hip.WxA16Linear.from_packed(lloyd))
+
+
+@pytest.mark.parametrize("uniform", [True, False])
+def test_wxfp8_linear_8bit(uniform):
+    import dartmoq_hip
+    packed = _packed8(128, 256, seed=6, uniform=uniform)
+    lin = dartmoq_hip.WxFP8Linear.from_wxa16(dartmoq_hip.WxA16Linear.from_packed(packed))
+    x = torch.randn(33, 256, generator=torch.Generator().manual_seed(2)).half()
+    out = lin(x.cuda()).float().cpu()
+    assert relerr(out, _dataflow(packed, x, "wxfp8")) < 2e-2
+    assert relerr(out, x.float() @ turboquant.dequantize_packed(packed).T) < 0.075

@@ -122,6 +122,22 @@ def test_layer_with_shared_expert(shared_layer, mode, tokens, tt):
     assert relerr(routed_only, ideal) > 0.1
 
 
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
+@pytest.mark.parametrize("tokens", [1, 90])
+def test_layer_with_8bit_shared_expert(small_layer, mode, tokens):
+    """The shared expert of a real checkpoint is quantized with the 8-bit uniform codebook: its
+    slices are work items of separate launches for 8-bit pools (int8 path under wxfp4)."""
+    import dataclasses
+    layer = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter,
+                                  seed=31, bit=8, uniform_codebook=True)
+    x, idx, w, out = _run(layer, mode, tokens, seed=9 + tokens)
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    ref = moe.reference_forward(layer, x, idx, w)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+    assert relerr(out, ref) < MODE_BOUND[mode], (mode, relerr(out, ref))
+
+
 def dataclasses_replace_shared(layer):
     import dataclasses
     return dataclasses.replace(layer, shared=None)

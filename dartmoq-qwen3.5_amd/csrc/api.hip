@@ -34,7 +34,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 6; }
+int dmq_abi_version(void) { return 7; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -319,6 +319,17 @@ int dmq_finalize_f16(const void* acc_f32, const void* add_f16, long n, void* out
   if (n % 4) return DMQ_ERR_ALIGN;
   return dmq_finalize_launch((const float*)acc_f32, (const __half*)add_f16, n, (__half*)out_f16,
                              (hipStream_t)stream);
+}
+
+int dmq_rms_norm(const void* x, int x_bf16, const void* weight, int weight_fp32, long rows, int n,
+                 long x_row_stride, long out_row_stride, float eps, void* out, void* stream) {
+  if (rows <= 0) return DMQ_OK;
+  if (!x || !weight || !out) return DMQ_ERR_NULL;
+  if (n <= 0) return DMQ_ERR_SHAPE;
+  if (n % 8 || x_row_stride % 8 || out_row_stride % 8) return DMQ_ERR_ALIGN;
+  if (x_row_stride < n || out_row_stride < n) return DMQ_ERR_SHAPE;
+  return dmq_rms_norm_launch(x, x_bf16, weight, weight_fp32, rows, n, x_row_stride, out_row_stride,
+                             eps, out, (hipStream_t)stream);
 }
 
 int dmq_fill_zero(void* ptr, long n_bytes, void* stream) {

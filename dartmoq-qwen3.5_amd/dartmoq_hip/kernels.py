@@ -86,6 +86,14 @@ def _gemm(mode, bit, x_codes, x_scale, w_gf, norms, lut, info, *, groups, n_out,
                              rows_total=rows_total, w_scale_byte=w_scale_byte, tt=tt)
 
 
+# ----------------------------------------------------------------------------- norm
+
+def rms_norm(x, weight, eps):
+    """turboquant_utils/norm_kernels.py:183-209 (Qwen3_5MoeRMSNorm.forward, the norm that feeds the
+    MoE block): (x * rsqrt(mean(x^2) + eps) * (1 + weight)).type_as(x), fp32 inside."""
+    return ops.rms_norm(x, weight, eps)
+
+
 # ----------------------------------------------------------------------------- layout / rotation
 
 def convert_to_group_first(indices_packed, norms, group_size, bit_width):

@@ -366,3 +366,27 @@ def finalize_f16(acc32: torch.Tensor, add: torch.Tensor | None = None) -> torch.
     check(load().dmq_finalize_f16(_ptr(acc32), _ptr(add), acc32.numel(), _ptr(out),
                                   _stream(acc32.device)), "finalize_f16")
     return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """out = x * rsqrt(mean(x^2, -1) + eps) * (1 + weight) in fp32, rounded once to x.dtype
+    (fp16 or bf16).  Rows may be strided (a chunk view) as long as their elements are contiguous."""
+    _need_cuda(x, weight)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("rms_norm takes fp16 or bf16 activations")
+    n = x.shape[-1]
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    x2 = x.reshape(-1, n) if x.is_contiguous() else x
+    if x2.dim() != 2:
+        x2 = x.contiguous().reshape(-1, n)
+    if weight.dtype not in (x.dtype, torch.float32):
+        weight = weight.float()
+    weight = weight.contiguous()
+    if weight.numel() != n:
+        raise ValueError("weight must hold one value per feature")
+    out = torch.empty((x2.shape[0], n), dtype=x.dtype, device=x.device)
+    check(load().dmq_rms_norm(_ptr(x2), int(x.dtype == torch.bfloat16), _ptr(weight),
+                              int(weight.dtype == torch.float32), x2.shape[0], n, x2.stride(0), n,
+                              float(eps), _ptr(out), _stream(x.device)), "rms_norm")
+    return out.reshape(x.shape)

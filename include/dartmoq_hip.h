@@ -49,7 +49,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 6). */
+/* Library / build identification: returns the ABI version (currently 7). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -219,6 +219,13 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* args, void* stream);
  * bit_partitioned_moe.py:967 with a fixed summation order and an fp32 sum.  hidden % 8 == 0. */
 int dmq_combine_slots(const void* slots_f16, int k, const void* add_f16, long tokens, int hidden,
                       void* out_f16, void* stream);
+
+/* rms_norm of turboquant_utils/norm_kernels.py:79-117, :183-209 (Qwen3_5MoeRMSNorm.forward: the
+ * norm in front of the MoE block): out = x * rsqrt(mean(x^2) + eps) * (1 + weight) in fp32, one
+ * rounding to the activation type.  x / out fp16 (x_bf16 == 0) or bf16 [rows, n] with the given
+ * row strides in elements; weight [n] in the activation type or fp32.  n and strides % 8 == 0. */
+int dmq_rms_norm(const void* x, int x_bf16, const void* weight, int weight_fp32, long rows, int n,
+                 long x_row_stride, long out_row_stride, float eps, void* out, void* stream);
 
 /* fp16(out32 (+ add16)) over n elements (n % 4 == 0). */
 int dmq_finalize_f16(const void* acc_f32, const void* add_f16, long n, void* out_f16, void* stream);

@@ -32,6 +32,8 @@ actquant.quantize_act_e2m1             8-point grid brute force, tie rule
 routing.*                              torch.topk / stable sort, invariants
 moe.reference_forward                  dense fp32 MoE on dequantized weights
 moe.quantized_forward (A8/FP8/FP4)     published module-level relerr anchors
+moe.shared_quantized_forward           dense SwiGLU MLP on dequantized Linears
+norm.rms_norm                          unit RMS, scale invariance, hand case
 =====================================  =======================================
 
 The Triton code generation boundary of the reference (tl.dot accumulation
@@ -39,4 +41,4 @@ order, fp16 accumulators) is not restated: parity unpinned there by design,
 fp16 outputs are compared within the stated tolerance against fp32 maths.
 """
 
-from . import codebook, packing, rotation, turboquant, luts, actquant, routing, moe  # noqa: F401
+from . import codebook, packing, rotation, turboquant, luts, actquant, routing, moe, norm  # noqa: F401

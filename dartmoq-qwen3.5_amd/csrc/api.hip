@@ -34,7 +34,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 7; }
+int dmq_abi_version(void) { return 8; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -319,6 +319,18 @@ int dmq_finalize_f16(const void* acc_f32, const void* add_f16, long n, void* out
   if (n % 4) return DMQ_ERR_ALIGN;
   return dmq_finalize_launch((const float*)acc_f32, (const __half*)add_f16, n, (__half*)out_f16,
                              (hipStream_t)stream);
+}
+
+int dmq_quantize_weights(const void* w_f16, long w_row_stride, const void* rot_f32,
+                         const void* boundaries_f32, int n_rows, int groups, int bit,
+                         void* indices_packed, void* norms_f16, void* stream) {
+  if (!dmq_valid_bit_wide(bit)) return DMQ_ERR_BIT;
+  if (n_rows <= 0 || groups <= 0) return DMQ_ERR_SHAPE;
+  if (!w_f16 || !rot_f32 || !boundaries_f32 || !indices_packed || !norms_f16) return DMQ_ERR_NULL;
+  if (w_row_stride % 8 || w_row_stride < (long)groups * DMQ_GS) return DMQ_ERR_ALIGN;
+  return dmq_quantize_weights_launch((const __half*)w_f16, w_row_stride, (const float*)rot_f32,
+                                     (const float*)boundaries_f32, n_rows, groups, bit,
+                                     (uint8_t*)indices_packed, (__half*)norms_f16, (hipStream_t)stream);
 }
 
 int dmq_rms_norm(const void* x, int x_bf16, const void* weight, int weight_fp32, long rows, int n,

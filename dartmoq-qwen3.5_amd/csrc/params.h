@@ -126,6 +126,9 @@ int dmq_group_first_launch(const uint8_t* idx, const __half* norms, int n_rows, 
                            int prescale, uint8_t* idx_gf, __half* norms_gf, hipStream_t s);
 int dmq_fold_e2m1_launch(const uint8_t* idx_gf, const uint8_t* nib, long rows, int bit, uint8_t* out,
                          hipStream_t s);
+int dmq_quantize_weights_launch(const __half* w, long w_stride, const float* rot, const float* bounds,
+                                int n_rows, int groups, int bit, uint8_t* idx_out, __half* norms_out,
+                                hipStream_t s);
 int dmq_rms_norm_launch(const void* x, int bf16, const void* weight, int weight_fp32, long rows, int n,
                         long x_stride, long out_stride, float eps, void* out, hipStream_t s);
 int dmq_finalize_launch(const float* acc, const __half* add, long n, __half* out, hipStream_t s);

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 7
+ABI_VERSION = 8
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER = 0, 1, 2
@@ -102,6 +102,8 @@ PROTOTYPES = {
     "dmq_combine_slots": (c_int, [c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p]),
     "dmq_finalize_f16": (c_int, [c_void_p, c_void_p, c_long, c_void_p, c_void_p]),
     "dmq_fill_zero": (c_int, [c_void_p, c_long, c_void_p]),
+    "dmq_quantize_weights": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p,
+                                     c_void_p, c_void_p]),
     "dmq_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_long, c_long, c_float,
                              c_void_p, c_void_p]),
     "dmq_moe_workspace_bytes": (c_size_t, [POINTER(LayerDesc), c_int]),

@@ -390,3 +390,29 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
                               int(weight.dtype == torch.float32), x2.shape[0], n, x2.stride(0), n,
                               float(eps), _ptr(out), _stream(x.device)), "rms_norm")
     return out.reshape(x.shape)
+
+
+def quantize_weights(w: torch.Tensor, rot_f32: torch.Tensor, boundaries: torch.Tensor, bit_width: int):
+    """TurboQuant quantizer on the GPU: w fp16 [N, K], rot fp32 [K/128, 128, 128], boundaries fp32
+    [2^bit - 1] -> (indices_packed u8 [N, K*bit/8], norms fp16 [N, K/128])."""
+    _check_bit(bit_width, (1, 2, 4, 8))
+    _need_cuda(w, rot_f32, boundaries)
+    if w.dtype != torch.float16:
+        w = w.half()
+    w = w.contiguous()
+    n, k = w.shape
+    groups = k // GROUP_SIZE
+    if k != groups * GROUP_SIZE:
+        raise ValueError(f"K ({k}) must be a multiple of {GROUP_SIZE}")
+    rot_f32 = rot_f32.float().contiguous()
+    boundaries = boundaries.float().contiguous()
+    if tuple(rot_f32.shape) != (groups, GROUP_SIZE, GROUP_SIZE):
+        raise ValueError(f"rot must be {(groups, GROUP_SIZE, GROUP_SIZE)}, got {tuple(rot_f32.shape)}")
+    if boundaries.numel() != (1 << bit_width) - 1:
+        raise ValueError(f"{(1 << bit_width) - 1} boundaries expected, got {boundaries.numel()}")
+    idx = torch.empty((n, k * bit_width // 8), dtype=torch.uint8, device=w.device)
+    norms = torch.empty((n, groups), dtype=torch.float16, device=w.device)
+    check(load().dmq_quantize_weights(_ptr(w), w.stride(0), _ptr(rot_f32), _ptr(boundaries), n, groups,
+                                      bit_width, _ptr(idx), _ptr(norms), _stream(w.device)),
+          "quantize_weights")
+    return idx, norms

@@ -49,7 +49,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 7). */
+/* Library / build identification: returns the ABI version (currently 8). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -81,6 +81,18 @@ int dmq_dequant_tile(const void* idx_gf, const void* codebook_f16, const void* n
  * idx_gf [rows, 128*bit/8] -> out [rows, 64], rows = G*N. */
 int dmq_fold_indices_to_e2m1(const void* idx_gf, const void* nib_lut, long rows, int bit,
                              void* out, void* stream);
+
+/* turboquant_quantize_packed_full, turboquant_utils/quantize.py:350-474 (rotation "qr"): per row
+ * and group of 128 features norm = max(||w||, 1e-8), Y = (w / norm) . P_g^T . sqrt(128),
+ * index = clamp(number of boundaries < Y, 0, 2^bit - 1), packed low bits first.
+ *   w fp16 [n_rows, w_row_stride >= groups*128]; rot fp32 [groups, 128, 128] (the matrices of
+ *   seeds seed + g*128); boundaries fp32 [2^bit - 1] ascending (codebook.py:77-100, or the uniform
+ *   grid of quantize.py:394-402); indices_packed u8 [n_rows, groups*128*bit/8]; norms fp16
+ *   [n_rows, groups].  bit 1, 2, 4 or 8.  The product runs on the fp32 matrix cores: indices equal
+ *   the torch quantizer's except where Y sits within fp32 rounding of a boundary. */
+int dmq_quantize_weights(const void* w_f16, long w_row_stride, const void* rot_f32,
+                         const void* boundaries_f32, int n_rows, int groups, int bit,
+                         void* indices_packed, void* norms_f16, void* stream);
 
 /* ------------------------------------------------------------------ routing */
 

@@ -131,6 +131,8 @@ class WxA16Linear:
         x2 = x.reshape(-1, self.in_features)
         src = x2 if x2.dtype == torch.float16 else x2.half()
         rows = src.shape[0]
+        if rows == 0:
+            return torch.empty(*shape[:-1], self.out_features, dtype=x.dtype, device=x.device)
         lut, extra = self._mode_ctx()
         codes, scale = ops.rotate(self.MODE, src, self.rot, extra_scale=extra, scale_fp32=False)
         out = ops.matmul_merged(self.MODE, self.bit_width, EPI_STORE, codes,

@@ -393,6 +393,8 @@ class WxA16BitPartitionedGroupMoE:
             x = x.half()
         x = x.contiguous()
         tokens = x.shape[0]
+        if tokens == 0:                         # an empty batch has an empty output
+            return torch.empty(shape, dtype=orig_dtype, device=x.device)
         router, keep = self._router_args(x, router_logits, topk_idx, topk_w)
         desc = self._descriptor()[0]
         ws = self._get_workspace(tokens)

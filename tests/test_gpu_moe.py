@@ -256,3 +256,25 @@ def test_forward_is_graph_capturable(small_layer, tokens):
         other = mod.forward(x.flip(0).contiguous(), router_logits=logits.flip(0).contiguous())
         torch.cuda.synchronize()
         assert torch.equal(other.flip(0), ref)
+
+
+def test_empty_batch_and_3d_input(small_layer):
+    """Zero tokens give an empty output; [batch, seq, hidden] inputs keep their shape (the
+    reference reshapes to [-1, hidden] and back, bit_partitioned_moe.py:1068-1069)."""
+    import dartmoq_hip
+    mod = make_module(small_layer, "wxa16")
+    h, e = small_layer.hidden, small_layer.num_experts
+    out = mod.forward(torch.zeros(0, h, dtype=torch.float16, device="cuda"),
+                      router_logits=torch.zeros(0, e, device="cuda"))
+    assert out.shape == (0, h) and out.dtype == torch.float16
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2, 7, h, generator=g).half().cuda()
+    logits = torch.randn(14, e, generator=g).cuda()
+    y3 = mod.forward(x, router_logits=logits)
+    y2 = mod.forward(x.reshape(14, h), router_logits=logits)
+    assert y3.shape == (2, 7, h) and torch.equal(y3.reshape(14, h), y2)
+    yb = mod.forward(x.bfloat16(), router_logits=logits)
+    assert yb.dtype == torch.bfloat16 and yb.shape == (2, 7, h)
+    packed = next(iter(small_layer.pools.values())).down
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed)
+    assert lin(torch.zeros(0, lin.in_features, dtype=torch.float16, device="cuda")).shape == (0, lin.out_features)

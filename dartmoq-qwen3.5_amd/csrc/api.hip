@@ -34,7 +34,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 8; }
+int dmq_abi_version(void) { return 9; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -229,10 +229,10 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     (b == 8 ? any_wide : any_narrow) = true;
   }
   if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
-  if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SCATTER) return DMQ_ERR_MODE;
+  if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SILU_ROT) return DMQ_ERR_MODE;
   const int ks = a->ks > 0 ? a->ks : 1;
   if (!dmq_gemm_config_ok(a->tt, ks)) return DMQ_ERR_MODE;
-  if (!a->items || !a->n_items || !a->out) return DMQ_ERR_NULL;
+  if (!a->items || !a->n_items || (!a->out && a->epi != DMQ_EPI_SILU_ROT)) return DMQ_ERR_NULL;
   for (int i = 0; i < a->n_pools; ++i) {
     const dmq_gemm_pool& q = a->pool[i];
     if (!q.act || !q.w || !q.norms || !q.expert_info) return DMQ_ERR_NULL;
@@ -243,18 +243,27 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (a->epi == DMQ_EPI_SCATTER && (!a->row_weight || !a->row_slot)) return DMQ_ERR_NULL;
   if (a->max_items <= 0) return DMQ_ERR_EMPTY;
   if (a->groups <= 0 || a->n_out <= 0) return DMQ_ERR_SHAPE;
-  const int feat_per_wave = (a->epi == DMQ_EPI_SILU) ? 32 : 64;
+  const bool silu = a->epi == DMQ_EPI_SILU || a->epi == DMQ_EPI_SILU_ROT;
+  const int feat_per_wave = silu ? 32 : 64;
   if (a->n_out % feat_per_wave) return DMQ_ERR_ALIGN;
-  if (a->epi == DMQ_EPI_SILU && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
+  if (silu && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
+  if (a->epi == DMQ_EPI_SILU_ROT) {
+    if (ks != 1 || any_wide) return DMQ_ERR_MODE;
+    if (a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
+    if (!a->post_out || (a->mode != DMQ_MODE_A16 && !a->post_scale)) return DMQ_ERR_NULL;
+    for (int i = 0; i < a->n_pools; ++i)
+      if (a->pool[i].mode == a->mode && !a->post_rot[i]) return DMQ_ERR_NULL;
+  }
   if (a->act_row_bytes < (long)a->groups * act_bytes_per_group(a->mode)) return DMQ_ERR_SHAPE;
 
   GemmLaunch L;
   GemmParams& p = L.p;
   for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
     const dmq_gemm_pool& q = a->pool[i < a->n_pools ? i : 0];
+    const int qi = i < a->n_pools ? i : 0;
     p.pool[i] = PoolW{(const uint8_t*)q.w, (const __half*)q.norms, q.lut, (const int*)q.expert_info,
                       (const uint8_t*)q.act, q.act_scale, (const int*)q.row_index, q.n_total, q.bit,
-                      q.mode, q.w_scale_byte};
+                      q.mode, q.w_scale_byte, (const __half*)a->post_rot[qi], a->post_extra_scale[qi]};
   }
   p.act_row_bytes = a->act_row_bytes;
   p.act_scale_stride = a->act_scale_stride;
@@ -270,6 +279,10 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.row_weight = (const float*)a->row_weight;
   p.row_slot = (const int*)a->row_slot;
   p.dbg_acc = (int*)a->dbg_acc;
+  p.post_out = (uint8_t*)a->post_out;
+  p.post_row_bytes = a->post_row_bytes;
+  p.post_scale = a->post_scale;
+  p.post_scale_stride = a->post_scale_stride;
   L.epi = a->epi;
   L.tt = a->tt;
   L.dbg = a->dbg_acc != nullptr;
@@ -490,6 +503,15 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if (!seen) modes[n_modes++] = m;
   }
 
+  // The gate_up GEMM rotates (and quantizes) its SiLU*up rows for the down projection itself when
+  // a workgroup owns whole blocks of 128 features: no K split, no 8-bit pools in the mode.
+  bool fuse_rot[DMQ_MAX_POOLS];
+  for (int mi = 0; mi < n_modes; ++mi) {
+    fuse_rot[mi] = (ks == 1);
+    for (int i = 0; i < P; ++i)
+      if (layer->pool[i].mode == modes[mi] && layer->pool[i].bit == 8) fuse_rot[mi] = false;
+  }
+
   // 1. top-k (when the router hands over logits), shared columns, sort by expert, per-pool
   //    expert_info, work items: one launch for small batches
   {
@@ -569,10 +591,13 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
     dmq_gemm_args g{};
-    g.mode = mode; g.epi = DMQ_EPI_SILU; g.tt = tt; g.ks = ks; g.nbl = nbl; g.n_pools = P;
+    g.mode = mode; g.epi = fuse_rot[mi] ? DMQ_EPI_SILU_ROT : DMQ_EPI_SILU;
+    g.tt = tt; g.ks = ks; g.nbl = nbl; g.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = pd.major != 0;
+      g.post_rot[i] = pd.dn_rot;
+      g.post_extra_scale[i] = pd.dn_extra_scale;
       g.pool[i] = dmq_gemm_pool{pd.gu_w, pd.gu_norms, pd.gu_lut, w.gu_info + (size_t)i * E * 4,
                                 hoisted ? w.xq[i] : w.xq_rows,
                                 hoisted ? w.xq_scale[i] : w.xq_rows_scale,
@@ -584,15 +609,18 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     g.groups = H / DMQ_GS; g.n_out = I; g.half_width = I; g.slice_is_groups = 0;
     g.items = w.items; g.n_items = w.n_items; g.max_items = w.max_items;
     g.out = w.act; g.out_stride = I;
+    g.post_out = w.actq; g.post_row_bytes = (long)I * 2;
+    g.post_scale = w.actq_scale; g.post_scale_stride = scale_stride_for(mode, I);
     rc = dmq_matmul_merged_gf(&g, stream);
     if (rc) return rc;
   }
 
   mark(3);
 
-  // 4. down input: per-expert rotation (+quantize) of act
+  // 4. down input: per-expert rotation (+quantize) of act, unless the gate_up launch did it
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
+    if (fuse_rot[mi]) continue;
     RotParams rp{};
     rp.x = (const __half*)w.act; rp.x_stride = I; rp.row_index = nullptr;
     rp.rows = 0; rp.groups = I / DMQ_GS; rp.n_hoisted = 0; rp.hoisted_items_per_pool = 1;

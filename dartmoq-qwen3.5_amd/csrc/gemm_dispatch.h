@@ -44,6 +44,9 @@ static int dmq_gemm_launch_epi(const GemmLaunch& L) {
       }
       return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_STORE, false>(L);
     case DMQ_EPI_SILU: return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_SILU, false>(L);
+    case DMQ_EPI_SILU_ROT:
+      if constexpr (KS == 1) return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_SILU_ROT, false>(L);
+      return DMQ_ERR_MODE;
     case DMQ_EPI_SCATTER: return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_SCATTER, false>(L);
   }
   return DMQ_ERR_MODE;

@@ -63,6 +63,11 @@ struct PoolW {
   int bit;
   int mode;                    // items of pools whose mode differs from the kernel's are skipped
   int w_scale_byte;            // FP4: constant e8m0 byte of the weight blocks
+  // DMQ_EPI_SILU_ROT: rotation matrices [groups_total, 128, 128] fp16 applied to the SiLU*up rows
+  // (matrix of block b of an item = post_rot[item's down slice + b]) and the scale factor folded
+  // into the stored activation scale
+  const __half* post_rot;
+  float post_extra;
 };
 
 struct GemmParams {
@@ -85,6 +90,11 @@ struct GemmParams {
   const float* row_weight;     // SCATTER: routing weight of logical row r
   const int* row_slot;         // SCATTER: destination row (token * top_k + slot) of logical row r
   int* dbg_acc;                // optional int32 [rows, groups, n_out] per-group accumulators (A8)
+  // DMQ_EPI_SILU_ROT: rotated (+ quantized) rows: codes [rows, post_row_bytes], scales
+  uint8_t* post_out;
+  long post_row_bytes;
+  void* post_scale;            // A8/FP8: fp16 [rows, post_scale_stride]; FP4: u8 [rows, post_scale_stride]
+  int post_scale_stride;
 };
 
 template <int MODE> struct ModeTraits;
@@ -178,6 +188,16 @@ template <int WW, int TT> constexpr int dmq_ring_depth() {
 }
 
 // Tiling facts shared by the kernel and its host launcher.
+// Bytes of LDS the fused down-rotation epilogue needs beyond the staging slots: the fp16 SiLU*up
+// tile of the block (16*TT rows x 256 B; fp16 layers reuse a staging slot of that very size) and
+// the per-wave row maxima of the quantizers.
+template <int MODE, int TT, int EPI> struct PostGeom {
+  static constexpr bool ON = (EPI == DMQ_EPI_SILU_ROT);
+  static constexpr int TILE = (ON && MODE != DMQ_MODE_A16) ? 16 * TT * 256 : 0;
+  static constexpr int WMAX = (ON && MODE != DMQ_MODE_A16) ? 4 * 16 * TT * 4 : 0;
+  static constexpr int BYTES = (TILE + WMAX) > 16 ? (TILE + WMAX) : 16;
+};
+
 template <int MODE, int NT, int TT, int KS> struct GemmGeom {
   static constexpr int AW = ModeTraits<MODE>::ACT_WORDS;          // activation words per lane and group
   static constexpr int AB = AW * 16;                              // activation bytes per row and group
@@ -193,8 +213,9 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
 
 template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
-                                              uint8_t* smem2, int token_start, int token_count,
-                                              int slice_start, int ttile, int nb, int nbc) {
+                                              uint8_t* smem2, uint8_t* smem_post, int token_start,
+                                              int token_count, int slice_start, int post_slice,
+                                              int ttile, int nb, int nbc) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   using GG = GemmGeom<MODE, NT, TT, KS>;
@@ -204,7 +225,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr bool STAGE = GG::STAGE;
   constexpr int PF = GG::PF;
   constexpr int ROWPARTS = 4 / KS;                                   // waves along the features
-  constexpr int UNIT = (EPI == DMQ_EPI_SILU) ? 2 : 1;                // tiles finalized together
+  constexpr bool SILU = (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT);
+  constexpr int UNIT = SILU ? 2 : 1;                                 // tiles finalized together
   constexpr int UNITS = NT / UNIT;
   constexpr int FEAT_TILES = NT / UNIT;                              // output tiles per wave
   constexpr int PPG = (MODE == DMQ_MODE_FP4) ? 64 : (DMQ_GS * BIT / 8);
@@ -228,7 +250,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   int wrow[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    if (EPI == DMQ_EPI_SILU) wrow[j] = slice_start + ((j & 1) ? p.half_width : 0) + featw + (j >> 1) * 16;
+    if (SILU) wrow[j] = slice_start + ((j & 1) ? p.half_width : 0) + featw + (j >> 1) * 16;
     else wrow[j] = (p.slice_is_groups ? 0 : slice_start) + featw + j * 16;
   }
   const int g_base = p.slice_is_groups ? slice_start : 0;
@@ -428,7 +450,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
           half4_t h = {(_Float16)total_acc[j][t][0], (_Float16)total_acc[j][t][1],
                        (_Float16)total_acc[j][t][2], (_Float16)total_acc[j][t][3]};
           *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat_k + j * 16 + 4 * q) = h;
-        } else if (EPI == DMQ_EPI_SILU) {
+        } else if (SILU) {
           half4_t h;
 #pragma unroll
           for (int r = 0; r < 4; ++r)
@@ -497,7 +519,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     const uint32_t s_off = (uint32_t)s_phys * (uint32_t)p.act_row_bytes + sc0 * 16;
     // lane (l16, q) stages the norm of row l16 of its wave's n-tile q
     const bool n_active = q < NT;
-    const uint32_t n_off = 2u * (uint32_t)((EPI == DMQ_EPI_SILU)
+    const uint32_t n_off = 2u * (uint32_t)(SILU
         ? slice_start + ((q & 1) ? p.half_width : 0) + featw + (q >> 1) * 16 + l16
         : (p.slice_is_groups ? 0 : slice_start) + featw + q * 16 + l16);
     // thread t < 16*TT stages the scale word of tile row t
@@ -585,6 +607,154 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       for (int j = 0; j < NT; ++j) dmq_load_words<WW>(wbase + lane_off(w_off[j]), pk[j]);
     };
 
+    // ---- fused epilogue of the gate_up GEMM: SiLU*up rows of the block (one group of 128
+    // features of the down projection) -> per-expert rotation -> (quantization) -> codes.
+    // The fp16 tile of the block meets in LDS in the staged layout (fp16 layers reuse the slot
+    // the finished step has consumed), every wave rotates it onto 32 of the 128 outputs with
+    // its quarter of the rotation matrix, and the quantizers take the row maximum over the four
+    // waves.  Same arithmetic, in the same order, as the stand-alone rotation kernel.
+    auto epilogue_rot = [&](uint8_t* free_slot) {
+      if constexpr (EPI == DMQ_EPI_SILU_ROT) {
+        constexpr int PITCH = 256;                                 // fp16 row of one group
+        const int blk = feat_k - 32 * wave;                        // first feature of the block (feat_k is the wave's)
+        uint8_t* tile = (MODE == DMQ_MODE_A16) ? free_slot : smem_post;
+        // quarter of the rotation matrix this wave applies: output tiles 2*wave, 2*wave + 1
+        const __half* prot = pw.post_rot + (long)(post_slice + blk / DMQ_GS) * (DMQ_GS * DMQ_GS) +
+                             (long)(32 * wave + l16) * DMQ_GS + 8 * q;
+        uint4_t pa[2][4];
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int s = 0; s < 4; ++s) pa[jt][s] = *(const uint4_t*)(prot + (long)jt * 16 * DMQ_GS + 32 * s);
+        __syncthreads();                                           // every wave is done with the slot
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+          const int row = t * 16 + l16;
+#pragma unroll
+          for (int j = 0; j < NT; j += 2) {
+            half4_t h;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
+            // features 32*wave + (j/2)*16 + 4q .. +3 of the group: 8 bytes inside 16-byte chunk c
+            const int f = 32 * wave + (j >> 1) * 16 + 4 * q;
+            const int c = f >> 3;
+            *(half4_t*)(tile + row * PITCH + ((c ^ (row & 15)) * 16) + (f & 7) * 2) = h;
+          }
+        }
+        __syncthreads();
+        float4_t racc[2][TT];
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+          for (int t = 0; t < TT; ++t) racc[jt][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            const int row = t * 16 + l16;
+            // features 32s + 8q .. +7 of the row, the assignment of the stand-alone rotation kernel
+            const uint4_t braw = *(const uint4_t*)(tile + row * PITCH + (((4 * s + q) ^ (row & 15)) * 16));
+            const half8_t b = __builtin_bit_cast(half8_t, braw);
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+              racc[jt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, pa[jt][s]), b,
+                                                                   racc[jt][t], 0, 0, 0);
+          }
+        }
+        const int col0 = blk + 32 * wave + 4 * q;                  // + 16*jt: first of the lane's 4 outputs
+        if constexpr (MODE == DMQ_MODE_A16) {
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            if (!avalid[t]) continue;
+            uint8_t* orow = p.post_out + (long)rlog[t] * p.post_row_bytes;
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt) {
+              const half4_t h = {(_Float16)racc[jt][t][0], (_Float16)racc[jt][t][1],
+                                 (_Float16)racc[jt][t][2], (_Float16)racc[jt][t][3]};
+              *(half4_t*)(orow + (col0 + 16 * jt) * 2) = h;
+            }
+          }
+        } else if constexpr (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
+          float* wmax = (float*)(smem_post + 16 * TT * PITCH);     // [wave][row of the tile]
+          float amax[TT];
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            float m = 0.f;
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) m = fmaxf(m, fabsf(racc[jt][t][r]));
+            m = fmaxf(m, __shfl_xor(m, 16, 64));
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            if (q == 0) wmax[wave * (16 * TT) + t * 16 + l16] = m;
+          }
+          __syncthreads();
+          const float qmax = (MODE == DMQ_MODE_A8) ? 127.0f : 448.0f;
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            const int row = t * 16 + l16;
+            amax[t] = fmaxf(fmaxf(wmax[row], wmax[16 * TT + row]),
+                            fmaxf(wmax[2 * 16 * TT + row], wmax[3 * 16 * TT + row]));
+            const float sc = fmaxf(__fdiv_rn(amax[t], qmax), 1e-8f);
+            if (!avalid[t]) continue;
+            uint8_t* orow = p.post_out + (long)rlog[t] * p.post_row_bytes;
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt) {
+              uint32_t word = 0;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float y = __fdiv_rn(racc[jt][t][r], sc);
+                uint32_t code;
+                if (MODE == DMQ_MODE_A8) {
+                  y = fminf(fmaxf(rintf(y), -127.f), 127.f);
+                  code = (uint32_t)(int)y & 0xffu;
+                } else {
+                  y = fminf(fmaxf(y, -448.f), 448.f);
+                  code = dmq_f32_to_e4m3(y);
+                }
+                word |= code << (8 * r);
+              }
+              *(uint32_t*)(orow + col0 + 16 * jt) = word;
+            }
+            if (wave == 0 && q == 0)
+              ((__half*)p.post_scale)[(long)rlog[t] * p.post_scale_stride + blk / DMQ_GS] =
+                  __float2half_rn(sc * pw.post_extra);
+          }
+        } else {   // FP4: the wave's 32 outputs are one MX block
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            float m = 0.f;
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) m = fmaxf(m, fabsf(racc[jt][t][r]));
+            m = fmaxf(m, __shfl_xor(m, 16, 64));
+            m = fmaxf(fmaxf(m, __shfl_xor(m, 32, 64)), 1e-30f);
+            const float z = __fdiv_rn(m, 6.0f);
+            const float e = ceilf((float)log2((double)z));
+            const float sblk = fmaxf(exp2f(e), 1e-30f);
+            if (!avalid[t]) continue;
+            uint8_t* orow = p.post_out + (long)rlog[t] * p.post_row_bytes;
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt) {
+              uint32_t half_word = 0;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const float y = fminf(fmaxf(__fdiv_rn(racc[jt][t][r], sblk), -6.f), 6.f);
+                const uint32_t nib = dmq_e2m1_mag(fabsf(y)) | ((y < 0.f) ? 8u : 0u);
+                half_word |= nib << (4 * r);
+              }
+              *(uint16_t*)(orow + (col0 + 16 * jt) / 2) = (uint16_t)half_word;
+            }
+            if (q == 0)
+              ((uint8_t*)p.post_scale)[(long)rlog[t] * p.post_scale_stride + (blk / DMQ_GS) * 4 + wave] =
+                  (uint8_t)fminf(fmaxf(e + 127.0f, 0.f), 254.f);
+          }
+        }
+      }
+    };
+
     // A workgroup walks nbc consecutive n-blocks of its item as one stream of nbc * G steps
     // (step = one group of one n-block), so the loads of the next n-block are in flight while
     // the current one finishes; the sums are stored and cleared at each n-block boundary.
@@ -637,7 +807,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         next_load();
         stage_store((u & 1) ^ 1, srb[(u + 1) % D]);
         if (live && ++cg == G) {                       // n-block finished
-          epilogue();
+          if constexpr (EPI == DMQ_EPI_SILU_ROT) epilogue_rot(stage + (u & 1) * SLOT);
+          else epilogue();
 #pragma unroll
           for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -702,6 +873,8 @@ void dmq_gemm_gf_kernel(GemmParams p) {
 #define DMQ_LDS_PAD 0
 #endif
   __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2 + DMQ_LDS_PAD];
+  __shared__ __attribute__((aligned(16))) uint8_t smem_post[PostGeom<MODE, TT, EPI>::BYTES];
+  static_assert(EPI != DMQ_EPI_SILU_ROT || KS == 1, "the fused rotation needs the whole block in one workgroup");
 
   DMQ_MARK(0);
   DMQ_WG_MARK(0);
@@ -725,18 +898,21 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   const int token_start = r0[3];
   const int token_count = r1[0];
   const int slice_start = p.slice_is_groups ? r1[2] : r1[1];
+  // first down group of the item's expert: its gate_up slice starts at weight row 2 * start, its
+  // down slice at group start / 128 (holds for items of either origin)
+  const int post_slice = r1[1] / (2 * DMQ_GS);
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE) return;
   if (WIDE != (pw.bit == 8)) return;
   if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc);
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc);
   } else if constexpr (WIDE) {
-    dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc);
+    dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc);
   } else {
     switch (pw.bit) {
-      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;
-      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;
-      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, token_start, token_count, slice_start, ttile, nb, nbc); break;
+      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc); break;
+      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc); break;
+      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc); break;
     }
   }
 }

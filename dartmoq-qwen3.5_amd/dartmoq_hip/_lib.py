@@ -14,10 +14,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 8
+ABI_VERSION = 9
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
-EPI_STORE, EPI_SILU, EPI_SCATTER = 0, 1, 2
+EPI_STORE, EPI_SILU, EPI_SCATTER, EPI_SILU_ROT = 0, 1, 2, 3
 MODE_BY_NAME = {"wxa16": MODE_A16, "wxa8": MODE_A8, "wxfp8": MODE_FP8, "wxfp4": MODE_FP4}
 
 # status -> exception type, mirroring the reference wrappers (ValueError for bad bit widths,
@@ -44,6 +44,9 @@ class GemmArgs(Structure):
         ("items", c_void_p), ("n_items", c_void_p), ("max_items", c_int),
         ("out", c_void_p), ("out_stride", c_long),
         ("row_weight", c_void_p), ("row_slot", c_void_p), ("dbg_acc", c_void_p),
+        ("post_rot", c_void_p * MAX_POOLS), ("post_extra_scale", c_float * MAX_POOLS),
+        ("post_out", c_void_p), ("post_row_bytes", c_long),
+        ("post_scale", c_void_p), ("post_scale_stride", c_int),
     ]
 
 

@@ -11,7 +11,8 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import (EPI_SCATTER, EPI_SILU, EPI_STORE, MODE_A16, MODE_A8, MODE_FP4, MODE_FP8, GemmArgs,
+from ._lib import (EPI_SILU_ROT,  # noqa: F401
+                   EPI_SCATTER, EPI_SILU, EPI_STORE, MODE_A16, MODE_A8, MODE_FP4, MODE_FP8, GemmArgs,
                    check, load)
 
 GROUP_SIZE = 128
@@ -288,8 +289,10 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
-                 row_weight=None, row_slot=None, dbg_acc=None):
-    """Merged dequant-GEMM launch over up to four pools sharing one work-item list."""
+                 row_weight=None, row_slot=None, dbg_acc=None, post=None):
+    """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
+    (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
+    out=codes tensor [rows, *], scale=scale tensor or None)."""
     a = GemmArgs()
     a.mode, a.epi, a.tt, a.ks, a.nbl, a.n_pools = mode, epi, tt, ks, nbl, len(pools)
     dev = None
@@ -317,6 +320,15 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.row_weight = row_weight.data_ptr() if row_weight is not None else None
     a.row_slot = row_slot.data_ptr() if row_slot is not None else None
     a.dbg_acc = dbg_acc.data_ptr() if dbg_acc is not None else None
+    if post is not None:
+        for i, r in enumerate(post["rot"]):
+            a.post_rot[i] = r.data_ptr() if r is not None else None
+            a.post_extra_scale[i] = float(post["extra"][i])
+        a.post_out = post["out"].data_ptr()
+        a.post_row_bytes = post["out"].stride(0) * post["out"].element_size()
+        if post.get("scale") is not None:
+            a.post_scale = post["scale"].data_ptr()
+            a.post_scale_stride = post["scale"].stride(0)
     check(load().dmq_matmul_merged_gf(ctypes.byref(a), _stream(dev)), "matmul_merged_gf")
     return out
 
@@ -324,7 +336,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
 def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *, groups, n_out,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
-                  tiling=None, dbg_acc=None):
+                  tiling=None, dbg_acc=None, post=None):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -344,7 +356,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         slice_is_groups=slice_is_groups, tt=tt, ks=ks, nbl=nbl, out=out,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
-                        dbg_acc=dbg_acc)
+                        dbg_acc=dbg_acc, post=post)
 
 
 def combine_slots(slots: torch.Tensor, top_k: int, add: torch.Tensor | None = None) -> torch.Tensor:

@@ -44,12 +44,14 @@ enum {
 enum { DMQ_MODE_A16 = 0, DMQ_MODE_A8 = 1, DMQ_MODE_FP8 = 2, DMQ_MODE_FP4 = 3 };
 /* STORE: fp16 [rows, n_out].  SILU: fp16 silu(gate)*up [rows, I].  SCATTER: fp16 routing-weighted
  * rows stored at out[row_slot[r]] (one slot per (token, top-k slot)); dmq_combine_slots adds
- * the k slots of each token in fp32, in slot order. */
-enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2 };
+ * the k slots of each token in fp32, in slot order.  SILU_ROT: SILU followed in the same kernel
+ * by the per-expert rotation (+ quantization) of the down projection's input, i.e. the output is
+ * what dmq_rotate_tiled would make of the SILU rows (post_* fields of dmq_gemm_args). */
+enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_ROT = 3 };
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 8). */
+/* Library / build identification: returns the ABI version (currently 9). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -160,7 +162,9 @@ int dmq_rotate(int mode, const void* x, long x_stride, const void* row_index, co
 /* Same, for rows grouped by expert: work item (pool, e, i) covers rows
  * token_start_e + i*tile_rows .. of expert_info.  With rot_per_expert != 0 group g of expert e
  * uses rot[slice_start_e + g] (the per-expert down rotations, seed + original_start of
- * triton_kernels.py:1310), otherwise rot[g].  max_items bounds the item list. */
+ * triton_kernels.py:1310), otherwise rot[g].  The slice is read from the work items, which must
+ * therefore be built from this expert_info (dmq_build_tiles) or come from dmq_route_permute; the
+ * caller guarantees slice_start_e + groups <= number of matrices.  max_items bounds the list. */
 int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_index,
                      const void* rot, int rot_per_expert, int groups, const void* expert_info,
                      const void* items, const void* n_items, int tile_rows, int max_items,
@@ -213,6 +217,18 @@ typedef struct {
   const void* row_weight;   /* SCATTER: fp32 routing weight per row */
   const void* row_slot;     /* SCATTER: int32 destination slot row per row */
   void* dbg_acc;            /* A8, tt == 1, ks == 1, STORE only: int32 [rows, groups, n_out] or NULL */
+  /* DMQ_EPI_SILU_ROT (ks == 1, n_out % 128 == 0): per pool the rotation matrices fp16
+   * [groups_total, 128, 128] (the matrix of group g of an expert is post_rot[slice_g + g], slice_g
+   * the expert's first down group = gate_up slice_start / 256) and the factor folded into the
+   * stored scales; rotated codes go to post_out [rows, post_row_bytes] (fp16 / int8 / e4m3 /
+   * packed e2m1 by mode), scales to post_scale (fp16 [rows, post_scale_stride] for A8 / FP8, u8
+   * for FP4, unused for A16).  `out` is not written. */
+  const void* post_rot[DMQ_MAX_POOLS];
+  float post_extra_scale[DMQ_MAX_POOLS];
+  void* post_out;
+  long post_row_bytes;
+  void* post_scale;
+  int post_scale_stride;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

@@ -262,3 +262,53 @@ def test_gemm_argument_errors():
     with pytest.raises(ValueError):            # activation rows shorter than groups * 128
         ops.matmul_merged(A16, 2, STORE, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info,
                           groups=4, n_out=128, slice_is_groups=False, rows_total=16, tt=1)
+
+
+@pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])
+@pytest.mark.parametrize("tt,nbl", [(1, 1), (2, 2), (4, 1)])
+def test_fused_down_rotation_equals_separate_kernels(mode, tt, nbl):
+    """DMQ_EPI_SILU_ROT: the gate_up GEMM hands over the rotated (+ quantized) input of the down
+    projection.  It must be bit for bit what the SiLU epilogue followed by the per-expert rotation
+    kernel produces (same fp16 SiLU*up rows, same MFMA order, same quantizer)."""
+    from dartmoq_hip import ops
+    from dartmoq_hip._lib import EPI_SILU_ROT
+    bit, k, inter = 2, 256, 256
+    counts = [9, 70, 0, 33]
+    n_exp = len(counts)
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(17 + mode)
+    idx_gf, norms_gf, cb = _pool(bit, 2 * inter * n_exp, k, 91)
+    x_rot = torch.randn(rows_total, k, generator=g) * 0.7
+    act, scale, _oc, _os, lut, _ol, _wbs, nfac, wsb = _mode_inputs(mode, x_rot, cb)
+    norms_used = (norms_gf.float() * nfac).half() if mode == FP4 else norms_gf
+    w_dev = idx_gf.cuda()
+    if mode == FP4:
+        w_dev = ops.fold_indices_to_e2m1(w_dev, lut, bit)
+    info = [(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(n_exp)]
+    info_dev = torch.tensor(info, dtype=torch.int32).cuda()
+    dinfo = [(starts[e], counts[e], e * (inter // 128), inter // 128) for e in range(n_exp)]
+    dinfo_dev = torch.tensor(dinfo, dtype=torch.int32).cuda()
+    rot = (torch.randn(n_exp * inter // 128, 128, 128, generator=g) / 128 ** 0.5).half().cuda()
+    extra = 0.37
+    tiling = ops.build_tiles(info_dev, rows_total, 16 * tt)
+    n_items, items, max_items = tiling
+    common = dict(groups=k // 128, n_out=inter, half_width=inter, slice_is_groups=False,
+                  rows_total=rows_total, w_scale_byte=wsb, tt=tt, nbl=nbl, tiling=tiling)
+    args = (mode, bit)
+    tens = (act.cuda(), None if scale is None else scale.cuda(), w_dev, norms_used.cuda(),
+            None if mode == FP4 else lut.cuda(), info_dev)
+    silu = ops.matmul_merged(*args, SILU, *tens, **common)
+    # the rotation kernel takes the down slice of an expert from its own work items
+    dn_items, ditems, dmax = ops.build_tiles(dinfo_dev, rows_total, 16 * tt)
+    want_codes, want_scale = ops.rotate_tiled(mode, silu, rot, dinfo_dev, dn_items, ditems, 16 * tt,
+                                              dmax, rows_total, rot_per_expert=True,
+                                              extra_scale=extra, tt=tt)
+    codes, sc, _ = ops._alloc_codes(mode, rows_total, inter, "cuda", False)
+    codes.view(torch.uint8).fill_(0x5a)
+    want = want_codes.clone()
+    ops.matmul_merged(*args, EPI_SILU_ROT, *tens, out=silu, out_stride=inter,
+                      post=dict(rot=[rot], extra=[extra], out=codes, scale=sc), **common)
+    torch.cuda.synchronize()
+    assert torch.equal(codes.view(torch.uint8), want.view(torch.uint8))
+    if sc is not None:
+        assert torch.equal(sc.view(torch.uint8), want_scale.view(torch.uint8))

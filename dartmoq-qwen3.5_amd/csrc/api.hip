@@ -592,7 +592,9 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     const int mode = modes[mi];
     dmq_gemm_args g{};
     g.mode = mode; g.epi = fuse_rot[mi] ? DMQ_EPI_SILU_ROT : DMQ_EPI_SILU;
-    g.tt = tt; g.ks = ks; g.nbl = nbl; g.n_pools = P;
+    // the gate_up blocks are four times as long as the down blocks (K = H against K = I) and end in
+    // the rotation epilogue: more than two per workgroup costs more in balance than it saves
+    g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = pd.major != 0;

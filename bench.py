@@ -11,7 +11,8 @@ the timed region starts.  The 2 bpw layer (~216 MB packed) fits in the 256 MB In
 the steps rotate through three independent copies of the layer.
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the gate_up dequant-GEMM of the
-largest bit pool), timed live with events on the stream it runs on; `cpu_baseline` is the CPU
+largest bit pool, which also rotates its output rows for the down projection), timed live with
+events on the stream it runs on; `cpu_baseline` is the CPU
 oracle (dequantize-then-matmul, fp32) timed on the host cores on a bounded sample.
 """
 
@@ -102,6 +103,12 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
         rows += r_b
         distinct += d_b
     gu_flops = 2.0 * rows * h * 2 * i
+    # without a K split the same launch also rotates its SiLU*up rows for the down projection:
+    # 2*I*128 flop per row and one 32 KiB matrix per (distinct expert, down group)
+    fused_rot = aux["ks"] == 1 and all(bw.bit != 8 for bw in mod.bit_weights.values())
+    if fused_rot:
+        gu_flops += 2.0 * rows * i * 128
+        gu_bytes += distinct * (i // 128) * 128 * 128 * 2
     gu_ms = stage_ms["merged_gate_up"]
     t_hbm, t_mfma = gu_bytes / HBM_PEAK, gu_flops / MFMA_PEAK[mode]
     if t_hbm >= t_mfma:
@@ -112,8 +119,9 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
                 "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
-    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={aux['ks']},SILU> merged gate_up, "
-                       f"nbl={aux['nbl']}",
+    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={aux['ks']},"
+                       f"{'SILU_ROT' if fused_rot else 'SILU'}> merged gate_up"
+                       f"{' + down rotation' if fused_rot else ''}, nbl={min(aux['nbl'], 2)}",
                 launch_ms=gu_ms,
                 algorithmic_bytes=gu_bytes, algorithmic_flops=gu_flops,
                 distinct_experts=distinct, routed_rows=rows)

@@ -148,3 +148,33 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
                        capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_argument_validation_of_later_entry_points():
+    """Status codes of the routing / norm / quantizer / routed-forward entry points for bad
+    arguments (rejected before any launch)."""
+    from dartmoq_hip import _lib
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.dmq_rms_norm(p, 0, p, 0, 4, 12, 16, 16, 1e-6, p, None) == 2            # n % 8
+    assert lib.dmq_rms_norm(p, 0, None, 0, 4, 16, 16, 16, 1e-6, p, None) == 6         # no weight
+    assert lib.dmq_rms_norm(p, 0, p, 0, 4, 16, 8, 16, 1e-6, p, None) == 3             # stride < n
+    assert lib.dmq_rms_norm(p, 0, p, 0, 0, 16, 16, 16, 1e-6, p, None) == 0            # nothing to do
+    assert lib.dmq_quantize_weights(p, 128, p, p, 4, 1, 3, p, p, None) == 1           # bit 3
+    assert lib.dmq_quantize_weights(p, 64, p, p, 4, 1, 4, p, p, None) == 2            # row shorter than K
+    assert lib.dmq_quantize_weights(p, 128, None, p, 4, 1, 4, p, p, None) == 6
+    assert lib.dmq_route_topk_shared(None, 0, None, None, 4, 8, 2, 0, p, p, 128, 1, p, p, None) == 6
+    assert lib.dmq_route_topk_shared(p, 0, None, None, 4, 8, 2, 0, None, p, 128, 1, p, p, None) == 6
+    assert lib.dmq_route_topk_shared(p, 0, None, None, 4, 8, 2, 0, p, p, 128, -1, p, p, None) == 3
+    d = _lib.LayerDesc()
+    r = _lib.RouterArgs()
+    assert lib.dmq_moe_ffn_forward_routed(ctypes.byref(d), ctypes.byref(r), p, 4, None, p, p, 64, 0, 0, 0,
+                                          None, None, None) == 6                       # no pools / router
+    a = _lib.GemmArgs()
+    a.n_pools, a.mode, a.tt, a.epi = 1, 0, 1, 3
+    a.pool[0].bit = 8
+    a.pool[0].mode = 0
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) in (5, 6)                  # fused rotation: no 8-bit pools
+    a.epi = 7
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # unknown epilogue

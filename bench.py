@@ -105,7 +105,7 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     gu_flops = 2.0 * rows * h * 2 * i
     # without a K split the same launch also rotates its SiLU*up rows for the down projection:
     # 2*I*128 flop per row and one 32 KiB matrix per (distinct expert, down group)
-    fused_rot = aux["ks"] == 1 and all(bw.bit != 8 for bw in mod.bit_weights.values())
+    fused_rot = aux["ks"] in (1, -2, -4) and all(bw.bit != 8 for bw in mod.bit_weights.values())
     if fused_rot:
         gu_flops += 2.0 * rows * i * 128
         gu_bytes += distinct * (i // 128) * 128 * 128 * 2
@@ -119,9 +119,10 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
                 "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
-    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={aux['ks']},"
+    shared_k = f", K shared by {-aux['ks']} workgroups" if aux["ks"] < 0 else ""
+    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={max(aux['ks'], 1)},"
                        f"{'SILU_ROT' if fused_rot else 'SILU'}> merged gate_up"
-                       f"{' + down rotation' if fused_rot else ''}, nbl={min(aux['nbl'], 2)}",
+                       f"{' + down rotation' if fused_rot else ''}, nbl={min(aux['nbl'], 2)}{shared_k}",
                 launch_ms=gu_ms,
                 algorithmic_bytes=gu_bytes, algorithmic_flops=gu_flops,
                 distinct_experts=distinct, routed_rows=rows)

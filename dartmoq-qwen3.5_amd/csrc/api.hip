@@ -23,7 +23,19 @@ static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE
 
 // K split across the four waves of a workgroup: a handful of routed rows leaves most CUs idle
 // unless every wave takes a quarter of K; otherwise the waves own different output features
-static inline int pick_ks(int tt, long rows) { return (tt == 1 && rows <= 64) ? 4 : 1; }
+// K split of the 16-row tile kernels for short work lists.  Up to 128 routed rows leave most CUs
+// with at most one workgroup: two workgroups then share the K range of every gate_up block
+// (negative value; needs an even number of groups).  Splitting K over the four waves of a
+// workgroup instead only pays for a handful of rows.
+static inline int pick_ks(int tt, long rows, int groups) {
+  if (tt != 1) return 1;
+  if (rows <= 128 && groups % 2 == 0) return -2;
+  return rows <= 16 ? 4 : 1;
+}
+
+// rows up to which the gate_up GEMM may share the K range of a block between workgroups (bounds
+// the fp32 scratch of the partial sums)
+#define DMQ_SPLIT_MAX_ROWS 1024
 
 // Feature blocks one workgroup walks back to back.  With few row tiles every block gets its own
 // workgroup (parallelism); with many, a workgroup amortizes its start-up over several blocks.
@@ -34,7 +46,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 9; }
+int dmq_abi_version(void) { return 10; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -255,6 +267,13 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
       if (a->pool[i].mode == a->mode && !a->post_rot[i]) return DMQ_ERR_NULL;
   }
   if (a->act_row_bytes < (long)a->groups * act_bytes_per_group(a->mode)) return DMQ_ERR_SHAPE;
+  const int wsplit = a->k_split > 1 ? a->k_split : 1;
+  if (wsplit > 1) {
+    if ((wsplit != 2 && wsplit != 4) || !silu || ks != 1 || a->tt != 1 || any_wide) return DMQ_ERR_MODE;
+    if (a->groups % wsplit || a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
+    if (!a->split_partial || !a->split_counter) return DMQ_ERR_NULL;
+    if (a->split_rows <= 0) return DMQ_ERR_SHAPE;
+  }
 
   GemmLaunch L;
   GemmParams& p = L.p;
@@ -283,6 +302,10 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.post_row_bytes = a->post_row_bytes;
   p.post_scale = a->post_scale;
   p.post_scale_stride = a->post_scale_stride;
+  p.wsplit = wsplit;
+  p.split_rows = a->split_rows;
+  p.split_partial = (float*)a->split_partial;
+  p.split_counter = (int*)a->split_counter;
   L.epi = a->epi;
   L.tt = a->tt;
   L.dbg = a->dbg_acc != nullptr;
@@ -296,13 +319,13 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
     // several n-blocks per workgroup need every block complete and the waves on distinct features
     int nbl = a->nbl > 0 ? a->nbl : 1;
-    if (lks > 1 || a->n_out % feat_per_block) nbl = 1;
+    if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block) nbl = 1;
     if (nbl > p.n_blocks) nbl = p.n_blocks;
     p.nbl = nbl;
     L.p = p;
     L.ks = lks;
     L.wide = wide;
-    long work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl);
+    long work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
     work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
     if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
     L.grid = (int)work;
@@ -379,6 +402,9 @@ struct MoeWorkspace {
   uint8_t* xq[DMQ_MAX_POOLS];        // hoisted pools: codes by token; others share xq_rows
   uint8_t* xq_scale[DMQ_MAX_POOLS];
   uint8_t *xq_rows, *xq_rows_scale, *act, *actq, *actq_scale;
+  float* split_partial;              // gate_up K range shared between workgroups: fp32 sums
+  int* split_counter;
+  int split_rows, split_counters;
   void* sort_scratch;
   size_t sort_scratch_bytes;
   int max_items, tile_rows;
@@ -426,6 +452,10 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.act = take(R * I * 2);
   w.actq = take(R * I * 2);
   w.actq_scale = take(R * (I / DMQ_GS) * 4);
+  w.split_rows = (int)(R < DMQ_SPLIT_MAX_ROWS ? R : DMQ_SPLIT_MAX_ROWS);
+  w.split_partial = (float*)take((size_t)4 * w.split_rows * 2 * I * 4);
+  w.split_counters = (int)((R / 16 + E) * (I / DMQ_GS));
+  w.split_counter = (int*)take((size_t)w.split_counters * 4);
   w.bytes = off;
   return w;
 }
@@ -475,7 +505,14 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   if (P > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
   if (tt <= 0) tt = pick_tt(tokens, K, E);
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
-  if (ks <= 0) ks = pick_ks(tt, (long)tokens * K);
+  if (ks == 0) ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
+  // ks < 0: -ks workgroups share the K range of a gate_up block; the other launches do not split
+  const int wsplit = ks < 0 ? -ks : 1;
+  if (ks < 0) {
+    if ((wsplit != 2 && wsplit != 4) || tt != 1 || (H / DMQ_GS) % wsplit) return DMQ_ERR_MODE;
+    if ((long)tokens * K > DMQ_SPLIT_MAX_ROWS) return DMQ_ERR_LIMIT;
+    ks = 1;
+  }
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   if (nbl <= 0) nbl = pick_nbl((long)tokens * K, tt);
   const int rot_tt = tt;               // a rotation wave covers one row tile of the work items
@@ -485,7 +522,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   int rc;
   if (aux_out) {
     long* aux = (long*)aux_out;
-    aux[0] = tt; aux[1] = ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
+    aux[0] = tt; aux[1] = wsplit > 1 ? -wsplit : ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
     aux[3] = w.max_items; aux[4] = (long)((uint8_t*)w.n_items - (uint8_t*)workspace);
     aux[5] = nbl;
   }
@@ -535,6 +572,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       plan.n_items = w.n_items; plan.items = w.items;
       sp.sorted_tokens = w.sorted_tokens; sp.sorted_weights = w.sorted_weights;
       sp.sorted_rows = w.sorted_rows;
+      if (wsplit > 1) { sp.clear_words = w.split_counter; sp.clear_count = w.split_counters; }
       rc = dmq_route_small_launch(sp, st);
     } else {
       const void* tk_idx = router->topk_idx;
@@ -550,6 +588,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
                              w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
                              w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items,
                              w.items, w.sort_scratch, w.sort_scratch_bytes, stream);
+      if (!rc && wsplit > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
     }
   }
   if (rc) return rc;
@@ -613,6 +652,12 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     g.out = w.act; g.out_stride = I;
     g.post_out = w.actq; g.post_row_bytes = (long)I * 2;
     g.post_scale = w.actq_scale; g.post_scale_stride = scale_stride_for(mode, I);
+    bool mode_wide = false;
+    for (int i = 0; i < P; ++i) mode_wide |= (layer->pool[i].mode == mode && layer->pool[i].bit == 8);
+    if (wsplit > 1 && !mode_wide) {
+      g.k_split = wsplit; g.split_rows = w.split_rows;
+      g.split_partial = w.split_partial; g.split_counter = w.split_counter;
+    }
     rc = dmq_matmul_merged_gf(&g, stream);
     if (rc) return rc;
   }

@@ -95,6 +95,13 @@ struct GemmParams {
   long post_row_bytes;
   void* post_scale;            // A8/FP8: fp16 [rows, post_scale_stride]; FP4: u8 [rows, post_scale_stride]
   int post_scale_stride;
+  // K range of one (item, block) shared by wsplit workgroups (16-row tiles, SiLU epilogues): each
+  // parks its fp32 sums in its plane of split_partial and takes a ticket; the last one adds the
+  // planes in plane order and runs the epilogue
+  int wsplit;                  // 1, 2 or 4
+  int split_rows;              // rows of one plane
+  float* split_partial;        // fp32 [wsplit, split_rows, 2 * n_out]
+  int* split_counter;          // int32 [max_items * n_blocks], zero before the launch and after it
 };
 
 template <int MODE> struct ModeTraits;
@@ -215,7 +222,8 @@ template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
                                               uint8_t* smem2, uint8_t* smem_post, int token_start,
                                               int token_count, int slice_start, int post_slice,
-                                              int ttile, int nb, int nbc) {
+                                              int ttile, int nb, int nbc, int split, int* ticket,
+                                              int* wg_flag) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   using GG = GemmGeom<MODE, NT, TT, KS>;
@@ -231,6 +239,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr int FEAT_TILES = NT / UNIT;                              // output tiles per wave
   constexpr int PPG = (MODE == DMQ_MODE_FP4) ? 64 : (DMQ_GS * BIT / 8);
   constexpr int FPB = ROWPARTS * FEAT_TILES * 16;                    // output features per n-block
+  constexpr bool XSPLIT = STAGE && TT == 1 && SILU;                  // K range shared across workgroups
   static_assert(NT % UNIT == 0, "SiLU epilogue pairs gate/up tiles");
 
   const int lane = threadIdx.x & 63;
@@ -755,6 +764,60 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       }
     };
 
+    // ---- K range shared by several workgroups: park the sums of the valid rows in this
+    // workgroup's plane, take a ticket, and let the last arrival add the planes (always in plane
+    // order, its own from registers, so the result does not depend on the order of arrival).
+    // The planes are written and read with device-scope accesses, which go past the per-XCD L2
+    // on their own: no cache-wide write-back or invalidate, only a wait for this wave's stores
+    // to be acknowledged before the workgroup takes its ticket.
+    auto split_gather = [&](int nsplit_) -> bool {
+      using u64 = unsigned long long;
+      const long row_floats = 2L * p.n_out;
+      const long plane = (long)p.split_rows * row_floats;
+      float* base = p.split_partial + (long)rlog[0] * row_floats + feat_k + 4 * q;
+      const bool mine = avalid[0] && wave_active;
+      if (mine) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          u64* dst = (u64*)(base + (long)split * plane + ((j & 1) ? p.n_out : 0) + (j >> 1) * 16);
+          const float2_t lo = {total_acc[j][0][0], total_acc[j][0][1]};
+          const float2_t hi = {total_acc[j][0][2], total_acc[j][0][3]};
+          __hip_atomic_store(dst, __builtin_bit_cast(u64, lo), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(dst + 1, __builtin_bit_cast(u64, hi), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        const int t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (t == nsplit_ - 1)                           // ready for the next launch
+          __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *wg_flag = t;
+      }
+      __syncthreads();
+      if (*wg_flag != nsplit_ - 1) return false;
+      if (mine) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          float4_t sum = (float4_t){0.f, 0.f, 0.f, 0.f};
+          for (int s = 0; s < nsplit_; ++s) {
+            float4_t v = total_acc[j][0];
+            if (s != split) {
+              const u64* src = (const u64*)(base + (long)s * plane + ((j & 1) ? p.n_out : 0) + (j >> 1) * 16);
+              const float2_t lo = __builtin_bit_cast(
+                  float2_t, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+              const float2_t hi = __builtin_bit_cast(
+                  float2_t, __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+              v = (float4_t){lo[0], lo[1], hi[0], hi[1]};
+            }
+            sum += v;
+          }
+          total_acc[j][0] = sum;
+        }
+      }
+      return true;
+    };
+
     // A workgroup walks nbc consecutive n-blocks of its item as one stream of nbc * G steps
     // (step = one group of one n-block), so the loads of the next n-block are in flight while
     // the current one finishes; the sums are stored and cleared at each n-block boundary.
@@ -766,7 +829,9 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     static_assert(D % 2 == 0, "the LDS slot of a ring entry is fixed by its parity");
     uint32_t pkb[D][NT][WW];
     Staged srb[D];
-    const int G = g_hi;
+    const int nsplit = XSPLIT ? p.wsplit : 1;
+    const int G = XSPLIT ? p.groups / nsplit : g_hi;   // groups this workgroup contracts
+    const int g_first = XSPLIT ? split * G : 0;
     const int steps = nbc * G;
     int lk = 0, lg = 0;                                // load position: n-block, group
     auto next_load = [&]() {
@@ -778,8 +843,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_fetch<BIT, T::ES>(pw.lut, threadIdx.x, lutw);
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      stage_load(lk, lg, srb[u]);
-      load_packed(lk, lg, pkb[u]);
+      stage_load(lk, g_first + lg, srb[u]);
+      load_packed(lk, g_first + lg, pkb[u]);
       next_load();
     }
     DMQ_MARK(1);
@@ -794,7 +859,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 #pragma unroll
       for (int u = 0; u < D; ++u) {
         const bool live = sb + u < steps;              // uniform over the workgroup
-        stage_load(lk, lg, srb[u]);                    // entry u went to LDS one step ago
+        stage_load(lk, g_first + lg, srb[u]);          // entry u went to LDS one step ago
         if (live) {
           uint32_t xa[TT][AW];
           uint2_t nr[NT];
@@ -803,12 +868,16 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
           stage_read(u & 1, xa, nr, xs, xsb);
           compute(cg, pkb[u], nr, xa, xs, xsb);
         }
-        load_packed(lk, lg, pkb[u]);
+        load_packed(lk, g_first + lg, pkb[u]);
         next_load();
         stage_store((u & 1) ^ 1, srb[(u + 1) % D]);
         if (live && ++cg == G) {                       // n-block finished
-          if constexpr (EPI == DMQ_EPI_SILU_ROT) epilogue_rot(stage + (u & 1) * SLOT);
-          else epilogue();
+          bool whole = true;                           // uniform over the workgroup
+          if constexpr (XSPLIT) { if (nsplit > 1) whole = split_gather(nsplit); }
+          if (whole) {
+            if constexpr (EPI == DMQ_EPI_SILU_ROT) epilogue_rot(stage + (u & 1) * SLOT);
+            else epilogue();
+          }
 #pragma unroll
           for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -881,15 +950,21 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   // Workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD gets a contiguous range of
   // the work list, so the workgroups that share an activation tile (the feature blocks of an
   // item) and those that share weights (the row tiles of an expert) meet in one L2.
-  const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl;      // workgroups per item
+  constexpr bool XSPLIT = KS == 1 && TT == 1 && (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT);
+  __shared__ int wg_flag;
+  const int wsplit = XSPLIT ? p.wsplit : 1;
+  const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl * wsplit;   // workgroups per item
   const int total = p.n_items[0] * nbg;
   const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
   const int slot = blockIdx.x / DMQ_XCDS;
   const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
   if (slot >= per_xcd || unit >= total) return;
   const int item = unit / nbg;
-  const int nb = (unit - item * nbg) * p.nbl;
+  const int sub = unit - item * nbg;
+  const int split = sub % wsplit;                        // workgroups sharing a block are neighbours
+  const int nb = (sub / wsplit) * p.nbl;
   const int nbc = min(p.nbl, p.n_blocks - nb);
+  int* ticket = XSPLIT ? p.split_counter + (long)item * p.n_blocks + nb : nullptr;
   const int4_t* rec = (const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * item);
   const int4_t r0 = rec[0];
   const int4_t r1 = rec[1];
@@ -905,14 +980,14 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   if (pw.mode != MODE) return;
   if (WIDE != (pw.bit == 8)) return;
   if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc);
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
   } else if constexpr (WIDE) {
-    dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc);
+    dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
   } else {
     switch (pw.bit) {
-      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc); break;
-      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc); break;
-      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc); break;
+      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;
+      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;
+      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;
     }
   }
 }

@@ -104,6 +104,8 @@ struct RouteSmallParams {
   int* sorted_tokens;
   float* sorted_weights;
   int* sorted_rows;
+  int* clear_words;              // optional: clear_count int32 words set to zero by the launch
+  int clear_count;
 };
 int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream);
 

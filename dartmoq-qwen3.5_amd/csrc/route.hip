@@ -417,6 +417,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   const int rows = p.tokens * kt;
   const int experts = p.plan.experts;
   for (int i = tid; i < 16 * experts; i += 1024) s_hist[i] = 0;
+  for (int i = tid; i < p.clear_count; i += 1024) p.clear_words[i] = 0;
   // top-k (or the caller's), shared columns: the rows of the next token of the wave are requested
   // before the current token is worked on
   auto tokens_of_wave = [&](auto nv_tag) {

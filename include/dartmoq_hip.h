@@ -229,6 +229,17 @@ typedef struct {
   long post_row_bytes;
   void* post_scale;
   int post_scale_stride;
+  /* k_split = 2 or 4 (0 / 1 = off): the groups of one (work item, feature block) are shared by
+   * that many workgroups, for short work lists that leave most of the chip idle.  tt == 1,
+   * ks <= 1, a SILU epilogue, groups % k_split == 0; nbl is ignored.  Each workgroup parks its
+   * fp32 sums in split_partial (fp32 [k_split, split_rows, 2 * n_out], split_rows >= every routed
+   * row index + 1) and the last to arrive adds them in a fixed order and runs the epilogue.
+   * split_counter: int32 [max_items * n_out / 128], zero before the launch; the launch leaves it
+   * zero. */
+  int k_split;
+  int split_rows;
+  void* split_partial;
+  void* split_counter;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more
@@ -288,8 +299,10 @@ size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens);
  * and its WxA8 / WxFP8 / WxFP4 subclasses, routed experts only:
  *   x fp16 [tokens, hidden]; topk_idx int32 / topk_w fp32 [tokens, top_k];
  *   out fp16 [tokens, hidden] = sum_k w * down_e(silu(gate_e(x)) * up_e(x)) (+ add_f16).
- * Every expert must belong to exactly one pool.  tt <= 0 / ks <= 0 / nbl <= 0 pick the tiling
- * (rows per tile, K split, feature blocks per workgroup) from tokens. */
+ * Every expert must belong to exactly one pool.  tt <= 0 / ks == 0 / nbl <= 0 pick the tiling
+ * (rows per tile, K split, feature blocks per workgroup) from tokens.  ks > 0 splits K over the
+ * waves of a workgroup (1 or 4); ks = -2 / -4 shares the K range of the gate_up GEMM between
+ * that many workgroups instead (k_split of dmq_gemm_args: tt == 1, at most 1024 routed rows). */
 int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                         const void* topk_w, int tokens, const void* add_f16, void* out,
                         void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,

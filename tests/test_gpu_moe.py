@@ -278,3 +278,58 @@ def test_empty_batch_and_3d_input(small_layer):
     packed = next(iter(small_layer.pools.values())).down
     lin = dartmoq_hip.WxA16Linear.from_packed(packed)
     assert lin(torch.zeros(0, lin.in_features, dtype=torch.float16, device="cuda")).shape == (0, lin.out_features)
+
+
+@pytest.fixture(scope="module")
+def four_group_layer():
+    bits = moe.assign_bits(16, {2: 0.75, 1: 0.125, 4: 0.125}, seed=2)
+    return moe.build_layer(512, 256, 16, 4, bits, seed=11)
+
+
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
+@pytest.mark.parametrize("tokens,split", [(1, 4), (7, 2), (40, 4), (200, 2)])
+def test_layer_with_k_shared_between_workgroups(four_group_layer, mode, tokens, split):
+    """ks = -2 / -4: the groups of every gate_up block are contracted by 2 / 4 workgroups that
+    meet through fp32 partial sums in the workspace.  Same bounds against the oracles as the
+    unsplit forward, the same bits on every call (the partial sums are added in a fixed order and
+    the arrival counters return to zero), and agreement with the unsplit forward up to the
+    rounding of the changed summation order."""
+    layer = four_group_layer
+    g = torch.Generator().manual_seed(5 * tokens + split)
+    x = torch.randn(tokens, layer.hidden, generator=g).half()
+    logits = routing.zipf_logits(tokens, layer.num_experts, tokens + split)
+    w, idx = routing.route_topk(logits, layer.top_k)
+    mod = make_module(layer, mode)
+    mod.tt_override = 1
+    mod.ks_override = 1
+    plain = mod.forward(x.cuda(), topk_idx=idx.cuda().int(), topk_w=w.cuda()).clone()
+    mod.ks_override = -split
+    first = mod.forward(x.cuda(), topk_idx=idx.cuda().int(), topk_w=w.cuda()).clone()
+    again = mod.forward(x.cuda(), topk_idx=idx.cuda().int(), topk_w=w.cuda()).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(first, again)
+    out = first.cpu().float()
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+    assert relerr(out, plain.cpu().float()) < tight
+    if mode == "wxa16":
+        ref = moe.reference_forward(layer, x, idx, w)
+        assert max_rel(out, ref) <= 1e-2 and cosine(out, ref) >= 0.9999
+
+
+def test_k_sharing_argument_errors(small_layer):
+    mod = make_module(small_layer, "wxa16")
+    x = torch.zeros(4, small_layer.hidden, dtype=torch.float16, device="cuda")
+    idx = torch.zeros(4, small_layer.top_k, dtype=torch.int32, device="cuda")
+    idx[:] = torch.arange(small_layer.top_k, dtype=torch.int32)
+    w = torch.full((4, small_layer.top_k), 0.25, device="cuda")
+    mod.ks_override = -4                       # two groups cannot be shared four ways
+    with pytest.raises(ValueError):
+        mod.forward(x, topk_idx=idx, topk_w=w)
+    mod.ks_override = -3
+    with pytest.raises(ValueError):
+        mod.forward(x, topk_idx=idx, topk_w=w)
+    mod.ks_override, mod.tt_override = -2, 2   # 16-row tiles only
+    with pytest.raises(ValueError):
+        mod.forward(x, topk_idx=idx, topk_w=w)

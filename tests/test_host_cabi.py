@@ -178,3 +178,31 @@ def test_argument_validation_of_later_entry_points():
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) in (5, 6)                  # fused rotation: no 8-bit pools
     a.epi = 7
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # unknown epilogue
+
+
+def test_k_sharing_argument_validation():
+    """k_split of the merged GEMM: 2 or 4 workgroups per block, 16-row tiles, SiLU epilogues,
+    groups divisible, scratch present (all rejected before any launch)."""
+    from dartmoq_hip import _lib
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    a = _lib.GemmArgs()
+    a.mode, a.epi, a.tt, a.n_pools = 0, _lib.EPI_SILU, 1, 1
+    q = a.pool[0]
+    q.w = q.norms = q.lut = q.expert_info = q.act = p
+    q.n_total, q.bit, q.mode = 256, 2, 0
+    a.items = a.n_items = a.out = p
+    a.max_items, a.groups, a.n_out, a.half_width, a.act_row_bytes = 4, 4, 128, 128, 1024
+    a.k_split = 3
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5
+    a.k_split = 2
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 6           # no scratch
+    a.split_partial = a.split_counter = p
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 3           # split_rows missing
+    a.split_rows, a.tt = 16, 2
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # 16-row tiles only
+    a.tt, a.epi = 1, _lib.EPI_STORE
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # SiLU epilogues only
+    a.epi, a.k_split, a.groups, a.act_row_bytes = _lib.EPI_SILU, 4, 6, 2048
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 2           # 6 groups, 4 workgroups

@@ -12,6 +12,18 @@
 #include "params.h"
 #include <type_traits>
 
+// developer instrumentation of the one-workgroup routing kernel: wall-clock stamps (100 MHz) of
+// thread 0 at the phase boundaries, read back with dmq_route_trace_read
+#ifdef DMQ_TRACE
+static __device__ long long dmq_route_marks[32];
+#define DMQ_RMARK(i) do { if (threadIdx.x == 0) dmq_route_marks[i] = wall_clock64(); } while (0)
+extern "C" int dmq_route_trace_read(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(dmq_route_marks), sizeof(long long) * 32);
+}
+#else
+#define DMQ_RMARK(i)
+#endif
+
 // ------------------------------------------------------------------------------ top-k
 // Wave-wide max / min through data-parallel lane moves: xor 1, xor 2, mirror within 8 and within
 // 16 lanes leave every lane with the result of its row of 16; the four rows are then combined
@@ -216,21 +228,93 @@ __device__ __forceinline__ int block_scan_incl(int v, int* wave_tot) {
   return v + add;
 }
 
-// Per-pool expert_info and the work-item list from the per-expert counts and offsets in LDS
-// (pools in caller order, experts ascending).  Called by all 1024 threads of the workgroup.
-__device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* s_cnt, const int* s_off,
-                                                int* wave_tot, int* carry_p) {
+// 64-bit variant of the scan: four 16-bit fields scanned at once
+__device__ __forceinline__ unsigned long long block_scan_incl_u64(unsigned long long v,
+                                                                  unsigned long long* wave_tot) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned long long o = __shfl_up(v, d, 64);
+    if (lane >= d) v += o;
+  }
+  if (lane == 63) wave_tot[wave] = v;
+  __syncthreads();
+  unsigned long long add = 0;
+  for (int w = 0; w < wave; ++w) add += wave_tot[w];
+  return v + add;
+}
+
+// Slice tables of thread tid's expert in every pool, requested early by the callers so that the
+// memory latency hides behind the counting phases (one pass: experts <= 1024).
+struct PlanSlices { int ss[DMQ_MAX_POOLS], sc[DMQ_MAX_POOLS]; };
+__device__ __forceinline__ PlanSlices plan_load_slices(const PlanParams& p) {
+  PlanSlices s;
   const int tid = threadIdx.x;
-  if (tid == 0) *carry_p = 0;
-  // the slice tables of all pools are requested at once when one pass covers the experts
-  int ss_pre[DMQ_MAX_POOLS], sc_pre[DMQ_MAX_POOLS];
   const bool pre = p.experts <= 1024;
 #pragma unroll
   for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
     const bool ok = pre && pool < p.pools && tid < p.experts;
-    ss_pre[pool] = ok ? p.slice_start_rows[pool * p.experts + tid] : -1;
-    sc_pre[pool] = ok ? p.slice_count_rows[pool * p.experts + tid] : 0;
+    s.ss[pool] = ok ? p.slice_start_rows[pool * p.experts + tid] : -1;
+    s.sc[pool] = ok ? p.slice_count_rows[pool * p.experts + tid] : 0;
   }
+  return s;
+}
+
+// Per-pool expert_info and the work-item list from the per-expert counts and offsets in LDS
+// (pools in caller order, experts ascending).  Called by all 1024 threads of the workgroup.
+// With one expert per thread and fewer than 65536 items the tile counts of the (up to four)
+// pools are scanned together, 16 bits each: one scan and two barriers for the whole list.
+__device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* s_cnt, const int* s_off,
+                                                int* wave_tot, unsigned long long* wave_tot64,
+                                                int* carry_p, const PlanSlices& pre_s) {
+  const int tid = threadIdx.x;
+  const bool pre = p.experts <= 1024;
+  if (pre && p.max_items < 65536) {
+    const int e = tid;
+    const bool live = e < p.experts;
+    const int ts = live ? s_off[e] : 0;
+    int ntile[DMQ_MAX_POOLS], tcs[DMQ_MAX_POOLS];
+    unsigned long long packed = 0;
+#pragma unroll
+    for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+      ntile[pool] = 0; tcs[pool] = 0;
+      if (pool < p.pools && live) {
+        const int ss = pre_s.ss[pool], sc = pre_s.sc[pool];
+        const int tc = (ss >= 0) ? s_cnt[e] : 0;
+        tcs[pool] = tc;
+        ntile[pool] = (tc + p.tile_rows - 1) / p.tile_rows;
+        packed |= (unsigned long long)ntile[pool] << (16 * pool);
+        int4_t* gi = (int4_t*)(p.gu_info + ((long)pool * p.experts + e) * 4);
+        *gi = (int4_t){ts, tc, ss >= 0 ? ss : 0, sc};
+        int4_t* di = (int4_t*)(p.dn_info + ((long)pool * p.experts + e) * 4);
+        *di = (int4_t){ts, tc, ss >= 0 ? ss / (2 * DMQ_GS) : 0, sc / (2 * DMQ_GS)};
+      }
+    }
+    const unsigned long long incl = block_scan_incl_u64(packed, wave_tot64);
+    if (tid == 1023) wave_tot64[16] = incl;            // per-pool totals
+    __syncthreads();
+    const unsigned long long totals = wave_tot64[16];
+    int base = 0;
+#pragma unroll
+    for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+      if (pool < p.pools) {
+        const int first = base + (int)((incl >> (16 * pool)) & 0xffffu) - ntile[pool];
+        const int ss = pre_s.ss[pool];
+        for (int i = 0; i < ntile[pool]; ++i) {
+          if (first + i < p.max_items) {
+            int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * (first + i));
+            it[0] = (int4_t){pool, e, i, ts};
+            it[1] = (int4_t){tcs[pool], ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
+          }
+        }
+        base += (int)((totals >> (16 * pool)) & 0xffffu);
+      }
+    }
+    if (tid == 0) p.n_items[0] = min(base, p.max_items);
+    return;
+  }
+  if (tid == 0) *carry_p = 0;
   __syncthreads();
 #pragma unroll
   for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
@@ -239,8 +323,8 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
       const int e = base + tid;
       int ntile = 0, ts = 0, tc = 0, gu_ss = 0, dn_ss = 0;
       if (e < p.experts) {
-        const int ss = pre ? ss_pre[pool] : p.slice_start_rows[pool * p.experts + e];
-        const int sc = pre ? sc_pre[pool] : p.slice_count_rows[pool * p.experts + e];
+        const int ss = pre ? pre_s.ss[pool] : p.slice_start_rows[pool * p.experts + e];
+        const int sc = pre ? pre_s.sc[pool] : p.slice_count_rows[pool * p.experts + e];
         tc = (ss >= 0) ? s_cnt[e] : 0;
         ts = s_off[e];
         gu_ss = ss >= 0 ? ss : 0;
@@ -277,8 +361,10 @@ void dmq_plan_kernel(PlanParams p) {
   __shared__ int partial[1024];
   __shared__ int s_cnt[DMQ_SORT_MAX_EXPERTS];
   __shared__ int s_off[DMQ_SORT_MAX_EXPERTS + 1];
+  __shared__ unsigned long long wave_tot64[17];
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
+  const PlanSlices slices = plan_load_slices(p);       // in flight during the counting phases
   // The chunk axis of the histogram is split over `parts` threads per expert so that all 1024
   // threads load; a thread keeps at most 16 loads in flight and its values stay in registers
   // when its share of the chunks fits (16 per thread: up to 64 chunks at <= 256 experts).
@@ -354,7 +440,7 @@ void dmq_plan_kernel(PlanParams p) {
     if (!one_pass) __syncthreads();
   }
 
-  plan_emit_items(p, s_cnt, s_off, wave_tot, &carry);
+  plan_emit_items(p, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices);
 }
 
 // Stable scatter of one chunk.  The rows of one token name distinct experts, so the lanes of a
@@ -409,6 +495,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   __shared__ int s_hist[16 * DMQ_ROUTE_SMALL_EXPERTS];
   __shared__ int s_idx[DMQ_ROUTE_SMALL_ROWS];
   __shared__ float s_w[DMQ_ROUTE_SMALL_ROWS];
+  __shared__ unsigned long long wave_tot64[17];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -416,8 +503,11 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   const int kt = k + p.sg.n_shared;
   const int rows = p.tokens * kt;
   const int experts = p.plan.experts;
+  DMQ_RMARK(0);
+  const PlanSlices slices = plan_load_slices(p.plan);  // in flight during the top-k
   for (int i = tid; i < 16 * experts; i += 1024) s_hist[i] = 0;
   for (int i = tid; i < p.clear_count; i += 1024) p.clear_words[i] = 0;
+  DMQ_RMARK(1);
   // top-k (or the caller's), shared columns: the rows of the next token of the wave are requested
   // before the current token is worked on
   auto tokens_of_wave = [&](auto nv_tag) {
@@ -453,7 +543,9 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   if (!p.logits || p.router_experts <= 256) tokens_of_wave(std::integral_constant<int, 4>{});
   else if (p.router_experts <= 512) tokens_of_wave(std::integral_constant<int, 8>{});
   else tokens_of_wave(std::integral_constant<int, 16>{});
+  DMQ_RMARK(2);
   __syncthreads();
+  DMQ_RMARK(3);
   // rows per (wave chunk, expert)
   const int r = tid;
   const int e_r = (r < rows) ? s_idx[r] : -1;
@@ -476,6 +568,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
     if (tid == 0) { s_off[0] = 0; p.plan.offsets[0] = 0; }
   }
   __syncthreads();
+  DMQ_RMARK(4);
   // s_hist[w, e] <- sorted position of the first row of wave chunk w routed to expert e
   if (tid < experts) {
     int at = s_off[tid];
@@ -487,7 +580,9 @@ void dmq_route_small_kernel(RouteSmallParams p) {
     }
   }
   __syncthreads();
-  plan_emit_items(p.plan, s_cnt, s_off, wave_tot, &carry);
+  DMQ_RMARK(5);
+  plan_emit_items(p.plan, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices);
+  DMQ_RMARK(6);
   // stable scatter of the wave's chunk: tokens one after the other, the rows of a token name
   // distinct experts
   const int base = wave * 64;
@@ -505,6 +600,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
       p.sorted_rows[at] = r;
     }
   }
+  DMQ_RMARK(7);
 }
 
 // Work items for a caller-supplied expert_info (merged-GEMM entry points): one workgroup.

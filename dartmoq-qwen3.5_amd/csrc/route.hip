@@ -267,7 +267,8 @@ __device__ __forceinline__ PlanSlices plan_load_slices(const PlanParams& p) {
 // pools are scanned together, 16 bits each: one scan and two barriers for the whole list.
 __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* s_cnt, const int* s_off,
                                                 int* wave_tot, unsigned long long* wave_tot64,
-                                                int* carry_p, const PlanSlices& pre_s) {
+                                                int* carry_p, const PlanSlices& pre_s,
+                                                int* item_first = nullptr) {
   const int tid = threadIdx.x;
   const bool pre = p.experts <= 1024;
   if (pre && p.max_items < 65536) {
@@ -296,6 +297,37 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
     __syncthreads();
     const unsigned long long totals = wave_tot64[16];
     int base = 0;
+    if (item_first) {
+      // Long batches: an expert with many rows has many tiles, so the records are written one
+      // per thread: item_first[pool * experts + e] is the first record of (pool, e), and record i
+      // belongs to the last entry that starts at or before i.
+#pragma unroll
+      for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
+        if (pool < p.pools) {
+          if (live) item_first[pool * p.experts + e] = base + (int)((incl >> (16 * pool)) & 0xffffu) - ntile[pool];
+          base += (int)((totals >> (16 * pool)) & 0xffffu);
+        }
+      }
+      __syncthreads();
+      const int n = min(base, p.max_items);
+      const int entries = p.pools * p.experts;
+      for (int i = tid; i < n; i += 1024) {
+        int lo = 0, hi = entries;                        // first entry that starts after i
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (item_first[mid] <= i) lo = mid + 1; else hi = mid;
+        }
+        const int idx = lo - 1;
+        const int pool = idx / p.experts;
+        const int ex = idx - pool * p.experts;
+        const int ss = p.slice_start_rows[idx];
+        int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * i);
+        it[0] = (int4_t){pool, ex, i - item_first[idx], s_off[ex]};
+        it[1] = (int4_t){s_cnt[ex], ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
+      }
+      if (tid == 0) p.n_items[0] = n;
+      return;
+    }
 #pragma unroll
     for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
       if (pool < p.pools) {
@@ -362,8 +394,10 @@ void dmq_plan_kernel(PlanParams p) {
   __shared__ int s_cnt[DMQ_SORT_MAX_EXPERTS];
   __shared__ int s_off[DMQ_SORT_MAX_EXPERTS + 1];
   __shared__ unsigned long long wave_tot64[17];
+  __shared__ int item_first[DMQ_MAX_POOLS * 1024];
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
+  DMQ_RMARK(8);
   const PlanSlices slices = plan_load_slices(p);       // in flight during the counting phases
   // The chunk axis of the histogram is split over `parts` threads per expert so that all 1024
   // threads load; a thread keeps at most 16 loads in flight and its values stay in registers
@@ -406,6 +440,7 @@ void dmq_plan_kernel(PlanParams p) {
     if (!one_pass) __syncthreads();                    // partial[] is reused by the next pass
   }
   __syncthreads();
+  DMQ_RMARK(9);
   // expert offsets: exclusive scan of counts, 1024 experts per pass
   for (int base = 0; base < p.experts; base += 1024) {
     const int e = base + tid;
@@ -418,6 +453,7 @@ void dmq_plan_kernel(PlanParams p) {
   }
   if (tid == 0) { s_off[0] = 0; p.offsets[0] = 0; }
   __syncthreads();
+  DMQ_RMARK(10);
   // hist[c, e] <- position of the first row of chunk c routed to expert e
   for (int ebase = 0; ebase < p.experts; ebase += epad) {
     const int e = ebase + el;
@@ -439,8 +475,9 @@ void dmq_plan_kernel(PlanParams p) {
     }
     if (!one_pass) __syncthreads();
   }
-
-  plan_emit_items(p, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices);
+  DMQ_RMARK(11);
+  plan_emit_items(p, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices, item_first);
+  DMQ_RMARK(12);
 }
 
 // Stable scatter of one chunk.  The rows of one token name distinct experts, so the lanes of a

@@ -126,12 +126,13 @@ size_t dmq_route_scratch_bytes(int tokens, int k, int experts) {
   return (size_t)n_chunks * experts * sizeof(int);
 }
 
-int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
+// pool_order / lead_pools: see PlanParams (NULL = pools in index order, n_items[1] not written)
+static int route_permute_ordered(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
                       int pools, const void* slice_start, const void* slice_count, int tile_rows,
                       int max_items, void* counts, void* offsets, void* sorted_tokens,
                       void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
                       void* n_items, void* items, void* scratch, size_t scratch_bytes,
-                      void* stream) {
+                      const int* pool_order, int lead_pools, void* stream) {
   if (!topk_idx || !topk_w || !slice_start || !slice_count || !counts || !offsets ||
       !sorted_tokens || !sorted_weights || !sorted_rows || !gu_info || !dn_info || !n_items ||
       !items || !scratch)
@@ -147,6 +148,8 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
   plan.slice_start_rows = (const int*)slice_start; plan.slice_count_rows = (const int*)slice_count;
   plan.offsets = (int*)offsets; plan.gu_info = (int*)gu_info; plan.dn_info = (int*)dn_info;
   plan.n_items = (int*)n_items; plan.items = (int*)items;
+  for (int i = 0; i < DMQ_MAX_POOLS; ++i) plan.pool_order[i] = pool_order ? pool_order[i] : i;
+  plan.lead_pools = pool_order ? lead_pools : -1;
   if ((long)tokens * k <= DMQ_ROUTE_SMALL_ROWS && experts <= DMQ_ROUTE_SMALL_EXPERTS && k <= 64) {
     RouteSmallParams sp{};                   // one launch instead of three
     sp.in_idx = (const int*)topk_idx; sp.in_w = (const float*)topk_w;
@@ -159,6 +162,18 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
   return dmq_route_permute_launch((const int*)topk_idx, (const float*)topk_w, tokens, k, plan,
                                   (int*)sorted_tokens, (float*)sorted_weights, (int*)sorted_rows,
                                   (hipStream_t)stream);
+}
+
+int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
+                      int pools, const void* slice_start, const void* slice_count, int tile_rows,
+                      int max_items, void* counts, void* offsets, void* sorted_tokens,
+                      void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
+                      void* n_items, void* items, void* scratch, size_t scratch_bytes,
+                      void* stream) {
+  return route_permute_ordered(topk_idx, topk_w, tokens, k, experts, pools, slice_start, slice_count,
+                               tile_rows, max_items, counts, offsets, sorted_tokens, sorted_weights,
+                               sorted_rows, gu_info, dn_info, n_items, items, scratch, scratch_bytes,
+                               nullptr, -1, stream);
 }
 
 int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_items, int pool,
@@ -187,10 +202,8 @@ int dmq_rotate(int mode, const void* x, long x_stride, const void* row_index, co
   p.x = (const __half*)x; p.x_stride = x_stride; p.row_index = nullptr;
   p.rows = rows; p.groups = groups;
   p.n_hoisted = 1; p.hoisted_pool[0] = 0;
-  const long row_tiles = (rows + 16 * tt - 1) / (16 * tt);
-  p.hoisted_items_per_pool = (int)(row_tiles * groups);
   p.items = nullptr; p.n_items = nullptr; p.tile_rows = 16 * tt; p.scale_fp32 = scale_fp32;
-  return dmq_rotate_dispatch(mode, p, row_tiles * groups, tt, (hipStream_t)stream);
+  return dmq_rotate_dispatch(mode, p, 0, tt, (hipStream_t)stream);
 }
 
 int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_index, const void* rot,
@@ -211,7 +224,7 @@ int dmq_rotate_tiled(int mode, const void* x, long x_stride, const void* row_ind
                    (const int*)expert_info, extra_scale, mode, 0, rot_per_expert ? 1 : 0};
   for (int i = 0; i < DMQ_MAX_POOLS; ++i) p.pool[i] = rp;     // items may carry any pool id
   p.x = (const __half*)x; p.x_stride = x_stride; p.row_index = (const int*)row_index;
-  p.rows = 0; p.groups = groups; p.n_hoisted = 0; p.hoisted_items_per_pool = 1;
+  p.rows = 0; p.groups = groups; p.n_hoisted = 0;
   p.items = (const int*)items; p.n_items = (const int*)n_items; p.tile_rows = tile_rows;
   p.scale_fp32 = scale_fp32;
   const long n = (long)max_items * (tile_rows / (16 * tt)) * groups;
@@ -549,6 +562,16 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       if (layer->pool[i].mode == modes[mi] && layer->pool[i].bit == 8) fuse_rot[mi] = false;
   }
 
+  // The pools whose rows are rotated per work item come first in the item list, so that the
+  // rotation launch knows their items as a prefix (n_items[1]) and touches no other record.
+  int pool_order[DMQ_MAX_POOLS] = {0, 1, 2, 3}, lead_pools = 0;
+  {
+    int n = 0;
+    for (int i = 0; i < P; ++i) if (layer->pool[i].major == 0) pool_order[n++] = i;
+    lead_pools = n;
+    for (int i = 0; i < P; ++i) if (layer->pool[i].major != 0) pool_order[n++] = i;
+  }
+
   // 1. top-k (when the router hands over logits), shared columns, sort by expert, per-pool
   //    expert_info, work items: one launch for small batches
   {
@@ -570,6 +593,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       plan.slice_count_rows = (const int*)layer->slice_count;
       plan.offsets = w.offsets; plan.gu_info = w.gu_info; plan.dn_info = w.dn_info;
       plan.n_items = w.n_items; plan.items = w.items;
+      for (int i = 0; i < DMQ_MAX_POOLS; ++i) plan.pool_order[i] = pool_order[i];
+      plan.lead_pools = lead_pools;
       sp.sorted_tokens = w.sorted_tokens; sp.sorted_weights = w.sorted_weights;
       sp.sorted_rows = w.sorted_rows;
       if (wsplit > 1) { sp.clear_words = w.split_counter; sp.clear_count = w.split_counters; }
@@ -584,10 +609,11 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
         if (rc) return rc;
         tk_idx = w.topk_idx; tk_w = w.topk_w;
       }
-      rc = dmq_route_permute(tk_idx, tk_w, tokens, K, E, P, layer->slice_start, layer->slice_count,
-                             w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
-                             w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items,
-                             w.items, w.sort_scratch, w.sort_scratch_bytes, stream);
+      rc = route_permute_ordered(tk_idx, tk_w, tokens, K, E, P, layer->slice_start, layer->slice_count,
+                                 w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
+                                 w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items,
+                                 w.items, w.sort_scratch, w.sort_scratch_bytes, pool_order,
+                                 lead_pools, stream);
       if (!rc && wsplit > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
     }
   }
@@ -600,9 +626,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     RotParams rp{};
     rp.x = (const __half*)x; rp.x_stride = H; rp.row_index = w.sorted_tokens;
     rp.rows = tokens; rp.groups = H / DMQ_GS;
-    rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0;
-    const long row_tiles = (tokens + 16 * rot_tt - 1) / (16 * rot_tt);
-    rp.hoisted_items_per_pool = (int)(row_tiles * rp.groups);
+    rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0; rp.items_prefix = 1;
     bool any_tiled = false;
     for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
       const int pi = i < P ? i : 0;
@@ -617,8 +641,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       if (live && hoisted) rp.hoisted_pool[rp.n_hoisted++] = i;
       if (live && !hoisted) any_tiled = true;
     }
-    long n = (long)rp.n_hoisted * rp.hoisted_items_per_pool;
-    if (any_tiled) n += (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
+    long n = 0;                                    // waves of the per-work-item part
+    if (any_tiled) n = (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
     else rp.items = nullptr;
     rc = dmq_rotate_dispatch(mode, rp, n, rot_tt, st);
     if (rc) return rc;
@@ -670,7 +694,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if (fuse_rot[mi]) continue;
     RotParams rp{};
     rp.x = (const __half*)w.act; rp.x_stride = I; rp.row_index = nullptr;
-    rp.rows = 0; rp.groups = I / DMQ_GS; rp.n_hoisted = 0; rp.hoisted_items_per_pool = 1;
+    rp.rows = 0; rp.groups = I / DMQ_GS; rp.n_hoisted = 0;
     rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0;
     for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
       const int pi = i < P ? i : 0;

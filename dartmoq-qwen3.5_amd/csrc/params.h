@@ -27,11 +27,12 @@ struct RotParams {
   int groups;              // groups per row
   int n_hoisted;
   int hoisted_pool[DMQ_MAX_POOLS];
-  int hoisted_items_per_pool;   // ceil(rows / (16*TT)) * groups
+  int hoisted_wgs_per_pool;     // ceil(ceil(rows / (16*TT)) / 4) * groups, set by the launcher
   const int* items;        // [*, DMQ_ITEM_WORDS] work-item records
   const int* n_items;
   int tile_rows;           // rows per work item (multiple of 16*TT)
   int scale_fp32;
+  int items_prefix;        // 1: only the first n_items[1] items belong to tiled pools
 };
 
 struct QuantParams {
@@ -81,8 +82,14 @@ struct PlanParams {
   int* offsets;                  // [experts + 1]
   int* gu_info;                  // [pools, experts, 4]
   int* dn_info;                  // [pools, experts, 4]  slice in groups: start/128, I/128
-  int* n_items;                  // [1]
+  int* n_items;                  // [1]; [2] when lead_pools >= 0
   int* items;                    // [max_items, DMQ_ITEM_WORDS]
+  // Order in which the pools' items are listed (a permutation of 0 .. pools-1).  With
+  // lead_pools >= 0, n_items[1] receives the number of items of the first lead_pools pools of
+  // that order (the layer forward lists the pools whose rows are rotated per work item first, so
+  // their items are a prefix of the list); lead_pools < 0 leaves n_items[1] alone.
+  int pool_order[DMQ_MAX_POOLS];
+  int lead_pools;
 };
 
 // One-workgroup routing for small batches: top-k (or a copy of the caller's top-k), the shared
@@ -109,7 +116,7 @@ struct RouteSmallParams {
 };
 int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream);
 
-int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream);
+int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream);
 int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
 int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx, const float* in_w,
                           int tokens, int experts, int k, int renorm, float* out_w, int* out_idx,

@@ -35,25 +35,30 @@ void dmq_rotate_kernel(RotParams p) {
   const int q = lane >> 4;
   constexpr int ROWS_PER_ITEM = 16 * TT;
 
-  long item = (long)blockIdx.x * 4 + wave;
+  // Workgroups [0, n_hoisted * hoisted_wgs_per_pool) rotate whole-batch pools: a workgroup owns
+  // one group and four consecutive row tiles (one per wave) and stages the group's matrix in LDS
+  // once.  The remaining workgroups take one work item per wave and read their matrices (one
+  // per expert with rot_use_slice) straight from memory.
+  __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
   int pool, g, r_first, r_end, rot_g;
   const int* row_index = nullptr;
-  const long hoisted_total = (long)p.n_hoisted * p.hoisted_items_per_pool;
-  if (item < hoisted_total) {
-    pool = p.hoisted_pool[item / p.hoisted_items_per_pool];
-    const long local = item % p.hoisted_items_per_pool;
-    g = (int)(local % p.groups);
-    r_first = (int)(local / p.groups) * ROWS_PER_ITEM;
+  const long hoisted_wgs = (long)p.n_hoisted * p.hoisted_wgs_per_pool;
+  const bool staged = (long)blockIdx.x < hoisted_wgs;                 // uniform over the workgroup
+  if (staged) {
+    pool = p.hoisted_pool[blockIdx.x / p.hoisted_wgs_per_pool];
+    const int local = blockIdx.x % p.hoisted_wgs_per_pool;
+    g = local % p.groups;
+    r_first = ((local / p.groups) * 4 + wave) * ROWS_PER_ITEM;
     r_end = p.rows;
     rot_g = g;
   } else {
     if (!p.items) return;
-    item -= hoisted_total;
+    long item = ((long)blockIdx.x - hoisted_wgs) * 4 + wave;
     g = (int)(item % p.groups);
     const long rt = item / p.groups;
     const int sub = p.tile_rows / ROWS_PER_ITEM;          // waves per work item
     const long tile = rt / sub;
-    if (tile >= p.n_items[0]) return;
+    if (tile >= p.n_items[p.items_prefix ? 1 : 0]) return;
     const int* it = p.items + DMQ_ITEM_WORDS * tile;
     pool = it[0];
     if (p.pool[pool].hoisted) return;
@@ -67,6 +72,21 @@ void dmq_rotate_kernel(RotParams p) {
   }
   const RotPool& rp = p.pool[pool];
   if (rp.mode != MODE) return;
+  if (staged) {
+    // 2048 chunks of 16 bytes, eight per thread; chunk c of row r sits at position c ^ (r % 16) so
+    // that the sixteen rows a wave reads at once spread over all banks
+    const uint4_t* src = (const uint4_t*)(rp.rot + (long)rot_g * (DMQ_GS * DMQ_GS));
+    uint4_t v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = src[threadIdx.x + 256 * i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      const int row = c >> 4;
+      *(uint4_t*)(mat + row * 256 + (((c & 15) ^ (row & 15)) * 16)) = v[i];
+    }
+    __syncthreads();
+  }
   if (r_first >= r_end) return;
 
   int rlog[TT];
@@ -87,21 +107,34 @@ void dmq_rotate_kernel(RotParams p) {
 #pragma unroll
     for (int t = 0; t < TT; ++t) acc[j][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
+  // same MFMA order on both paths (steps outer, output tiles inner): the results do not depend
+  // on where the matrix comes from
+  auto product = [&](auto load_a) {
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    half8_t b[TT];
+    for (int s = 0; s < 4; ++s) {
+      half8_t b[TT];
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-      uint4_t raw = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
-      b[t] = __builtin_bit_cast(half8_t, raw);
+      for (int t = 0; t < TT; ++t) {
+        uint4_t raw = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
+        b[t] = __builtin_bit_cast(half8_t, raw);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const half8_t a = __builtin_bit_cast(half8_t, load_a(j, s));
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[j][t], 0, 0, 0);
+      }
     }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      half8_t a = __builtin_bit_cast(half8_t, *(const uint4_t*)(prow + (long)j * 16 * DMQ_GS + 32 * s));
-#pragma unroll
-      for (int t = 0; t < TT; ++t)
-        acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[t], acc[j][t], 0, 0, 0);
-    }
+  };
+  if (staged) {
+    // row j*16 + l16 of the matrix, chunk 4s + q
+    const uint8_t* mrow = mat + l16 * 256;
+    product([&](int j, int s) {
+      return *(const uint4_t*)(mrow + j * (16 * 256) + (((4 * s + q) ^ l16) * 16));
+    });
+  } else {
+    product([&](int j, int s) { return *(const uint4_t*)(prow + (long)j * 16 * DMQ_GS + 32 * s); });
   }
 
 #pragma unroll
@@ -244,9 +277,17 @@ void dmq_quantize_kernel(QuantParams p) {
 }
 
 // --------------------------------------------------------------------------------------------
+// tiled_waves: waves of the per-work-item part (max_items * tile_rows / (16*tt) * groups); the
+// whole-batch pools add n_hoisted * ceil(row tiles / 4) * groups workgroups in front
 template <int MODE>
-static int launch_rotate(const RotParams& p, long items, int tt, hipStream_t stream) {
-  const int grid = (int)((items + 3) / 4);
+static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStream_t stream) {
+  RotParams p = p_in;
+  const long row_tiles = ((long)p.rows + 16 * tt - 1) / (16 * tt);
+  p.hoisted_wgs_per_pool = (int)(((row_tiles + 3) / 4) * p.groups);
+  if (p.hoisted_wgs_per_pool < 1) p.hoisted_wgs_per_pool = 1;
+  const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + (tiled_waves + 3) / 4;
+  if (total > 0x7fffffffL) return DMQ_ERR_LIMIT;
+  const int grid = (int)total;
   if (grid <= 0) return DMQ_OK;
   if (tt == 4) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 4>), dim3(grid), dim3(256), 0, stream, p);
   else if (tt == 2) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 2>), dim3(grid), dim3(256), 0, stream, p);
@@ -254,12 +295,12 @@ static int launch_rotate(const RotParams& p, long items, int tt, hipStream_t str
   return dmq_check_launch();
 }
 
-int dmq_rotate_dispatch(int mode, const RotParams& p, long items, int tt, hipStream_t stream) {
+int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream) {
   switch (mode) {
-    case DMQ_MODE_A16: return launch_rotate<DMQ_MODE_A16>(p, items, tt, stream);
-    case DMQ_MODE_A8: return launch_rotate<DMQ_MODE_A8>(p, items, tt, stream);
-    case DMQ_MODE_FP8: return launch_rotate<DMQ_MODE_FP8>(p, items, tt, stream);
-    case DMQ_MODE_FP4: return launch_rotate<DMQ_MODE_FP4>(p, items, tt, stream);
+    case DMQ_MODE_A16: return launch_rotate<DMQ_MODE_A16>(p, tiled_waves, tt, stream);
+    case DMQ_MODE_A8: return launch_rotate<DMQ_MODE_A8>(p, tiled_waves, tt, stream);
+    case DMQ_MODE_FP8: return launch_rotate<DMQ_MODE_FP8>(p, tiled_waves, tt, stream);
+    case DMQ_MODE_FP4: return launch_rotate<DMQ_MODE_FP4>(p, tiled_waves, tt, stream);
   }
   return DMQ_ERR_MODE;
 }

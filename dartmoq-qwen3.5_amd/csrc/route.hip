@@ -245,6 +245,11 @@ __device__ __forceinline__ unsigned long long block_scan_incl_u64(unsigned long 
   return v + add;
 }
 
+// Element `i` (run-time) of a four-entry register array, without indexing it through memory.
+__device__ __forceinline__ int pick4(const int (&v)[DMQ_MAX_POOLS], int i) {
+  return i == 0 ? v[0] : (i == 1 ? v[1] : (i == 2 ? v[2] : v[3]));
+}
+
 // Slice tables of thread tid's expert in every pool, requested early by the callers so that the
 // memory latency hides behind the counting phases (one pass: experts <= 1024).
 struct PlanSlices { int ss[DMQ_MAX_POOLS], sc[DMQ_MAX_POOLS]; };
@@ -296,16 +301,18 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
     if (tid == 1023) wave_tot64[16] = incl;            // per-pool totals
     __syncthreads();
     const unsigned long long totals = wave_tot64[16];
-    int base = 0;
+    int base = 0, lead = 0;
     if (item_first) {
       // Long batches: an expert with many rows has many tiles, so the records are written one
-      // per thread: item_first[pool * experts + e] is the first record of (pool, e), and record i
-      // belongs to the last entry that starts at or before i.
+      // per thread: item_first[o * experts + e] is the first record of (o-th pool of the order,
+      // e), and record i belongs to the last entry that starts at or before i.
 #pragma unroll
-      for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
-        if (pool < p.pools) {
-          if (live) item_first[pool * p.experts + e] = base + (int)((incl >> (16 * pool)) & 0xffffu) - ntile[pool];
+      for (int o = 0; o < DMQ_MAX_POOLS; ++o) {
+        if (o < p.pools) {
+          const int pool = p.pool_order[o];
+          if (live) item_first[o * p.experts + e] = base + (int)((incl >> (16 * pool)) & 0xffffu) - pick4(ntile, pool);
           base += (int)((totals >> (16 * pool)) & 0xffffu);
+          if (o + 1 == p.lead_pools) lead = base;
         }
       }
       __syncthreads();
@@ -318,45 +325,56 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
           if (item_first[mid] <= i) lo = mid + 1; else hi = mid;
         }
         const int idx = lo - 1;
-        const int pool = idx / p.experts;
-        const int ex = idx - pool * p.experts;
-        const int ss = p.slice_start_rows[idx];
+        const int o = idx / p.experts;
+        const int ex = idx - o * p.experts;
+        const int pool = p.pool_order[o];
+        const int ss = p.slice_start_rows[pool * p.experts + ex];
         int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * i);
         it[0] = (int4_t){pool, ex, i - item_first[idx], s_off[ex]};
         it[1] = (int4_t){s_cnt[ex], ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
       }
-      if (tid == 0) p.n_items[0] = n;
+      if (tid == 0) {
+        p.n_items[0] = n;
+        if (p.lead_pools >= 0) p.n_items[1] = min(lead, p.max_items);
+      }
       return;
     }
 #pragma unroll
-    for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
-      if (pool < p.pools) {
-        const int first = base + (int)((incl >> (16 * pool)) & 0xffffu) - ntile[pool];
-        const int ss = pre_s.ss[pool];
-        for (int i = 0; i < ntile[pool]; ++i) {
+    for (int o = 0; o < DMQ_MAX_POOLS; ++o) {
+      if (o < p.pools) {
+        const int pool = p.pool_order[o];
+        const int nt = pick4(ntile, pool);
+        const int first = base + (int)((incl >> (16 * pool)) & 0xffffu) - nt;
+        const int ss = pick4(pre_s.ss, pool);
+        const int tc = pick4(tcs, pool);
+        for (int i = 0; i < nt; ++i) {
           if (first + i < p.max_items) {
             int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * (first + i));
             it[0] = (int4_t){pool, e, i, ts};
-            it[1] = (int4_t){tcs[pool], ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
+            it[1] = (int4_t){tc, ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
           }
         }
         base += (int)((totals >> (16 * pool)) & 0xffffu);
+        if (o + 1 == p.lead_pools) lead = base;
       }
     }
-    if (tid == 0) p.n_items[0] = min(base, p.max_items);
+    if (tid == 0) {
+      p.n_items[0] = min(base, p.max_items);
+      if (p.lead_pools >= 0) p.n_items[1] = min(lead, p.max_items);
+    }
     return;
   }
   if (tid == 0) *carry_p = 0;
   __syncthreads();
-#pragma unroll
-  for (int pool = 0; pool < DMQ_MAX_POOLS; ++pool) {
-    if (pool >= p.pools) break;
+  int lead = 0;
+  for (int o = 0; o < p.pools; ++o) {
+    const int pool = p.pool_order[o];
     for (int base = 0; base < p.experts; base += 1024) {
       const int e = base + tid;
       int ntile = 0, ts = 0, tc = 0, gu_ss = 0, dn_ss = 0;
       if (e < p.experts) {
-        const int ss = pre ? pre_s.ss[pool] : p.slice_start_rows[pool * p.experts + e];
-        const int sc = pre ? pre_s.sc[pool] : p.slice_count_rows[pool * p.experts + e];
+        const int ss = pre ? pick4(pre_s.ss, pool) : p.slice_start_rows[pool * p.experts + e];
+        const int sc = pre ? pick4(pre_s.sc, pool) : p.slice_count_rows[pool * p.experts + e];
         tc = (ss >= 0) ? s_cnt[e] : 0;
         ts = s_off[e];
         gu_ss = ss >= 0 ? ss : 0;
@@ -380,8 +398,12 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
       if (tid == 1023) *carry_p = incl + *carry_p;
       __syncthreads();
     }
+    if (o + 1 == p.lead_pools) lead = *carry_p;
   }
-  if (tid == 0) p.n_items[0] = min(*carry_p, p.max_items);
+  if (tid == 0) {
+    p.n_items[0] = min(*carry_p, p.max_items);
+    if (p.lead_pools >= 0) p.n_items[1] = min(lead, p.max_items);
+  }
 }
 
 __global__ __launch_bounds__(1024)

@@ -23,6 +23,10 @@ struct LutGeom {
   static constexpr int EB = ELEMS * ES;                 // payload bytes per entry
   static constexpr int STRIDE = EB < 4 ? 4 : EB;        // bytes between copies
   static constexpr int COPIES = DMQ_LUT_ROW / STRIDE;
+  // 2-bit codebooks (4 values: 8 bytes of fp16, 4 bytes of int8 / e4m3) fit the source operands
+  // of one byte permute, so every lane composes table entries itself instead of receiving them
+  // from the lane that fetched them
+  static constexpr bool PERM_BUILD = (BIT == 2) && (DMQ_LUT_ROW == 128);
 };
 
 // Entry `e` of the table: the codebook values of the 8/BIT indices packed in byte value e.
@@ -31,6 +35,17 @@ __device__ __forceinline__ void dmq_lut_fetch(const void* codebook, int e, uint3
   using G = LutGeom<BIT, ES>;
   constexpr uint32_t mask = (1u << BIT) - 1u;
   w[0] = w[1] = w[2] = w[3] = 0u;
+  if constexpr (G::PERM_BUILD) {        // the whole codebook, same for every thread
+    if (ES == 2) {
+      const uint16_t* cb = (const uint16_t*)codebook;
+      w[0] = (uint32_t)cb[0] | ((uint32_t)cb[1] << 16);
+      w[1] = (uint32_t)cb[2] | ((uint32_t)cb[3] << 16);
+    } else {
+      const uint8_t* cb = (const uint8_t*)codebook;
+      w[0] = (uint32_t)cb[0] | ((uint32_t)cb[1] << 8) | ((uint32_t)cb[2] << 16) | ((uint32_t)cb[3] << 24);
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < G::ELEMS; ++j) {
     uint32_t idx = ((uint32_t)e >> (j * BIT)) & mask;
@@ -53,6 +68,32 @@ __device__ __forceinline__ void dmq_lut_store_wave(uint8_t* tbl, int wave, const
   constexpr int DW = G::STRIDE / 4;                     // dwords per copy
   constexpr int RPW = 256 / DMQ_LUT_ROW;                // table rows per 256-byte store
   const int lane = threadIdx.x & 63;
+  if constexpr (G::PERM_BUILD) {
+    // Store t of wave v covers the eight entries 64 v + 8 t .. + 7: lane l writes 16 bytes (two or
+    // four copies) of entry e = 64 v + 8 t + l / 8.  The four indices of e are (l/8) & 3,
+    // ((l/8) >> 2) | (t & 1) << 1, t >> 1 and v: only the first two depend on the lane.
+    const uint32_t sub = (uint32_t)lane >> 3;
+    uint8_t* dst = tbl + ((long)wave * 64 + sub) * DMQ_LUT_ROW + (lane & 7) * 16;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const uint32_t i0 = sub & 3u, i1 = (sub >> 2) | ((uint32_t)(t & 1) << 1);
+      const uint32_t i2 = (uint32_t)(t >> 1), i3 = (uint32_t)wave;
+      uint4_t v;
+      if (ES == 2) {
+        const uint32_t s0 = 0x01000100u + i0 * 0x0202u + i1 * 0x02020000u;
+        const uint32_t s1 = 0x01000100u + i2 * 0x0202u + i3 * 0x02020000u;
+        const uint32_t e0 = __builtin_amdgcn_perm(w[1], w[0], s0);
+        const uint32_t e1 = __builtin_amdgcn_perm(w[1], w[0], s1);
+        v = (uint4_t){e0, e1, e0, e1};
+      } else {
+        const uint32_t sel = i0 | (i1 << 8) | (i2 << 16) | (i3 << 24);
+        const uint32_t e0 = __builtin_amdgcn_perm(0u, w[0], sel);
+        v = (uint4_t){e0, e0, e0, e0};
+      }
+      *(uint4_t*)(dst + t * 8 * DMQ_LUT_ROW) = v;
+    }
+    return;
+  }
   const int d = lane % DW;
   uint32_t* dst = (uint32_t*)(tbl + (long)wave * 64 * DMQ_LUT_ROW) + lane;
 #pragma unroll

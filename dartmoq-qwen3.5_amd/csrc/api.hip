@@ -36,6 +36,11 @@ static inline int pick_ks(int tt, long rows, int groups) {
 // rows up to which the gate_up GEMM may share the K range of a block between workgroups (bounds
 // the fp32 scratch of the partial sums)
 #define DMQ_SPLIT_MAX_ROWS 1024
+// single-block workgroups at the end of every XCD's share of a GEMM launch that otherwise walks
+// several blocks per workgroup: one round of resident workgroups (32 CUs x 3)
+#ifndef DMQ_TAIL_SLOTS
+#define DMQ_TAIL_SLOTS 96
+#endif
 
 // Feature blocks one workgroup walks back to back.  With few row tiles every block gets its own
 // workgroup (parallelism); with many, a workgroup amortizes its start-up over several blocks.
@@ -335,11 +340,20 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block) nbl = 1;
     if (nbl > p.n_blocks) nbl = p.n_blocks;
     p.nbl = nbl;
+    // several blocks per workgroup: the tail of every XCD's share is cut into single blocks
+    p.tail_slots = (nbl > 1 && wsplit == 1 && p.n_blocks % nbl == 0) ? DMQ_TAIL_SLOTS : 0;
     L.p = p;
     L.ks = lks;
     L.wide = wide;
-    long work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
-    work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
+    long work;
+    if (p.tail_slots > 0) {
+      long per_xcd = ((long)a->max_items * p.n_blocks + DMQ_XCDS - 1) / DMQ_XCDS;
+      per_xcd = (per_xcd + nbl - 1) / nbl * nbl;
+      work = (per_xcd / nbl + p.tail_slots) * DMQ_XCDS;
+    } else {
+      work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
+      work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
+    }
     if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
     L.grid = (int)work;
     int rc = DMQ_ERR_MODE;

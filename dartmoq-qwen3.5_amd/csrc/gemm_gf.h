@@ -83,6 +83,8 @@ struct GemmParams {
   const int* n_items;          // device scalar
   int n_blocks;                // blocks of output features per item
   int nbl;                     // consecutive blocks one workgroup walks (1 unless KS == 1)
+  int tail_slots;              // > 0: the last tail_slots blocks of every XCD's share go one per
+                               // workgroup (nbl > 1, nbl divides n_blocks, wsplit == 1)
   // outputs
   __half* out;                 // STORE / SILU: fp16 [rows, out_stride]
   long out_stride;
@@ -953,17 +955,40 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   constexpr bool XSPLIT = KS == 1 && TT == 1 && (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT);
   __shared__ int wg_flag;
   const int wsplit = XSPLIT ? p.wsplit : 1;
-  const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl * wsplit;   // workgroups per item
-  const int total = p.n_items[0] * nbg;
-  const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
-  const int slot = blockIdx.x / DMQ_XCDS;
-  const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
-  if (slot >= per_xcd || unit >= total) return;
-  const int item = unit / nbg;
-  const int sub = unit - item * nbg;
-  const int split = sub % wsplit;                        // workgroups sharing a block are neighbours
-  const int nb = (sub / wsplit) * p.nbl;
-  const int nbc = min(p.nbl, p.n_blocks - nb);
+  int item, nb, nbc, split = 0;
+  if (p.tail_slots > 0) {
+    // Workgroups are dispatched in index order as slots free up, so the order of the list is the
+    // schedule: the head of an XCD's share goes nbl blocks per workgroup (loads stay in flight
+    // across blocks, one table build for several blocks), its last tail_slots blocks one per
+    // workgroup, so that the last round of workgroups is short and full instead of long and
+    // half empty.
+    const int total_blocks = p.n_items[0] * p.n_blocks;
+    int per_xcd = (total_blocks + DMQ_XCDS - 1) / DMQ_XCDS;
+    per_xcd = (per_xcd + p.nbl - 1) / p.nbl * p.nbl;
+    const int xcd = blockIdx.x % DMQ_XCDS;
+    const int slot = blockIdx.x / DMQ_XCDS;
+    const int nblk = min(per_xcd, total_blocks - xcd * per_xcd);     // blocks of this XCD
+    if (nblk <= 0) return;
+    const int big = max(0, (nblk - p.tail_slots) / p.nbl);            // workgroups with nbl blocks
+    const int first = slot < big ? slot * p.nbl : big * p.nbl + (slot - big);
+    if (first >= nblk) return;
+    const int blk = xcd * per_xcd + first;
+    item = blk / p.n_blocks;
+    nb = blk - item * p.n_blocks;
+    nbc = min(slot < big ? p.nbl : 1, p.n_blocks - nb);
+  } else {
+    const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl * wsplit;   // workgroups per item
+    const int total = p.n_items[0] * nbg;
+    const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
+    const int slot = blockIdx.x / DMQ_XCDS;
+    const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
+    if (slot >= per_xcd || unit >= total) return;
+    item = unit / nbg;
+    const int sub = unit - item * nbg;
+    split = sub % wsplit;                                  // workgroups sharing a block are neighbours
+    nb = (sub / wsplit) * p.nbl;
+    nbc = min(p.nbl, p.n_blocks - nb);
+  }
   int* ticket = XSPLIT ? p.split_counter + (long)item * p.n_blocks + nb : nullptr;
   const int4_t* rec = (const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * item);
   const int4_t r0 = rec[0];

@@ -27,7 +27,8 @@ struct RotParams {
   int groups;              // groups per row
   int n_hoisted;
   int hoisted_pool[DMQ_MAX_POOLS];
-  int hoisted_wgs_per_pool;     // ceil(ceil(rows / (16*TT)) / 4) * groups, set by the launcher
+  int hoisted_wgs_per_pool;     // set by the launcher
+  int hoisted_staged;           // 1: workgroup = one group x four row tiles, matrix staged in LDS
   const int* items;        // [*, DMQ_ITEM_WORDS] work-item records
   const int* n_items;
   int tile_rows;           // rows per work item (multiple of 16*TT)

@@ -43,12 +43,19 @@ void dmq_rotate_kernel(RotParams p) {
   int pool, g, r_first, r_end, rot_g;
   const int* row_index = nullptr;
   const long hoisted_wgs = (long)p.n_hoisted * p.hoisted_wgs_per_pool;
-  const bool staged = (long)blockIdx.x < hoisted_wgs;                 // uniform over the workgroup
-  if (staged) {
+  const bool hoisted = (long)blockIdx.x < hoisted_wgs;                // uniform over the workgroup
+  const bool staged = hoisted && p.hoisted_staged;
+  if (hoisted) {
     pool = p.hoisted_pool[blockIdx.x / p.hoisted_wgs_per_pool];
     const int local = blockIdx.x % p.hoisted_wgs_per_pool;
-    g = local % p.groups;
-    r_first = ((local / p.groups) * 4 + wave) * ROWS_PER_ITEM;
+    if (staged) {
+      g = local % p.groups;
+      r_first = ((local / p.groups) * 4 + wave) * ROWS_PER_ITEM;
+    } else {                      // few rows: one (row tile, group) per wave, more workgroups
+      const int idx = local * 4 + wave;
+      g = idx % p.groups;
+      r_first = (idx / p.groups) * ROWS_PER_ITEM;
+    }
     r_end = p.rows;
     rot_g = g;
   } else {
@@ -72,6 +79,24 @@ void dmq_rotate_kernel(RotParams p) {
   }
   const RotPool& rp = p.pool[pool];
   if (rp.mode != MODE) return;
+
+  int rlog[TT];
+  bool valid[TT];
+  const __half* xrow[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) {
+    rlog[t] = r_first + t * 16 + l16;
+    valid[t] = rlog[t] < r_end;
+    int phys = valid[t] ? (row_index ? row_index[rlog[t]] : rlog[t]) : 0;
+    xrow[t] = p.x + (long)phys * p.x_stride + g * DMQ_GS + 8 * q;
+  }
+  // the rows of the tile are requested before the matrix is staged, so both are in flight together
+  uint4_t xraw[4][TT];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+      xraw[s][t] = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
   if (staged) {
     // 2048 chunks of 16 bytes, eight per thread; chunk c of row r sits at position c ^ (r % 16) so
     // that the sixteen rows a wave reads at once spread over all banks
@@ -88,17 +113,6 @@ void dmq_rotate_kernel(RotParams p) {
     __syncthreads();
   }
   if (r_first >= r_end) return;
-
-  int rlog[TT];
-  bool valid[TT];
-  const __half* xrow[TT];
-#pragma unroll
-  for (int t = 0; t < TT; ++t) {
-    rlog[t] = r_first + t * 16 + l16;
-    valid[t] = rlog[t] < r_end;
-    int phys = valid[t] ? (row_index ? row_index[rlog[t]] : rlog[t]) : 0;
-    xrow[t] = p.x + (long)phys * p.x_stride + g * DMQ_GS + 8 * q;
-  }
   const __half* prow = rp.rot + (long)rot_g * (DMQ_GS * DMQ_GS) + (long)l16 * DMQ_GS + 8 * q;
 
   float4_t acc[8][TT];
@@ -114,10 +128,7 @@ void dmq_rotate_kernel(RotParams p) {
     for (int s = 0; s < 4; ++s) {
       half8_t b[TT];
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        uint4_t raw = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
-        b[t] = __builtin_bit_cast(half8_t, raw);
-      }
+      for (int t = 0; t < TT; ++t) b[t] = __builtin_bit_cast(half8_t, xraw[s][t]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const half8_t a = __builtin_bit_cast(half8_t, load_a(j, s));
@@ -277,13 +288,20 @@ void dmq_quantize_kernel(QuantParams p) {
 }
 
 // --------------------------------------------------------------------------------------------
+#ifndef DMQ_ROT_STAGE_MIN_TILES
+#define DMQ_ROT_STAGE_MIN_TILES 1
+#endif
 // tiled_waves: waves of the per-work-item part (max_items * tile_rows / (16*tt) * groups); the
 // whole-batch pools add n_hoisted * ceil(row tiles / 4) * groups workgroups in front
 template <int MODE>
 static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStream_t stream) {
   RotParams p = p_in;
   const long row_tiles = ((long)p.rows + 16 * tt - 1) / (16 * tt);
-  p.hoisted_wgs_per_pool = (int)(((row_tiles + 3) / 4) * p.groups);
+  // four row tiles share a staged matrix; measured faster than one matrix read per wave at
+  // every batch size (a single row tile included: four waves fetch the matrix together)
+  p.hoisted_staged = row_tiles >= DMQ_ROT_STAGE_MIN_TILES;
+  p.hoisted_wgs_per_pool = p.hoisted_staged ? (int)(((row_tiles + 3) / 4) * p.groups)
+                                            : (int)((row_tiles * p.groups + 3) / 4);
   if (p.hoisted_wgs_per_pool < 1) p.hoisted_wgs_per_pool = 1;
   const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + (tiled_waves + 3) / 4;
   if (total > 0x7fffffffL) return DMQ_ERR_LIMIT;

@@ -266,7 +266,9 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   for (int i = 0; i < a->n_pools; ++i) {
     const dmq_gemm_pool& q = a->pool[i];
     if (!q.act || !q.w || !q.norms || !q.expert_info) return DMQ_ERR_NULL;
-    if (q.mode == a->mode && a->mode != DMQ_MODE_FP4 && !q.lut) return DMQ_ERR_NULL;
+    if (q.mode == a->mode && a->mode != DMQ_MODE_FP4 && !q.lut &&
+        !(a->mode == DMQ_MODE_A8 && q.bit == 8))          // 8-bit int8: NULL = identity table
+      return DMQ_ERR_NULL;
     if (q.mode == a->mode && a->mode != DMQ_MODE_A16 && !q.act_scale) return DMQ_ERR_NULL;
     if (q.n_total <= 0 || q.n_total % 16) return DMQ_ERR_ALIGN;
   }

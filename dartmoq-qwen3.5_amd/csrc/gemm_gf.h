@@ -134,12 +134,20 @@ template <int N> __device__ __forceinline__ void dmq_load_words(const uint8_t* p
 }
 
 // Expand the packed bytes of MFMA step S into the lane's operand words.
-template <int MODE, int BIT, int S>
+// IDENT (int8 operands, 8-bit indices): the table is the identity w = idx - 128 of a uniform
+// codebook, so the operand bytes are the index bytes with the top bit flipped and no table is read.
+template <int MODE, int BIT, int S, bool IDENT = false>
 __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t lane_base,
                                                  const uint32_t* pk, uint32_t* w) {
   using T = ModeTraits<MODE>;
   using G = LutGeom<BIT, T::ES>;
   constexpr int BYTES = (4 * BIT) / T::STEPS;           // packed bytes per step
+  if constexpr (IDENT) {
+    static_assert(MODE == DMQ_MODE_A8 && BIT == 8, "identity table: int8 operands, 8-bit indices");
+#pragma unroll
+    for (int i = 0; i < BYTES / 4; ++i) w[i] = pk[S * (BYTES / 4) + i] ^ 0x80808080u;
+    return;
+  }
   auto one = [&](auto bc) {
     constexpr int b = decltype(bc)::value;
     constexpr int bi = S * BYTES + b;
@@ -220,7 +228,7 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
                                                        : (RED_BYTES > 16 ? RED_BYTES : 16);
 };
 
-template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG>
+template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG, bool IDENT = false>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
                                               uint8_t* smem2, uint8_t* smem_post, int token_start,
                                               int token_count, int slice_start, int post_slice,
@@ -330,11 +338,11 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr int WQ = (MODE == DMQ_MODE_FP4) ? 1 : T::STEPS * OPW;
   auto dequant_tile = [&](const uint32_t (&pkj)[WW], uint32_t (&w)[WQ]) {
     if constexpr (MODE != DMQ_MODE_FP4) {
-      dmq_dequant_step<MODE, BIT, 0>(tbl, lane_base, pkj, w);
-      if constexpr (T::STEPS > 1) dmq_dequant_step<MODE, BIT, 1>(tbl, lane_base, pkj, w + OPW);
+      dmq_dequant_step<MODE, BIT, 0, IDENT>(tbl, lane_base, pkj, w);
+      if constexpr (T::STEPS > 1) dmq_dequant_step<MODE, BIT, 1, IDENT>(tbl, lane_base, pkj, w + OPW);
       if constexpr (T::STEPS > 2) {
-        dmq_dequant_step<MODE, BIT, 2>(tbl, lane_base, pkj, w + 2 * OPW);
-        dmq_dequant_step<MODE, BIT, 3>(tbl, lane_base, pkj, w + 3 * OPW);
+        dmq_dequant_step<MODE, BIT, 2, IDENT>(tbl, lane_base, pkj, w + 2 * OPW);
+        dmq_dequant_step<MODE, BIT, 3, IDENT>(tbl, lane_base, pkj, w + 3 * OPW);
       }
     }
   };
@@ -360,7 +368,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         const half8_t n8 = {n, n, n, n, n, n, n, n};
         auto step = [&](auto sc) {
           constexpr int s = decltype(sc)::value;
-          if (j + 1 < NT) dmq_dequant_step<MODE, BIT, s>(tbl, lane_base, pk[j + 1 < NT ? j + 1 : j], wn + s * OPW);
+          if (j + 1 < NT) dmq_dequant_step<MODE, BIT, s, IDENT>(tbl, lane_base, pk[j + 1 < NT ? j + 1 : j], wn + s * OPW);
           const half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[4 * s], wq[4 * s + 1],
                                                                     wq[4 * s + 2], wq[4 * s + 3]}) * n8;
 #pragma unroll
@@ -496,7 +504,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     };
     // the first chunk is in flight while the look-up table is built
     if (g_lo < g_hi) load_chunk(g_lo);
-    if (MODE != DMQ_MODE_FP4) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
+    if (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
     __syncthreads();
     for (int g0 = g_lo; g0 < g_hi; g0 += PF) {
       if (g0 != g_lo) load_chunk(g0);
@@ -842,7 +850,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     // the codebook entries of this thread's table row are requested first: they arrive while
     // the weights are still in flight and the table is ready one memory latency after launch
     uint32_t lutw[4];
-    if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_fetch<BIT, T::ES>(pw.lut, threadIdx.x, lutw);
+    if constexpr (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_fetch<BIT, T::ES>(pw.lut, threadIdx.x, lutw);
 #pragma unroll
     for (int u = 0; u < D; ++u) {
       stage_load(lk, g_first + lg, srb[u]);
@@ -850,7 +858,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       next_load();
     }
     DMQ_MARK(1);
-    if constexpr (MODE != DMQ_MODE_FP4) dmq_lut_store_wave<BIT, T::ES>(tbl, wave, lutw);
+    if constexpr (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_store_wave<BIT, T::ES>(tbl, wave, lutw);
     DMQ_MARK(2);
     stage_store(0, srb[0]);
     __syncthreads();
@@ -1007,7 +1015,10 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   if constexpr (MODE == DMQ_MODE_FP4) {
     dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
   } else if constexpr (WIDE) {
-    dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
+    if (MODE == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
+      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG, MODE == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
+    else
+      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
   } else {
     switch (pw.bit) {
       case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;

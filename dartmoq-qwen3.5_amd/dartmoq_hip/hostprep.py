@@ -102,6 +102,14 @@ def build_int8_lut(codebook: torch.Tensor):
     return build_int8_codebook(codebook)
 
 
+def int8_lut_for_launch(codebook: torch.Tensor, device):
+    """(table or None, step) as the int8 GEMM launches take it: 8-bit uniform codebooks pass no
+    table (the kernels compute w = idx - 128 from the index bytes), everything else its rounded
+    int8 table on the device."""
+    q, step = build_int8_lut(codebook)
+    return (None if codebook.numel() == 256 else q.to(device)), step
+
+
 def build_fp8_codebook(codebook: torch.Tensor, n_coarse: int = 512):
     """(cb_e4m3, cb_scale) by the log-grid scale search of triton_kernels_fp8.py:35-87."""
     cb = codebook.detach().float().cpu()

@@ -377,18 +377,6 @@ def wxa8_matmul_merged_in_features_gf(x_i8, x_scale, indices_packed_gf, codebook
                       norms_prescaled, cfg)
 
 
-_IDENTITY_CB: dict[str, torch.Tensor] = {}
-
-
-def _identity_cb(device) -> torch.Tensor:
-    """w = idx - 128 as a 256-entry int8 table: what the reference's IDENTITY_CB kernels compute
-    without a table (triton_kernels_a8.py:769-799)."""
-    key = str(device)
-    if key not in _IDENTITY_CB:
-        _IDENTITY_CB[key] = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8).to(device)
-    return _IDENTITY_CB[key]
-
-
 def wxa8_matmul_grouped_gf(x_i8, x_scale, indices_packed_gf, codebook_i8, norms_gf, group_size,
                            num_groups, bit_width: int = 8, identity_cb: bool = False, cfg=None):
     """triton_kernels_a8.py:769-799, the kernel of WxA8Linear.forward: the whole matrix, norms_gf
@@ -397,7 +385,7 @@ def wxa8_matmul_grouped_gf(x_i8, x_scale, indices_packed_gf, codebook_i8, norms_
     if identity_cb:
         if bit_width != 8:
             raise ValueError("identity_cb needs bit_width 8")
-        codebook_i8 = _identity_cb(x_i8.device)
+        codebook_i8 = None                      # the kernel computes idx - 128 itself
     return _qa_slice_rows(MODE_A8, "wxa8 grouped", x_i8, x_scale.half(), indices_packed_gf,
                           codebook_i8, norms_gf, group_size, num_groups * group_size, 0,
                           indices_packed_gf.shape[1], bit_width, True)

@@ -104,8 +104,7 @@ class WxA16Linear:
             if self.MODE == MODE_A16:
                 ctx = (self.codebook, 1.0)
             elif self.MODE == MODE_A8:
-                q, step = hostprep.build_int8_lut(self.codebook)
-                ctx = (q.to(self.device), step)
+                ctx = hostprep.int8_lut_for_launch(self.codebook, self.device)
             else:
                 q, scale = hostprep.build_fp8_codebook(self.codebook)
                 ctx = (q.to(self.device), scale)

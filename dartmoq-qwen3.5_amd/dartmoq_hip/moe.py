@@ -69,9 +69,9 @@ class BitPoolWeights:
         if mode == MODE_A16:
             ctx["gu_lut"], ctx["dn_lut"] = self.gu_codebook, self.dn_codebook
         elif mode == MODE_A8:
-            gq, gstep = hostprep.build_int8_lut(self.gu_codebook)
-            dq, dstep = hostprep.build_int8_lut(self.dn_codebook)
-            ctx.update(gu_lut=gq.to(dev), dn_lut=dq.to(dev), gu_extra=gstep, dn_extra=dstep)
+            gq, gstep = hostprep.int8_lut_for_launch(self.gu_codebook, dev)
+            dq, dstep = hostprep.int8_lut_for_launch(self.dn_codebook, dev)
+            ctx.update(gu_lut=gq, dn_lut=dq, gu_extra=gstep, dn_extra=dstep)
         elif mode == MODE_FP8:
             gq, gs_ = hostprep.build_fp8_codebook(self.gu_codebook)
             dq, ds_ = hostprep.build_fp8_codebook(self.dn_codebook)

@@ -183,7 +183,9 @@ int dmq_quantize_act(int mode, const void* x, int x_fp32, long x_stride, int row
 typedef struct {
   const void* w;            /* idx_gf, or folded e2m1 [G, N, 64] for FP4 */
   const void* norms;        /* norms_gf */
-  const void* lut;          /* fp16 / int8 / e4m3 codebook; unused for FP4 */
+  const void* lut;          /* fp16 / int8 / e4m3 codebook; unused for FP4.  DMQ_MODE_A8 with bit 8:
+                               NULL = the identity w = idx - 128 of a uniform codebook (the
+                               reference's IDENTITY_CB, triton_kernels_a8.py:769-799), no table read */
   const void* expert_info;
   const void* act;          /* activation codes of this pool, row-major */
   const void* act_scale;    /* fp16 [rows, act_scale_stride] (A8/FP8), u8 (FP4), NULL (A16) */

@@ -205,6 +205,10 @@ def test_wxa8_linear_8bit_identity_codebook():
     dummy = torch.zeros(256, dtype=torch.int8, device="cuda")
     o = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, dummy, norms_pre, 128, 4, 8, identity_cb=True)
     assert torch.equal(o, lin(x.cuda()))
+    # ... and the table-free kernel gives the bits of the look-up kernel fed the identity table
+    table = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8).cuda()
+    o_tab = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, table, norms_pre, 128, 4, 8, identity_cb=False)
+    assert torch.equal(o, o_tab)
     lloyd = _packed8(128, 256, seed=4, uniform=False)
     with pytest.raises(ValueError):
         dartmoq_hip.WxA8Linear.from_wxa16(dartmoq_hip.WxA16Linear.from_packed(lloyd))

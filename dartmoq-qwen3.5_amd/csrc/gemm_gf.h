@@ -186,6 +186,12 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
 #ifndef DMQ_SCHED
 #define DMQ_SCHED 1
 #endif
+#ifndef DMQ_KOUT
+#define DMQ_KOUT 1
+#endif
+#ifndef DMQ_KOUT_MIN_TT
+#define DMQ_KOUT_MIN_TT 2
+#endif
 #ifndef DMQ_FOLD_MIN_TT
 #define DMQ_FOLD_MIN_TT 2
 #endif
@@ -774,6 +780,64 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       }
     };
 
+    // ---- 64-row tiles of fp16 layers: MFMA steps outermost.  The activation operands of one step
+    // (16 registers) are read from the slot while the previous step computes instead of holding
+    // the whole tile (64 registers), and the look-ups run two (step, n-tile) pairs ahead of their
+    // MFMAs.  Every accumulator sees its operands in the same order as in the tile-outer loop.
+    constexpr bool KOUT = DMQ_KOUT && MODE == DMQ_MODE_A16 && FOLD && TT >= DMQ_KOUT_MIN_TT;
+    auto compute_kouter = [&](int buf, const uint32_t (&pk)[NT][WW]) {
+      if constexpr (KOUT) {
+        const uint8_t* slot = stage + buf * SLOT;
+        half8_t n8[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const _Float16 n = __builtin_bit_cast(
+              _Float16, *(const uint16_t*)(slot + NORM_OFF + ((wave * NT + j) * 16 + l16) * 2));
+          n8[j] = (half8_t){n, n, n, n, n, n, n, n};
+        }
+        uint4_t braw[2][TT];
+        auto read_b = [&](auto sc, uint4_t (&dst)[TT]) {
+          constexpr int s_ = decltype(sc)::value;
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            const int row = t * 16 + l16;
+            const int c = q * (AW / 4) + s_;
+            dst[t] = *(const uint4_t*)(slot + row * AB + ((c ^ (row & (NC - 1))) * 16));
+          }
+        };
+        uint32_t wq[3][4];
+        auto look = [&](auto mc) {
+          constexpr int m = decltype(mc)::value;
+          if constexpr (m < 4 * NT)
+            dmq_dequant_step<MODE, BIT, m / NT, IDENT>(tbl, lane_base, pk[m % NT], wq[m % 3]);
+        };
+        read_b(std::integral_constant<int, 0>{}, braw[0]);
+        look(std::integral_constant<int, 0>{});
+        look(std::integral_constant<int, 1>{});
+        auto micro = [&](auto mc) {
+          constexpr int m = decltype(mc)::value;
+          constexpr int s_ = m / NT, j = m % NT;
+          look(std::integral_constant<int, m + 2>{});
+          if constexpr (j == 0 && s_ + 1 < 4) read_b(std::integral_constant<int, s_ + 1>{}, braw[(s_ + 1) & 1]);
+          const half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[m % 3][0], wq[m % 3][1],
+                                                                    wq[m % 3][2], wq[m % 3][3]}) * n8[j];
+#pragma unroll
+          for (int t = 0; t < TT; ++t)
+            total_acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                a, __builtin_bit_cast(half8_t, braw[s_ & 1][t]), total_acc[j][t], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        micro(std::integral_constant<int, 0>{});  micro(std::integral_constant<int, 1>{});
+        micro(std::integral_constant<int, 2>{});  micro(std::integral_constant<int, 3>{});
+        micro(std::integral_constant<int, 4>{});  micro(std::integral_constant<int, 5>{});
+        micro(std::integral_constant<int, 6>{});  micro(std::integral_constant<int, 7>{});
+        micro(std::integral_constant<int, 8>{});  micro(std::integral_constant<int, 9>{});
+        micro(std::integral_constant<int, 10>{}); micro(std::integral_constant<int, 11>{});
+        micro(std::integral_constant<int, 12>{}); micro(std::integral_constant<int, 13>{});
+        micro(std::integral_constant<int, 14>{}); micro(std::integral_constant<int, 15>{});
+      }
+    };
+
     // ---- K range shared by several workgroups: park the sums of the valid rows in this
     // workgroup's plane, take a ticket, and let the last arrival add the planes (always in plane
     // order, its own from registers, so the result does not depend on the order of arrival).
@@ -871,12 +935,16 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         const bool live = sb + u < steps;              // uniform over the workgroup
         stage_load(lk, g_first + lg, srb[u]);          // entry u went to LDS one step ago
         if (live) {
-          uint32_t xa[TT][AW];
-          uint2_t nr[NT];
-          float xs[TT];
-          int xsb[TT];
-          stage_read(u & 1, xa, nr, xs, xsb);
-          compute(cg, pkb[u], nr, xa, xs, xsb);
+          if constexpr (KOUT) {
+            compute_kouter(u & 1, pkb[u]);
+          } else {
+            uint32_t xa[TT][AW];
+            uint2_t nr[NT];
+            float xs[TT];
+            int xsb[TT];
+            stage_read(u & 1, xa, nr, xs, xsb);
+            compute(cg, pkb[u], nr, xa, xs, xsb);
+          }
         }
         load_packed(lk, g_first + lg, pkb[u]);
         next_load();

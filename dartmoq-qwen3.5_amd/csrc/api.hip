@@ -38,6 +38,12 @@ static inline int pick_ks(int tt, long rows, int groups) {
 #define DMQ_SPLIT_MAX_ROWS 1024
 // single-block workgroups at the end of every XCD's share of a GEMM launch that otherwise walks
 // several blocks per workgroup: one round of resident workgroups (32 CUs x 3)
+#ifndef DMQ_DOWN_TT4_MIN_AVG
+#define DMQ_DOWN_TT4_MIN_AVG 512
+#endif
+#ifndef DMQ_TT4_MIN_AVG
+#define DMQ_TT4_MIN_AVG 112
+#endif
 #ifndef DMQ_TAIL_SLOTS
 #define DMQ_TAIL_SLOTS 96
 #endif
@@ -51,7 +57,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 10; }
+int dmq_abi_version(void) { return 11; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -288,6 +294,12 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   }
   if (a->act_row_bytes < (long)a->groups * act_bytes_per_group(a->mode)) return DMQ_ERR_SHAPE;
   const int wsplit = a->k_split > 1 ? a->k_split : 1;
+  int subs = 1;
+  if (a->item_tile_rows > 0) {
+    if (a->item_tile_rows % (16 * a->tt)) return DMQ_ERR_ALIGN;
+    subs = a->item_tile_rows / (16 * a->tt);
+    if (subs > 1 && wsplit > 1) return DMQ_ERR_MODE;
+  }
   if (wsplit > 1) {
     if ((wsplit != 2 && wsplit != 4) || !silu || ks != 1 || a->tt != 1 || any_wide) return DMQ_ERR_MODE;
     if (a->groups % wsplit || a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
@@ -323,6 +335,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.post_scale = a->post_scale;
   p.post_scale_stride = a->post_scale_stride;
   p.wsplit = wsplit;
+  p.subs = subs;
   p.split_rows = a->split_rows;
   p.split_partial = (float*)a->split_partial;
   p.split_counter = (int*)a->split_counter;
@@ -349,11 +362,11 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     L.wide = wide;
     long work;
     if (p.tail_slots > 0) {
-      long per_xcd = ((long)a->max_items * p.n_blocks + DMQ_XCDS - 1) / DMQ_XCDS;
+      long per_xcd = ((long)a->max_items * subs * p.n_blocks + DMQ_XCDS - 1) / DMQ_XCDS;
       per_xcd = (per_xcd + nbl - 1) / nbl * nbl;
       work = (per_xcd / nbl + p.tail_slots) * DMQ_XCDS;
     } else {
-      work = (long)a->max_items * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
+      work = (long)a->max_items * subs * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
       work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
     }
     if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
@@ -444,9 +457,10 @@ static inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static int pick_tt(int tokens, int top_k, int experts) {
   const long avg = (long)tokens * top_k / (experts > 0 ? experts : 1);
-  // 64-row tiles pay off once padding is small: they halve the look-ups per row but run two
-  // workgroups per CU instead of three
-  return avg <= 8 ? 1 : (avg <= 160 ? 2 : 4);
+  // 64-row work items pay off once the experts are big: the gate_up GEMM then halves its look-ups
+  // per row (two workgroups per CU instead of three); measured equal at 96 rows per expert, -1 %
+  // at 128, -4 % at 256.  The down GEMM keeps 32-row tiles on those items (down_tt below).
+  return avg <= 8 ? 1 : (avg <= DMQ_TT4_MIN_AVG ? 2 : 4);
 }
 
 static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* base) {
@@ -544,7 +558,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   }
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   if (nbl <= 0) nbl = pick_nbl((long)tokens * K, tt);
-  const int rot_tt = tt;               // a rotation wave covers one row tile of the work items
+  // a rotation wave covers 16 or 32 rows: 64-row work items are rotated by two waves each
+  const int rot_tt = tt > 2 ? 2 : tt;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
   if (w.bytes > workspace_bytes) return DMQ_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
@@ -732,7 +747,12 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
     dmq_gemm_args d{};
-    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt; d.ks = ks; d.nbl = nbl; d.n_pools = P;
+    // 64-row work items: the down GEMM (K = I, four steps per block) runs them as two 32-row tiles
+    // until the experts are big enough for its 64-row kernel to pay
+    const long avg_rows = (long)tokens * K / E;
+    const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
+    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt;
+    d.ks = ks; d.nbl = nbl; d.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       d.pool[i] = dmq_gemm_pool{pd.dn_w, pd.dn_norms, pd.dn_lut, w.dn_info + (size_t)i * E * 4,

@@ -83,6 +83,7 @@ struct GemmParams {
   const int* n_items;          // device scalar
   int n_blocks;                // blocks of output features per item
   int nbl;                     // consecutive blocks one workgroup walks (1 unless KS == 1)
+  int subs;                    // row tiles of this launch per work item (item rows / (16 * TT))
   int tail_slots;              // > 0: the last tail_slots blocks of every XCD's share go one per
                                // workgroup (nbl > 1, nbl divides n_blocks, wsplit == 1)
   // outputs
@@ -1038,7 +1039,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
     // across blocks, one table build for several blocks), its last tail_slots blocks one per
     // workgroup, so that the last round of workgroups is short and full instead of long and
     // half empty.
-    const int total_blocks = p.n_items[0] * p.n_blocks;
+    const int total_blocks = p.n_items[0] * p.subs * p.n_blocks;
     int per_xcd = (total_blocks + DMQ_XCDS - 1) / DMQ_XCDS;
     per_xcd = (per_xcd + p.nbl - 1) / p.nbl * p.nbl;
     const int xcd = blockIdx.x % DMQ_XCDS;
@@ -1054,7 +1055,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
     nbc = min(slot < big ? p.nbl : 1, p.n_blocks - nb);
   } else {
     const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl * wsplit;   // workgroups per item
-    const int total = p.n_items[0] * nbg;
+    const int total = p.n_items[0] * p.subs * nbg;
     const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
     const int slot = blockIdx.x / DMQ_XCDS;
     const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
@@ -1066,13 +1067,17 @@ void dmq_gemm_gf_kernel(GemmParams p) {
     nbc = min(p.nbl, p.n_blocks - nb);
   }
   int* ticket = XSPLIT ? p.split_counter + (long)item * p.n_blocks + nb : nullptr;
+  // a work item of 16 * TT * subs rows is `subs` row tiles of this launch
+  const int vsub = item % p.subs;
+  item /= p.subs;
   const int4_t* rec = (const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * item);
   const int4_t r0 = rec[0];
   const int4_t r1 = rec[1];
   const int pool = r0[0];
-  const int ttile = r0[2];
+  const int ttile = r0[2] * p.subs + vsub;
   const int token_start = r0[3];
   const int token_count = r1[0];
+  if (ttile * (16 * TT) >= token_count) return;          // row tile past the item's last row
   const int slice_start = p.slice_is_groups ? r1[2] : r1[1];
   // first down group of the item's expert: its gate_up slice starts at weight row 2 * start, its
   // down slice at group start / 128 (holds for items of either origin)

@@ -290,12 +290,14 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
-                 row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None):
+                 row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None,
+                 item_tile_rows=0):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
     out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 shares the groups
     of every (item, feature block) between that many workgroups (16-row tiles, SiLU epilogues);
-    ``rows_total`` then bounds the routed row indices."""
+    ``rows_total`` then bounds the routed row indices.  ``item_tile_rows``: rows per work item
+    when the list was built for a larger tile than 16 * tt."""
     a = GemmArgs()
     a.mode, a.epi, a.tt, a.ks, a.nbl, a.n_pools = mode, epi, tt, ks, nbl, len(pools)
     dev = None
@@ -332,6 +334,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
         if post.get("scale") is not None:
             a.post_scale = post["scale"].data_ptr()
             a.post_scale_stride = post["scale"].stride(0)
+    a.item_tile_rows = int(item_tile_rows)
     if k_split > 1:
         if rows_total is None:
             raise ValueError("k_split needs rows_total")
@@ -346,7 +349,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
 def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *, groups, n_out,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
-                  tiling=None, dbg_acc=None, post=None, k_split=0):
+                  tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -354,7 +357,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
     if tt is None:
         tt = pick_tt(rows_total, n_exp)
     if tiling is None:
-        tiling = build_tiles(expert_info, rows_total, 16 * tt)
+        tiling = build_tiles(expert_info, rows_total, item_tile_rows or 16 * tt)
     n_items, items, max_items = tiling
     if out is None:
         if epi == EPI_SCATTER:
@@ -366,7 +369,8 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         slice_is_groups=slice_is_groups, tt=tt, ks=ks, nbl=nbl, out=out,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
-                        dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total)
+                        dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total,
+                        item_tile_rows=item_tile_rows)
 
 
 def combine_slots(slots: torch.Tensor, top_k: int, add: torch.Tensor | None = None) -> torch.Tensor:

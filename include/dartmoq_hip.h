@@ -211,7 +211,8 @@ typedef struct {
   int n_out;                /* output features per row (SILU: I) */
   int half_width;           /* SILU: I */
   int slice_is_groups;      /* 0 gate_up (slice offsets rows), 1 down (slice offsets groups) */
-  const void* items;        /* from dmq_build_tiles / dmq_route_permute, tile_rows == 16*tt */
+  const void* items;        /* from dmq_build_tiles / dmq_route_permute, tile_rows == 16*tt, or
+                               item_tile_rows when that is set */
   const void* n_items;
   int max_items;
   void* out;                /* STORE/SILU: fp16 [rows, out_stride]; SCATTER: fp16 [slots, out_stride] */
@@ -242,6 +243,10 @@ typedef struct {
   int split_rows;
   void* split_partial;
   void* split_counter;
+  /* Rows per work item of `items` when it differs from 16*tt (0 = 16*tt): a multiple of 16*tt;
+   * the launch walks every item as item_tile_rows / (16*tt) row tiles.  Lets one work-item list
+   * serve launches of different tile sizes.  Not with k_split. */
+  int item_tile_rows;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

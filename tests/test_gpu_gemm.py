@@ -312,3 +312,37 @@ def test_fused_down_rotation_equals_separate_kernels(mode, tt, nbl):
     assert torch.equal(codes.view(torch.uint8), want.view(torch.uint8))
     if sc is not None:
         assert torch.equal(sc.view(torch.uint8), want_scale.view(torch.uint8))
+
+
+@pytest.mark.parametrize("mode", [A16, A8, FP4])
+@pytest.mark.parametrize("tt,item_rows", [(1, 64), (2, 64), (1, 32)])
+def test_work_items_larger_than_the_launch_tile(mode, tt, item_rows):
+    """item_tile_rows: one work-item list (64- or 32-row items) serves a launch with smaller row
+    tiles; every item is walked as item_tile_rows / (16 tt) tiles and the output equals, bit for
+    bit, the launch over items of its own tile size (ragged counts, an empty expert, counts that
+    end inside the first sub-tile)."""
+    from dartmoq_hip import ops
+    bit, k, n_slice = 2, 256, 128
+    counts = [70, 3, 0, 33, 64, 17]
+    n_exp = len(counts)
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(23 + mode)
+    idx_gf, norms_gf, cb = _pool(bit, n_slice * n_exp, k, 5)
+    x_rot = torch.randn(rows_total, k, generator=g) * 0.7
+    act, scale, _oc, _os, lut, _ol, _wbs, nfac, wsb = _mode_inputs(mode, x_rot, cb)
+    norms_used = (norms_gf.float() * nfac).half() if mode == FP4 else norms_gf
+    w_dev = idx_gf.cuda()
+    if mode == FP4:
+        w_dev = ops.fold_indices_to_e2m1(w_dev, lut, bit)
+    info = torch.tensor([(starts[e], counts[e], e * n_slice, n_slice) for e in range(n_exp)],
+                        dtype=torch.int32).cuda()
+    args = (mode, bit, STORE, act.cuda(), None if scale is None else scale.cuda(), w_dev,
+            norms_used.cuda(), None if mode == FP4 else lut.cuda(), info)
+    kw = dict(groups=k // 128, n_out=n_slice, slice_is_groups=False, rows_total=rows_total,
+              w_scale_byte=wsb, tt=tt)
+    own = ops.matmul_merged(*args, **kw)
+    big = ops.matmul_merged(*args, item_tile_rows=item_rows, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(own, big)
+    with pytest.raises(ValueError):                 # not a multiple of the launch tile
+        ops.matmul_merged(*args, item_tile_rows=48, **dict(kw, tt=2))

@@ -44,6 +44,9 @@ static inline int pick_ks(int tt, long rows, int groups) {
 #ifndef DMQ_TT4_MIN_AVG
 #define DMQ_TT4_MIN_AVG 112
 #endif
+#ifndef DMQ_HOIST_ALL_TOKENS
+#define DMQ_HOIST_ALL_TOKENS 512
+#endif
 #ifndef DMQ_TAIL_SLOTS
 #define DMQ_TAIL_SLOTS 96
 #endif
@@ -593,14 +596,21 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       if (layer->pool[i].mode == modes[mi] && layer->pool[i].bit == 8) fuse_rot[mi] = false;
   }
 
+  // Which pools rotate every token once instead of their routed rows: the caller's choice (pools
+  // expected to see more routed rows than tokens) and, for small batches, all of them: rotating a
+  // few dozen tokens for a pool that ends up using a handful is cheaper than the dependent
+  // per-work-item pass (same values either way).
+  bool whole_batch[DMQ_MAX_POOLS] = {false, false, false, false};
+  for (int i = 0; i < P; ++i) whole_batch[i] = layer->pool[i].major != 0 || tokens <= DMQ_HOIST_ALL_TOKENS;
+
   // The pools whose rows are rotated per work item come first in the item list, so that the
   // rotation launch knows their items as a prefix (n_items[1]) and touches no other record.
   int pool_order[DMQ_MAX_POOLS] = {0, 1, 2, 3}, lead_pools = 0;
   {
     int n = 0;
-    for (int i = 0; i < P; ++i) if (layer->pool[i].major == 0) pool_order[n++] = i;
+    for (int i = 0; i < P; ++i) if (!whole_batch[i]) pool_order[n++] = i;
     lead_pools = n;
-    for (int i = 0; i < P; ++i) if (layer->pool[i].major != 0) pool_order[n++] = i;
+    for (int i = 0; i < P; ++i) if (whole_batch[i]) pool_order[n++] = i;
   }
 
   // 1. top-k (when the router hands over logits), shared columns, sort by expert, per-pool
@@ -663,7 +673,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       const int pi = i < P ? i : 0;
       const dmq_pool_desc& pd = layer->pool[pi];
       const bool live = i < P && pd.mode == mode;
-      const bool hoisted = pd.major != 0;
+      const bool hoisted = whole_batch[pi];
       const long row_bytes = (long)H * 2;
       rp.pool[i] = RotPool{(const __half*)pd.gu_rot, hoisted ? w.xq[pi] : w.xq_rows, row_bytes,
                            hoisted ? (void*)w.xq_scale[pi] : (void*)w.xq_rows_scale,
@@ -691,7 +701,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
-      const bool hoisted = pd.major != 0;
+      const bool hoisted = whole_batch[i];
       g.post_rot[i] = pd.dn_rot;
       g.post_extra_scale[i] = pd.dn_extra_scale;
       g.pool[i] = dmq_gemm_pool{pd.gu_w, pd.gu_norms, pd.gu_lut, w.gu_info + (size_t)i * E * 4,

@@ -1,5 +1,6 @@
 // extern "C" surface of libdartmoq_hip.so: argument checks, workspace carving and launches.
 #include "params.h"
+#include "topk.h"
 #include "gemm_dispatch.h"
 
 __global__ __launch_bounds__(256) void dmq_fill_zero_kernel(uint32_t* p, long n_words) {
@@ -613,14 +614,63 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     for (int i = 0; i < P; ++i) if (whole_batch[i]) pool_order[n++] = i;
   }
 
+  // Rotation (+ quantization) of the gate_up input of one precision mode.  whole: the pools that
+  // rotate every token once (no dependence on the routing step); tiled: the pools rotated per
+  // work item; tp: the router's top-k rides the same launch.
+  auto rotate_gate_up_input = [&](int mode, bool whole, bool tiled, const TopkParams* tp,
+                                  int tp_fp16) -> int {
+    RotParams rp{};
+    rp.x = (const __half*)x; rp.x_stride = H; rp.row_index = w.sorted_tokens;
+    rp.rows = tokens; rp.groups = H / DMQ_GS;
+    rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0;
+    rp.items_prefix = 1;
+    bool any_tiled = false;
+    for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
+      const int pi = i < P ? i : 0;
+      const dmq_pool_desc& pd = layer->pool[pi];
+      const bool live = i < P && pd.mode == mode;
+      const bool hoisted = whole_batch[pi];
+      const long row_bytes = (long)H * 2;
+      rp.pool[i] = RotPool{(const __half*)pd.gu_rot, hoisted ? w.xq[pi] : w.xq_rows, row_bytes,
+                           hoisted ? (void*)w.xq_scale[pi] : (void*)w.xq_rows_scale,
+                           scale_stride_for(pd.mode, H), w.gu_info + (size_t)pi * E * 4,
+                           pd.gu_extra_scale, live ? pd.mode : -1, hoisted ? 1 : 0, 0};
+      if (live && hoisted && whole) rp.hoisted_pool[rp.n_hoisted++] = i;
+      if (live && !hoisted && tiled) any_tiled = true;
+    }
+    long n = 0;                                    // waves of the per-work-item part
+    if (any_tiled) n = (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
+    else rp.items = nullptr;
+    if (rp.n_hoisted == 0 && !any_tiled && !tp) return DMQ_OK;
+    return dmq_rotate_dispatch(mode, rp, n, rot_tt, st, tp, tp_fp16);
+  };
+  const bool route_small = (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
+                           K <= 64 && (!router->logits || tokens <= DMQ_ROUTE_SMALL_TOKENS);
+  // When the top-k is a launch of its own (logits, more than 16 tokens) it shares the launch of the
+  // whole-batch rotation of the first mode: neither needs the other, both are short.
+  bool whole_done[DMQ_MAX_POOLS] = {false, false, false, false};   // per mode
+  bool topk_done = false;
+  if (!route_small && router->logits) {
+    bool any_whole = false;
+    for (int i = 0; i < P; ++i) any_whole |= (whole_batch[i] && layer->pool[i].mode == modes[0]);
+    const int rk = K - n_shared, re = E - n_shared;
+    if (any_whole && re <= 1024 && rk <= 64 && rk <= re && rk > 0 && n_shared <= 64) {
+      const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
+      const TopkParams tp{router->logits, tokens, re, rk, router->renorm, w.topk_w, w.topk_idx, sg,
+                          (tokens + 3) / 4};
+      rc = rotate_gate_up_input(modes[0], true, false, &tp, router->logits_fp16);
+      if (rc) return rc;
+      whole_done[0] = true;
+      topk_done = true;
+    }
+  }
+
   // 1. top-k (when the router hands over logits), shared columns, sort by expert, per-pool
   //    expert_info, work items: one launch for small batches
   {
     const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
     const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
-    const bool small = (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
-                       K <= 64 && (!router->logits || tokens <= DMQ_ROUTE_SMALL_TOKENS);
-    if (small) {
+    if (route_small) {
       RouteSmallParams sp{};
       sp.logits = router->logits; sp.logits_fp16 = router->logits_fp16;
       sp.in_idx = (const int*)router->topk_idx; sp.in_w = (const float*)router->topk_w;
@@ -643,7 +693,9 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     } else {
       const void* tk_idx = router->topk_idx;
       const void* tk_w = router->topk_w;
-      if (router->logits || n_shared > 0) {
+      if (topk_done) {
+        tk_idx = w.topk_idx; tk_w = w.topk_w;
+      } else if (router->logits || n_shared > 0) {
         rc = dmq_route_topk_launch(router->logits, router->logits_fp16, (const int*)router->topk_idx,
                                    (const float*)router->topk_w, tokens, re, rk, router->renorm,
                                    w.topk_w, w.topk_idx, sg, st);
@@ -661,31 +713,10 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   if (rc) return rc;
   mark(1);
 
-  // 2. gate_up input: rotate (+quantize) once per token (hoisted pools) or per routed row
+  // 2. gate_up input: rotate (+quantize) once per token (whole-batch pools not yet done) and per
+  //    routed row (the other pools)
   for (int mi = 0; mi < n_modes; ++mi) {
-    const int mode = modes[mi];
-    RotParams rp{};
-    rp.x = (const __half*)x; rp.x_stride = H; rp.row_index = w.sorted_tokens;
-    rp.rows = tokens; rp.groups = H / DMQ_GS;
-    rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0; rp.items_prefix = 1;
-    bool any_tiled = false;
-    for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
-      const int pi = i < P ? i : 0;
-      const dmq_pool_desc& pd = layer->pool[pi];
-      const bool live = i < P && pd.mode == mode;
-      const bool hoisted = whole_batch[pi];
-      const long row_bytes = (long)H * 2;
-      rp.pool[i] = RotPool{(const __half*)pd.gu_rot, hoisted ? w.xq[pi] : w.xq_rows, row_bytes,
-                           hoisted ? (void*)w.xq_scale[pi] : (void*)w.xq_rows_scale,
-                           scale_stride_for(pd.mode, H), w.gu_info + (size_t)pi * E * 4,
-                           pd.gu_extra_scale, live ? pd.mode : -1, hoisted ? 1 : 0, 0};
-      if (live && hoisted) rp.hoisted_pool[rp.n_hoisted++] = i;
-      if (live && !hoisted) any_tiled = true;
-    }
-    long n = 0;                                    // waves of the per-work-item part
-    if (any_tiled) n = (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
-    else rp.items = nullptr;
-    rc = dmq_rotate_dispatch(mode, rp, n, rot_tt, st);
+    rc = rotate_gate_up_input(modes[mi], !whole_done[mi], true, nullptr, 0);
     if (rc) return rc;
   }
 

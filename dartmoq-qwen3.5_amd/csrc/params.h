@@ -117,7 +117,10 @@ struct RouteSmallParams {
 };
 int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream);
 
-int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream);
+struct TopkParams;
+// tp != NULL: the launch also runs the router's top-k (workgroups in front; logits fp16 or fp32)
+int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream,
+                        const TopkParams* tp = nullptr, int topk_fp16 = 0);
 int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
 int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx, const float* in_w,
                           int tokens, int experts, int k, int renorm, float* out_w, int* out_idx,

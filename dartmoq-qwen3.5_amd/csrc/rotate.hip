@@ -19,6 +19,8 @@
 // routed to their experts, following the layer's work-item list, and may pick the matrix by
 // expert (the down rotations).
 #include "params.h"
+#include "topk.h"
+#include <type_traits>
 
 __device__ __forceinline__ float wave_max16x4(float v) {
   v = fmaxf(v, __shfl_xor(v, 16, 64));
@@ -26,9 +28,10 @@ __device__ __forceinline__ float wave_max16x4(float v) {
   return v;
 }
 
+// One workgroup of the rotation launch (`block` = its index among the rotation workgroups, `mat` =
+// 32 KiB of LDS for the staged matrix).
 template <int MODE, int TT>
-__global__ __launch_bounds__(256)
-void dmq_rotate_kernel(RotParams p) {
+__device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int block, uint8_t* mat) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int l16 = lane & 15;
@@ -39,15 +42,14 @@ void dmq_rotate_kernel(RotParams p) {
   // one group and four consecutive row tiles (one per wave) and stages the group's matrix in LDS
   // once.  The remaining workgroups take one work item per wave and read their matrices (one
   // per expert with rot_use_slice) straight from memory.
-  __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
   int pool, g, r_first, r_end, rot_g;
   const int* row_index = nullptr;
   const long hoisted_wgs = (long)p.n_hoisted * p.hoisted_wgs_per_pool;
-  const bool hoisted = (long)blockIdx.x < hoisted_wgs;                // uniform over the workgroup
+  const bool hoisted = (long)block < hoisted_wgs;                // uniform over the workgroup
   const bool staged = hoisted && p.hoisted_staged;
   if (hoisted) {
-    pool = p.hoisted_pool[blockIdx.x / p.hoisted_wgs_per_pool];
-    const int local = blockIdx.x % p.hoisted_wgs_per_pool;
+    pool = p.hoisted_pool[block / p.hoisted_wgs_per_pool];
+    const int local = block % p.hoisted_wgs_per_pool;
     if (staged) {
       g = local % p.groups;
       r_first = ((local / p.groups) * 4 + wave) * ROWS_PER_ITEM;
@@ -60,7 +62,7 @@ void dmq_rotate_kernel(RotParams p) {
     rot_g = g;
   } else {
     if (!p.items) return;
-    long item = ((long)blockIdx.x - hoisted_wgs) * 4 + wave;
+    long item = ((long)block - hoisted_wgs) * 4 + wave;
     g = (int)(item % p.groups);
     const long rt = item / p.groups;
     const int sub = p.tile_rows / ROWS_PER_ITEM;          // waves per work item
@@ -228,6 +230,24 @@ void dmq_rotate_kernel(RotParams p) {
 }
 
 // --------------------------------------------------------------------------------------------
+template <int MODE, int TT>
+__global__ __launch_bounds__(256)
+void dmq_rotate_kernel(RotParams p) {
+  __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
+  dmq_rotate_wg<MODE, TT>(p, blockIdx.x, mat);
+}
+
+// The same launch with the router's top-k in front: workgroups [0, tp.blocks) take four tokens
+// each (one per wave), the rest rotate.  Neither part depends on the other, so the launch costs
+// the longer of the two instead of their sum.
+template <int MODE, int TT, typename LT>
+__global__ __launch_bounds__(256)
+void dmq_rotate_topk_kernel(RotParams p, TopkParams tp) {
+  __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
+  if ((int)blockIdx.x < tp.blocks) dmq_topk_wg<LT>(tp, blockIdx.x);
+  else dmq_rotate_wg<MODE, TT>(p, (int)blockIdx.x - tp.blocks, mat);
+}
+
 // Quantization of activations that are already rotated (no matrix product): one wave per
 // (row, group), two consecutive features per lane.
 template <int MODE>
@@ -294,7 +314,8 @@ void dmq_quantize_kernel(QuantParams p) {
 // tiled_waves: waves of the per-work-item part (max_items * tile_rows / (16*tt) * groups); the
 // whole-batch pools add n_hoisted * ceil(row tiles / 4) * groups workgroups in front
 template <int MODE>
-static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStream_t stream) {
+static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStream_t stream,
+                         const TopkParams* tp, int topk_fp16) {
   RotParams p = p_in;
   const long row_tiles = ((long)p.rows + 16 * tt - 1) / (16 * tt);
   // four row tiles share a staged matrix; measured faster than one matrix read per wave at
@@ -303,22 +324,37 @@ static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStr
   p.hoisted_wgs_per_pool = p.hoisted_staged ? (int)(((row_tiles + 3) / 4) * p.groups)
                                             : (int)((row_tiles * p.groups + 3) / 4);
   if (p.hoisted_wgs_per_pool < 1) p.hoisted_wgs_per_pool = 1;
-  const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + (tiled_waves + 3) / 4;
+  const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + (tiled_waves + 3) / 4 +
+                     (tp ? tp->blocks : 0);
   if (total > 0x7fffffffL) return DMQ_ERR_LIMIT;
   const int grid = (int)total;
   if (grid <= 0) return DMQ_OK;
+  if (tp) {
+    auto go = [&](auto tt_tag) {
+      constexpr int T_ = decltype(tt_tag)::value;
+      if (topk_fp16)
+        hipLaunchKernelGGL((dmq_rotate_topk_kernel<MODE, T_, __half>), dim3(grid), dim3(256), 0, stream, p, *tp);
+      else
+        hipLaunchKernelGGL((dmq_rotate_topk_kernel<MODE, T_, float>), dim3(grid), dim3(256), 0, stream, p, *tp);
+    };
+    if (tt == 4) go(std::integral_constant<int, 4>{});
+    else if (tt == 2) go(std::integral_constant<int, 2>{});
+    else go(std::integral_constant<int, 1>{});
+    return dmq_check_launch();
+  }
   if (tt == 4) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 4>), dim3(grid), dim3(256), 0, stream, p);
   else if (tt == 2) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 2>), dim3(grid), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 1>), dim3(grid), dim3(256), 0, stream, p);
   return dmq_check_launch();
 }
 
-int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream) {
+int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream,
+                        const TopkParams* tp, int topk_fp16) {
   switch (mode) {
-    case DMQ_MODE_A16: return launch_rotate<DMQ_MODE_A16>(p, tiled_waves, tt, stream);
-    case DMQ_MODE_A8: return launch_rotate<DMQ_MODE_A8>(p, tiled_waves, tt, stream);
-    case DMQ_MODE_FP8: return launch_rotate<DMQ_MODE_FP8>(p, tiled_waves, tt, stream);
-    case DMQ_MODE_FP4: return launch_rotate<DMQ_MODE_FP4>(p, tiled_waves, tt, stream);
+    case DMQ_MODE_A16: return launch_rotate<DMQ_MODE_A16>(p, tiled_waves, tt, stream, tp, topk_fp16);
+    case DMQ_MODE_A8: return launch_rotate<DMQ_MODE_A8>(p, tiled_waves, tt, stream, tp, topk_fp16);
+    case DMQ_MODE_FP8: return launch_rotate<DMQ_MODE_FP8>(p, tiled_waves, tt, stream, tp, topk_fp16);
+    case DMQ_MODE_FP4: return launch_rotate<DMQ_MODE_FP4>(p, tiled_waves, tt, stream, tp, topk_fp16);
   }
   return DMQ_ERR_MODE;
 }

@@ -10,6 +10,7 @@
 //   4. dmq_chunk_fill_kernel  one wave per chunk: write its rows to their sorted positions
 //   5. dmq_combine_kernel     out[t] = sum over the k slot rows of token t (fixed order)
 #include "params.h"
+#include "topk.h"
 #include <type_traits>
 
 // developer instrumentation of the one-workgroup routing kernel: wall-clock stamps (100 MHz) of
@@ -23,134 +24,6 @@ extern "C" int dmq_route_trace_read(long long* out) {
 #else
 #define DMQ_RMARK(i)
 #endif
-
-// ------------------------------------------------------------------------------ top-k
-// Wave-wide max / min through data-parallel lane moves: xor 1, xor 2, mirror within 8 and within
-// 16 lanes leave every lane with the result of its row of 16; the four rows are then combined
-// through scalar registers.  The result is uniform over the wave.
-template <typename F>
-__device__ __forceinline__ int wave_reduce_i32(int v, F op) {
-  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
-  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
-  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, true));   // row_half_mirror
-  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, true));   // row_mirror
-  const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
-  const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
-  return op(op(a, b), op(c, d));
-}
-__device__ __forceinline__ float wave_max_f32(float v) {
-  // finite floats and -inf order like their bit patterns after this monotone map
-  auto key = [](float f) { int b = __builtin_bit_cast(int, f); return b >= 0 ? b : (int)(0x80000000u - (unsigned)b); };
-  const int k = wave_reduce_i32(key(v), [](int x, int y) { return x > y ? x : y; });
-  return __builtin_bit_cast(float, k >= 0 ? k : (int)(0x80000000u - (unsigned)k));
-}
-__device__ __forceinline__ int wave_min_i32(int v) {
-  return wave_reduce_i32(v, [](int x, int y) { return x < y ? x : y; });
-}
-
-template <typename T> __device__ __forceinline__ float to_f32(T v);
-template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
-template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
-
-// Always-on shared experts ride the routed path as n_shared extra columns of the top-k arrays:
-// column k + j names expert `experts + j` with weight sigmoid(x . gate_row), rounded to fp16 after
-// the dot and after the sigmoid like an fp16 Linear followed by torch.sigmoid.  Wave-uniform result.
-__device__ __forceinline__ float dmq_shared_gate_value(const SharedGate& sg, int tok, int lane) {
-  const __half* xr = sg.x + (long)tok * sg.hidden;
-  float dot = 0.f;
-  for (int h = lane * 8; h < sg.hidden; h += 512) {
-    const half8_t a = *(const half8_t*)(xr + h);
-    const half8_t b = *(const half8_t*)(sg.gate_row + h);
-#pragma unroll
-    for (int c = 0; c < 8; ++c) dot += (float)a[c] * (float)b[c];
-  }
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) dot += __shfl_xor(dot, m, 64);
-  const float z = (float)(_Float16)dot;
-  return (float)(_Float16)(1.f / (1.f + expf(-z)));
-}
-
-__device__ __forceinline__ void dmq_shared_columns(const SharedGate& sg, int tok, int experts, int k,
-                                                   int lane, float* out_w, int* out_idx) {
-  if (sg.n_shared <= 0) return;
-  const float g = dmq_shared_gate_value(sg, tok, lane);
-  const int stride = k + sg.n_shared;
-  if (lane < sg.n_shared) {
-    out_w[(long)tok * stride + k + lane] = g;
-    out_idx[(long)tok * stride + k + lane] = experts + lane;
-  }
-}
-
-// softmax + top-k of one token by one wave: lane j < k returns the j-th largest probability and
-// its expert (lowest expert index wins ties).  NV values per lane cover up to 64 * NV experts;
-// the loads are a call of their own so that a caller can request the next token's row early.
-template <typename T, int NV>
-__device__ __forceinline__ void dmq_topk_load(const T* row, int experts, int lane, float (&v)[NV]) {
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    int e = lane + 64 * i;
-    v[i] = (e < experts) ? to_f32<T>(row[e]) : -INFINITY;
-  }
-}
-
-template <int NV>
-__device__ __forceinline__ void dmq_topk_select(float (&v)[NV], int experts, int k, int renorm, int lane,
-                                                float& my_w, int& my_e) {
-  float vmax = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) vmax = fmaxf(vmax, v[i]);
-  vmax = wave_max_f32(vmax);
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) sum += (lane + 64 * i < experts) ? expf(v[i] - vmax) : 0.f;
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) sum += __shfl_xor(sum, m, 64);
-
-  float my_v = -INFINITY;
-  my_e = 0;
-  for (int round = 0; round < k; ++round) {
-    float bv = -INFINITY;
-    int be = 0x7fffffff;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      int e = lane + 64 * i;
-      if (v[i] > bv) { bv = v[i]; be = e; }
-    }
-    // wave arg-max in two reductions: the largest value, then the lowest expert index holding it
-    const float top = wave_max_f32(bv);
-    be = wave_min_i32(bv == top ? be : 0x7fffffff);
-    if (lane == round) { my_v = top; my_e = be; }
-    if ((be & 63) == lane) {
-#pragma unroll
-      for (int i = 0; i < NV; ++i)
-        if (i == (be >> 6)) v[i] = -INFINITY;
-    }
-  }
-  // lane j turns the j-th logit into its probability; the kept mass is summed in round order
-  my_w = (lane < k) ? expf(my_v - vmax) / sum : 0.f;
-  if (renorm) {
-    float wsum = 0.f;
-    for (int j = 0; j < k; ++j) wsum += __shfl(my_w, j, 64);
-    my_w = my_w / wsum;
-  }
-}
-
-// The sum of exponentials runs over the same values in the same order for every NV, so the
-// weights do not depend on which instance serves a layer.
-template <typename T>
-__device__ __forceinline__ void dmq_topk_token(const T* row, int experts, int k, int renorm, int lane,
-                                               float& my_w, int& my_e) {
-  if (experts <= 256) {
-    float v[4]; dmq_topk_load<T, 4>(row, experts, lane, v);
-    dmq_topk_select<4>(v, experts, k, renorm, lane, my_w, my_e);
-  } else if (experts <= 512) {
-    float v[8]; dmq_topk_load<T, 8>(row, experts, lane, v);
-    dmq_topk_select<8>(v, experts, k, renorm, lane, my_w, my_e);
-  } else {
-    float v[16]; dmq_topk_load<T, 16>(row, experts, lane, v);
-    dmq_topk_select<16>(v, experts, k, renorm, lane, my_w, my_e);
-  }
-}
 
 // Widen caller-made top-k arrays [tokens, k] by the shared columns.
 __global__ __launch_bounds__(256)
@@ -169,20 +42,8 @@ void dmq_topk_widen_kernel(const int* in_idx, const float* in_w, int tokens, int
 
 template <typename T>
 __global__ __launch_bounds__(256)
-void dmq_topk_kernel(const T* logits, int tokens, int experts, int k, int renorm,
-                     float* out_w, int* out_idx, SharedGate sg) {
-  const int lane = threadIdx.x & 63;
-  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (tok >= tokens) return;
-  float my_w;
-  int my_e;
-  dmq_topk_token<T>(logits + (long)tok * experts, experts, k, renorm, lane, my_w, my_e);
-  const int stride = k + sg.n_shared;
-  if (lane < k) {
-    out_w[(long)tok * stride + lane] = my_w;
-    out_idx[(long)tok * stride + lane] = my_e;
-  }
-  dmq_shared_columns(sg, tok, experts, k, lane, out_w, out_idx);
+void dmq_topk_kernel(TopkParams tp) {
+  dmq_topk_wg<T>(tp, blockIdx.x);
 }
 
 // ------------------------------------------------------------------------------ counting
@@ -736,12 +597,11 @@ int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx
   if (!logits)
     hipLaunchKernelGGL(dmq_topk_widen_kernel, dim3(grid), dim3(256), 0, stream, in_idx, in_w, tokens,
                        experts, k, out_w, out_idx, sg);
-  else if (logits_fp16)
-    hipLaunchKernelGGL(dmq_topk_kernel<__half>, dim3(grid), dim3(256), 0, stream,
-                       (const __half*)logits, tokens, experts, k, renorm, out_w, out_idx, sg);
-  else
-    hipLaunchKernelGGL(dmq_topk_kernel<float>, dim3(grid), dim3(256), 0, stream,
-                       (const float*)logits, tokens, experts, k, renorm, out_w, out_idx, sg);
+  else {
+    const TopkParams tp{logits, tokens, experts, k, renorm, out_w, out_idx, sg, grid};
+    if (logits_fp16) hipLaunchKernelGGL(dmq_topk_kernel<__half>, dim3(grid), dim3(256), 0, stream, tp);
+    else hipLaunchKernelGGL(dmq_topk_kernel<float>, dim3(grid), dim3(256), 0, stream, tp);
+  }
   return dmq_check_launch();
 }
 

@@ -343,8 +343,9 @@ typedef struct {
 /* The whole layer from the router's output: dmq_moe_ffn_forward_staged plus the routing step.
  * layer->experts and layer->top_k count the n_shared always-on slices (experts E .. E+n_shared-1,
  * selected by every token with the gate value as routing weight).  For up to 1024 routed rows
- * and 512 experts (16 tokens when the top-k is computed here) top-k, shared columns, sort and
- * work-item list are a single one-workgroup launch.  stage_events / aux_out as in
+ * and 512 experts shared columns, sort and work-item list are a single one-workgroup launch,
+ * which also computes the top-k for up to 4 tokens; for more tokens the top-k shares the launch
+ * of the whole-batch rotation.  stage_events / aux_out as in
  * dmq_moe_ffn_forward_staged (the first stage then includes the top-k); both may be NULL. */
 int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_args* router,
                                const void* x, int tokens, const void* add_f16, void* out,

@@ -46,7 +46,7 @@ static inline int pick_ks(int tt, long rows, int groups) {
 #define DMQ_TT4_MIN_AVG 112
 #endif
 #ifndef DMQ_HOIST_ALL_TOKENS
-#define DMQ_HOIST_ALL_TOKENS 512
+#define DMQ_HOIST_ALL_TOKENS 1024
 #endif
 #ifndef DMQ_TAIL_SLOTS
 #define DMQ_TAIL_SLOTS 96

@@ -29,6 +29,7 @@ struct RotParams {
   int hoisted_pool[DMQ_MAX_POOLS];
   int hoisted_wgs_per_pool;     // set by the launcher
   int hoisted_staged;           // 1: workgroup = one group x four row tiles, matrix staged in LDS
+  int tiled_staged;             // same for the per-work-item part (set by the launcher)
   const int* items;        // [*, DMQ_ITEM_WORDS] work-item records
   const int* n_items;
   int tile_rows;           // rows per work item (multiple of 16*TT)

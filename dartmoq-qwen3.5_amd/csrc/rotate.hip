@@ -43,6 +43,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
   // once.  The remaining workgroups take one work item per wave and read their matrices (one
   // per expert with rot_use_slice) straight from memory.
   int pool, g, r_first, r_end, rot_g;
+  int stage_pool = -1;                                  // tiled workgroups: pool whose matrix is staged
   const int* row_index = nullptr;
   const long hoisted_wgs = (long)p.n_hoisted * p.hoisted_wgs_per_pool;
   const bool hoisted = (long)block < hoisted_wgs;                // uniform over the workgroup
@@ -60,6 +61,32 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
     }
     r_end = p.rows;
     rot_g = g;
+  } else if (p.tiled_staged) {
+    // per-work-item pools whose matrices depend on the group only: a workgroup owns one group and
+    // four consecutive row tiles of the item list and stages the matrix of its first item's
+    // pool; a wave whose item belongs to another pool reads its matrix from memory instead
+    if (!p.items) return;
+    const long tb = (long)block - hoisted_wgs;
+    g = (int)(tb % p.groups);
+    const long rt0 = (tb / p.groups) * 4;
+    const int sub = p.tile_rows / ROWS_PER_ITEM;          // waves per work item
+    const int n_lim = p.n_items[p.items_prefix ? 1 : 0];
+    if (rt0 / sub >= n_lim) return;                       // whole workgroup past the list
+    const int pool0 = p.items[DMQ_ITEM_WORDS * (rt0 / sub)];
+    stage_pool = (p.pool[pool0].mode == MODE && !p.pool[pool0].hoisted) ? pool0 : -1;
+    const long rt = rt0 + wave;
+    const long tile = rt / sub;
+    pool = pool0;
+    r_first = 0; r_end = 0; rot_g = g;
+    if (tile < n_lim) {
+      const int* it = p.items + DMQ_ITEM_WORDS * tile;
+      pool = it[0];
+      if (!p.pool[pool].hoisted && p.pool[pool].mode == MODE) {
+        r_first = it[3] + it[2] * p.tile_rows + (int)(rt % sub) * ROWS_PER_ITEM;
+        r_end = it[3] + it[4];
+      }
+    }
+    row_index = p.row_index;
   } else {
     if (!p.items) return;
     long item = ((long)block - hoisted_wgs) * 4 + wave;
@@ -80,7 +107,8 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
     row_index = p.row_index;
   }
   const RotPool& rp = p.pool[pool];
-  if (rp.mode != MODE) return;
+  const bool tiled_wg = !hoisted && p.tiled_staged;
+  if (!tiled_wg && rp.mode != MODE) return;
 
   int rlog[TT];
   bool valid[TT];
@@ -99,10 +127,12 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
 #pragma unroll
     for (int t = 0; t < TT; ++t)
       xraw[s][t] = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
-  if (staged) {
+  const bool stage_now = staged || (tiled_wg && stage_pool >= 0);   // uniform over the workgroup
+  if (stage_now) {
     // 2048 chunks of 16 bytes, eight per thread; chunk c of row r sits at position c ^ (r % 16) so
     // that the sixteen rows a wave reads at once spread over all banks
-    const uint4_t* src = (const uint4_t*)(rp.rot + (long)rot_g * (DMQ_GS * DMQ_GS));
+    const __half* src_rot = staged ? rp.rot : p.pool[stage_pool].rot;
+    const uint4_t* src = (const uint4_t*)(src_rot + (long)g * (DMQ_GS * DMQ_GS));
     uint4_t v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = src[threadIdx.x + 256 * i];
@@ -114,6 +144,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
     }
     __syncthreads();
   }
+  const bool from_lds = staged || (tiled_wg && pool == stage_pool);
   if (r_first >= r_end) return;
   const __half* prow = rp.rot + (long)rot_g * (DMQ_GS * DMQ_GS) + (long)l16 * DMQ_GS + 8 * q;
 
@@ -140,7 +171,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
       }
     }
   };
-  if (staged) {
+  if (from_lds) {
     // row j*16 + l16 of the matrix, chunk 4s + q
     const uint8_t* mrow = mat + l16 * 256;
     product([&](int j, int s) {
@@ -324,8 +355,17 @@ static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStr
   p.hoisted_wgs_per_pool = p.hoisted_staged ? (int)(((row_tiles + 3) / 4) * p.groups)
                                             : (int)((row_tiles * p.groups + 3) / 4);
   if (p.hoisted_wgs_per_pool < 1) p.hoisted_wgs_per_pool = 1;
-  const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + (tiled_waves + 3) / 4 +
-                     (tp ? tp->blocks : 0);
+  // per-work-item part: matrices that depend on the group only are staged per workgroup (one
+  // group, four row tiles); per-expert matrices (rot_use_slice) keep one task per wave
+  bool sliced = false;
+  for (int i = 0; i < DMQ_MAX_POOLS; ++i) sliced |= (p.pool[i].mode >= 0 && p.pool[i].rot_use_slice != 0);
+  p.tiled_staged = !sliced;
+  long tiled_wgs = (tiled_waves + 3) / 4;
+  if (p.tiled_staged && tiled_waves > 0) {
+    const long row_tasks = tiled_waves / p.groups;          // row tiles of the item list
+    tiled_wgs = ((row_tasks + 3) / 4) * p.groups;
+  }
+  const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + tiled_wgs + (tp ? tp->blocks : 0);
   if (total > 0x7fffffffL) return DMQ_ERR_LIMIT;
   const int grid = (int)total;
   if (grid <= 0) return DMQ_OK;

@@ -61,7 +61,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 11; }
+int dmq_abi_version(void) { return 12; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -286,7 +286,13 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (a->max_items <= 0) return DMQ_ERR_EMPTY;
   if (a->groups <= 0 || a->n_out <= 0) return DMQ_ERR_SHAPE;
   const bool silu = a->epi == DMQ_EPI_SILU || a->epi == DMQ_EPI_SILU_ROT;
-  const int feat_per_wave = silu ? 32 : 64;
+  // one n-tile per wave: the launch of a Linear with a handful of rows (any bit width)
+  const bool one_tile = a->nt == 1;
+  if (a->nt != 0 && a->nt != 4 && !one_tile) return DMQ_ERR_MODE;
+  if (one_tile && (a->epi != DMQ_EPI_STORE || a->tt != 1 || ks != 4 || a->mode == DMQ_MODE_FP4 ||
+                 a->dbg_acc || a->k_split > 1))
+    return DMQ_ERR_MODE;
+  const int feat_per_wave = silu ? 32 : (one_tile ? 16 : 64);
   if (a->n_out % feat_per_wave) return DMQ_ERR_ALIGN;
   if (silu && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
   if (a->epi == DMQ_EPI_SILU_ROT) {
@@ -305,8 +311,13 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (subs > 1 && wsplit > 1) return DMQ_ERR_MODE;
   }
   if (wsplit > 1) {
-    if ((wsplit != 2 && wsplit != 4) || !silu || ks != 1 || a->tt != 1 || any_wide) return DMQ_ERR_MODE;
-    if (a->groups % wsplit || a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
+    // SiLU epilogues: 2 or 4 workgroups, 1/2/4-bit pools; plain store (a Linear with a handful
+    // of rows): up to 16, any bit width
+    const bool store = a->epi == DMQ_EPI_STORE;
+    if (!silu && !store) return DMQ_ERR_MODE;
+    if (wsplit != 2 && wsplit != 4 && !(store && (wsplit == 8 || wsplit == 16))) return DMQ_ERR_MODE;
+    if (ks != 1 || a->tt != 1 || (any_wide && !store)) return DMQ_ERR_MODE;
+    if (a->groups % wsplit || (silu && a->n_out % DMQ_GS)) return DMQ_ERR_ALIGN;
     if (!a->split_partial || !a->split_counter) return DMQ_ERR_NULL;
     if (a->split_rows <= 0) return DMQ_ERR_SHAPE;
   }
@@ -345,13 +356,14 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.split_counter = (int*)a->split_counter;
   L.epi = a->epi;
   L.tt = a->tt;
+  L.nt = one_tile ? 1 : 4;
   L.dbg = a->dbg_acc != nullptr;
   L.stream = (hipStream_t)stream;
   // the 1/2/4-bit pools and the 8-bit pools of the mode are separate launches over the same work
   // list (each skips the items of the other kind); 8-bit pools never split K over the waves
   for (int wide = 0; wide < 2; ++wide) {
     if (!(wide ? any_wide : any_narrow)) continue;
-    const int lks = wide ? 1 : ks;
+    const int lks = (wide && !one_tile) ? 1 : ks;
     const int feat_per_block = (4 / lks) * feat_per_wave;
     p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
     // several n-blocks per workgroup need every block complete and the waves on distinct features

@@ -9,7 +9,8 @@ struct GemmLaunch {
   int tt;          // activation tiles of 16 rows per wave: 1, 2 or 4
   int ks;          // waves splitting K: 1, 2 or 4
   int dbg;
-  int wide;        // 1: the pools of 8-bit indices (ks must be 1), 0: the 1/2/4-bit pools
+  int wide;        // 1: the pools of 8-bit indices (ks must be 1 unless nt == 1), 0: the 1/2/4-bit pools
+  int nt;          // n-tiles per wave: 4, or 1 (plain store, tt == 1, ks == 4 only)
   int grid;
   hipStream_t stream;
 };
@@ -52,8 +53,27 @@ static int dmq_gemm_launch_epi(const GemmLaunch& L) {
   return DMQ_ERR_MODE;
 }
 
+// one n-tile per wave, K split over the four waves: the launch of a Linear with few rows
+template <int MODE>
+static int dmq_gemm_launch_narrow(const GemmLaunch& L) {
+  if constexpr (MODE != DMQ_MODE_FP4) {
+    if (L.wide)
+      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, 1, DMQ_EPI_STORE, 4, false, true, 1>), dim3(L.grid),
+                         dim3(256), 0, L.stream, L.p);
+    else
+      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, 1, DMQ_EPI_STORE, 4, false, false, 1>), dim3(L.grid),
+                         dim3(256), 0, L.stream, L.p);
+    return dmq_check_launch();
+  }
+  return DMQ_ERR_MODE;
+}
+
 template <int MODE>
 static int dmq_gemm_launch_mode(const GemmLaunch& L) {
+  if (L.nt == 1) {
+    if (L.tt != 1 || L.ks != 4 || L.epi != DMQ_EPI_STORE || L.dbg) return DMQ_ERR_MODE;
+    return dmq_gemm_launch_narrow<MODE>(L);
+  }
   if (L.dbg && !(MODE == DMQ_MODE_A8 && L.tt == 1 && L.ks == 1 && L.epi == DMQ_EPI_STORE))
     return DMQ_ERR_MODE;
   if (L.tt == 1 && L.ks == 4) return dmq_gemm_launch_epi<MODE, 1, 4>(L);

@@ -98,12 +98,12 @@ struct GemmParams {
   long post_row_bytes;
   void* post_scale;            // A8/FP8: fp16 [rows, post_scale_stride]; FP4: u8 [rows, post_scale_stride]
   int post_scale_stride;
-  // K range of one (item, block) shared by wsplit workgroups (16-row tiles, SiLU epilogues): each
-  // parks its fp32 sums in its plane of split_partial and takes a ticket; the last one adds the
-  // planes in plane order and runs the epilogue
-  int wsplit;                  // 1, 2 or 4
+  // K range of one (item, block) shared by wsplit workgroups (16-row tiles, SiLU and plain-store
+  // epilogues): each parks its fp32 sums in its plane of split_partial and takes a ticket; the
+  // last one adds the planes in plane order and runs the epilogue
+  int wsplit;                  // 1, 2, 4, 8 or 16
   int split_rows;              // rows of one plane
-  float* split_partial;        // fp32 [wsplit, split_rows, 2 * n_out]
+  float* split_partial;        // fp32 [wsplit, split_rows, 2 * n_out (SiLU) or n_out (store)]
   int* split_counter;          // int32 [max_items * n_blocks], zero before the launch and after it
 };
 
@@ -226,7 +226,9 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
   static constexpr int AW = ModeTraits<MODE>::ACT_WORDS;          // activation words per lane and group
   static constexpr int AB = AW * 16;                              // activation bytes per row and group
   static constexpr bool STAGE = (KS == 1);                        // activations through LDS
-  static constexpr int PF = 4;                                    // direct path: groups in flight
+  // direct path: groups in flight (a wave with a single n-tile keeps eight: its registers allow it
+  // and a 4096-wide K split over four waves is then one round trip)
+  static constexpr int PF = (NT == 1) ? 8 : 4;
   // staged path: one LDS slot = activation tile + norms of the 64*NT weight rows + tile scales
   static constexpr int SLOT = 16 * TT * AB + 128 * NT + 64 * TT;
   static constexpr int STAGE_BYTES = STAGE ? 2 * SLOT : 0;
@@ -256,7 +258,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr int FEAT_TILES = NT / UNIT;                              // output tiles per wave
   constexpr int PPG = (MODE == DMQ_MODE_FP4) ? 64 : (DMQ_GS * BIT / 8);
   constexpr int FPB = ROWPARTS * FEAT_TILES * 16;                    // output features per n-block
-  constexpr bool XSPLIT = STAGE && TT == 1 && SILU;                  // K range shared across workgroups
+  // K range shared across workgroups
+  constexpr bool XSPLIT = STAGE && TT == 1 && (SILU || EPI == DMQ_EPI_STORE);
   static_assert(NT % UNIT == 0, "SiLU epilogue pairs gate/up tiles");
 
   const int lane = threadIdx.x & 63;
@@ -847,14 +850,19 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     // to be acknowledged before the workgroup takes its ticket.
     auto split_gather = [&](int nsplit_) -> bool {
       using u64 = unsigned long long;
-      const long row_floats = 2L * p.n_out;
+      // one plane row holds the sums of a routed row: gate then up features (SiLU epilogues) or
+      // the output features (plain store)
+      const long row_floats = SILU ? 2L * p.n_out : (long)p.n_out;
       const long plane = (long)p.split_rows * row_floats;
       float* base = p.split_partial + (long)rlog[0] * row_floats + feat_k + 4 * q;
+      auto col = [&](int j) -> long {
+        return SILU ? (long)((j & 1) ? p.n_out : 0) + (j >> 1) * 16 : (long)j * 16;
+      };
       const bool mine = avalid[0] && wave_active;
       if (mine) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          u64* dst = (u64*)(base + (long)split * plane + ((j & 1) ? p.n_out : 0) + (j >> 1) * 16);
+          u64* dst = (u64*)(base + (long)split * plane + col(j));
           const float2_t lo = {total_acc[j][0][0], total_acc[j][0][1]};
           const float2_t hi = {total_acc[j][0][2], total_acc[j][0][3]};
           __hip_atomic_store(dst, __builtin_bit_cast(u64, lo), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -872,20 +880,28 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       __syncthreads();
       if (*wg_flag != nsplit_ - 1) return false;
       if (mine) {
+        // four planes are requested together; the sums are still taken in plane order
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           float4_t sum = (float4_t){0.f, 0.f, 0.f, 0.f};
-          for (int s = 0; s < nsplit_; ++s) {
-            float4_t v = total_acc[j][0];
-            if (s != split) {
-              const u64* src = (const u64*)(base + (long)s * plane + ((j & 1) ? p.n_out : 0) + (j >> 1) * 16);
-              const float2_t lo = __builtin_bit_cast(
-                  float2_t, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-              const float2_t hi = __builtin_bit_cast(
-                  float2_t, __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-              v = (float4_t){lo[0], lo[1], hi[0], hi[1]};
+          for (int s0 = 0; s0 < nsplit_; s0 += 4) {
+            float4_t v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int s = s0 + i;
+              v[i] = total_acc[j][0];
+              if (s < nsplit_ && s != split) {
+                const u64* src = (const u64*)(base + (long)s * plane + col(j));
+                const float2_t lo = __builtin_bit_cast(
+                    float2_t, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                const float2_t hi = __builtin_bit_cast(
+                    float2_t, __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                v[i] = (float4_t){lo[0], lo[1], hi[0], hi[1]};
+              }
             }
-            sum += v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (s0 + i < nsplit_) sum += v[i];
           }
           total_acc[j][0] = sum;
         }
@@ -1012,10 +1028,12 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 // WIDE kernels serve the pools of 8-bit indices (one byte per weight: twice the packed words per
 // lane of a 4-bit pool); they are separate instances so that their registers do not count against
 // the kernels of the 1/2/4-bit pools.  A launch skips the work items of the other kind.
-template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false>
+// NT: n-tiles of 16 features per wave.  Four everywhere except the instances for a Linear with a
+// handful of rows (NT = 1, K split over the four waves: a workgroup covers 16 features, so a
+// 4096-feature matrix gives 256 workgroups instead of 64).
+template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT = 4>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
-  constexpr int NT = 4;
   __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
 #ifndef DMQ_LDS_PAD
 #define DMQ_LDS_PAD 0
@@ -1029,7 +1047,8 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   // Workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD gets a contiguous range of
   // the work list, so the workgroups that share an activation tile (the feature blocks of an
   // item) and those that share weights (the row tiles of an expert) meet in one L2.
-  constexpr bool XSPLIT = KS == 1 && TT == 1 && (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT);
+  constexpr bool XSPLIT = KS == 1 && TT == 1 &&
+                          (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT || EPI == DMQ_EPI_STORE);
   __shared__ int wg_flag;
   const int wsplit = XSPLIT ? p.wsplit : 1;
   int item, nb, nbc, split = 0;

@@ -7,7 +7,7 @@ quantization/wxfp8/linear.py:37-100 (e4m3 activations and look-up table).  These
 of the shared expert of the MoE layer.  Like the reference's WxA8Linear._ensure_gf the module
 converts the checkpoint layout to group-first once (norms divided by sqrt(128)) and keeps the
 rotation matrices and the per-mode look-up table resident; a forward is two launches (rotate
-(+quantize), dequant GEMM) on the current stream.
+(+quantize), dequant GEMM) on the current stream, the GEMM tiled by batch size (_tiling).
 
 Bit widths 1, 2, 4 and 8 are built, all through a codebook look-up.  8-bit weights run on the int8
 path only with a uniform codebook (then the table is the identity w = idx - 128 and the step rides
@@ -22,6 +22,26 @@ from . import hostprep, ops
 from ._lib import EPI_STORE, MODE_A16, MODE_A8, MODE_FP8
 
 GROUP_SIZE = ops.GROUP_SIZE
+SPLIT_MAX_ROWS = 64          # batches up to this size split K between waves or workgroups
+
+
+_SPLIT_WS: dict = {}
+
+
+def _split_workspace(device, k: int, rows: int, n_out: int, items: int):
+    """fp32 planes and arrival counters of the K-sharing launches, one set per (device, stream):
+    launches on one stream run one after the other and every launch leaves the counters zero."""
+    dev = torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(dev).cuda_stream)
+    need_p = k * rows * n_out
+    need_c = items * ((n_out + 127) // 128)
+    ws = _SPLIT_WS.get(key)
+    if ws is None or ws[0].numel() < need_p or ws[1].numel() < need_c:
+        ws = (torch.empty(max(need_p, ws[0].numel() if ws else 0), dtype=torch.float32, device=dev),
+              torch.zeros(max(need_c, ws[1].numel() if ws else 0), dtype=torch.int32, device=dev))
+        _SPLIT_WS[key] = ws
+    return ws
 
 
 class WxA16Linear:
@@ -63,6 +83,7 @@ class WxA16Linear:
                                                              self.group_size, self.device)
         self._ctx: dict[int, tuple] = {}
         self._info: dict[int, torch.Tensor] = {}
+        self._tile_cache: dict = {}
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -121,13 +142,36 @@ class WxA16Linear:
         return info
 
     def _tiling(self, rows: int) -> dict:
-        """A Linear is a single "expert": with few rows its launch has out_features / 256
-        workgroups, so up to 64 rows the four waves of a workgroup split K instead and every
-        workgroup covers 64 features (four times as many workgroups; 41 -> 28 us for a 4-bit
-        4096 x 4096 matrix).  8-bit weights never split K inside a workgroup."""
-        if rows <= 64 and self.bit_width != 8:
+        """A Linear is a single "expert": with 16-row tiles its launch has rows / 16 x
+        out_features / 256 workgroups, far too few for 256 CUs when the rows are few.  Up to 16
+        rows every wave takes one n-tile and the four waves of a workgroup split K (a workgroup per
+        16 features: 35 -> 10 us for an 8-bit 4096 x 4096 matrix, 15 -> 10 us for a 4-bit one).  Up
+        to 64 rows the waves still split K over four n-tiles each, except for 8-bit weights, whose
+        K range is shared between four workgroups instead (fp32 partial sums, added in a fixed
+        order by the last workgroup to arrive: 35 -> 21 us)."""
+        if rows <= 16:
+            return {"tt": 1, "ks": 4, "nt": 1}
+        if rows > SPLIT_MAX_ROWS:
+            return {}
+        if self.bit_width != 8:
             return {"tt": 1, "ks": 4}
-        return {}
+        k = 4 if self.n_groups % 4 == 0 else (2 if self.n_groups % 2 == 0 else 1)
+        if k == 1:
+            return {"tt": 1}
+        # counters: one per (work item, feature block); the item list has rows // 16 + 1 slots
+        partial, counter = _split_workspace(self.device, k, rows, self.out_features, rows // 16 + 1)
+        return {"tt": 1, "ks": 1, "k_split": k, "split_ws": (partial, counter)}
+
+    def _tiles(self, rows: int, tile_rows: int):
+        """Work-item list of a batch of `rows` rows (device tensors, kept per batch size)."""
+        key = (rows, tile_rows)
+        t = self._tile_cache.get(key)
+        if t is None:
+            if len(self._tile_cache) >= 64:
+                self._tile_cache.pop(next(iter(self._tile_cache)))
+            t = ops.build_tiles(self._expert_info(rows), rows, tile_rows)
+            self._tile_cache[key] = t
+        return t
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -143,11 +187,14 @@ class WxA16Linear:
             return torch.empty(*shape[:-1], self.out_features, dtype=x.dtype, device=x.device)
         lut, extra = self._mode_ctx()
         codes, scale = ops.rotate(self.MODE, src, self.rot, extra_scale=extra, scale_fp32=False)
+        tiling = self._tiling(rows)
+        tt = tiling.get("tt") or ops.pick_tt(rows, 1)
+        tiling["tt"] = tt
         out = ops.matmul_merged(self.MODE, self.bit_width, EPI_STORE, codes,
                                 None if self.MODE == MODE_A16 else scale, self.indices_gf,
                                 self.norms_gf, lut, self._expert_info(rows), groups=self.n_groups,
                                 n_out=self.out_features, slice_is_groups=False, rows_total=rows,
-                                **self._tiling(rows))
+                                tiling=self._tiles(rows, 16 * tt), **tiling)
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out.reshape(*shape[:-1], self.out_features).to(x.dtype)

@@ -291,12 +291,15 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None,
-                 item_tile_rows=0):
+                 item_tile_rows=0, split_ws=None, nt=0):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
-    out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 shares the groups
-    of every (item, feature block) between that many workgroups (16-row tiles, SiLU epilogues);
-    ``rows_total`` then bounds the routed row indices.  ``item_tile_rows``: rows per work item
+    out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 (plain-store
+    epilogue: up to 16) shares the groups of every (item, feature block) between that many
+    workgroups (16-row tiles, SiLU and plain-store epilogues); ``rows_total`` then bounds the
+    routed row indices and ``split_ws`` = (fp32 planes, zeroed int32 counters) may bring the
+    scratch tensors in (allocated per call otherwise).  ``nt`` = 1: one n-tile per wave (plain
+    store, tt = 1, ks = 4; any bit width): the launch of a Linear with a handful of rows.  ``item_tile_rows``: rows per work item
     when the list was built for a larger tile than 16 * tt."""
     a = GemmArgs()
     a.mode, a.epi, a.tt, a.ks, a.nbl, a.n_pools = mode, epi, tt, ks, nbl, len(pools)
@@ -335,11 +338,19 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
             a.post_scale = post["scale"].data_ptr()
             a.post_scale_stride = post["scale"].stride(0)
     a.item_tile_rows = int(item_tile_rows)
+    a.nt = int(nt)
     if k_split > 1:
         if rows_total is None:
             raise ValueError("k_split needs rows_total")
-        partial = torch.empty((k_split, rows_total, 2 * n_out), dtype=torch.float32, device=dev)
-        counter = torch.zeros(max_items * ((n_out + 127) // 128), dtype=torch.int32, device=dev)
+        width = n_out if epi == EPI_STORE else 2 * n_out
+        n_counters = max_items * ((n_out + 127) // 128)
+        if split_ws is not None:
+            partial, counter = split_ws
+            if partial.numel() < k_split * rows_total * width or counter.numel() < n_counters:
+                raise ValueError("split_ws is too small for this launch")
+        else:
+            partial = torch.empty((k_split, rows_total, width), dtype=torch.float32, device=dev)
+            counter = torch.zeros(n_counters, dtype=torch.int32, device=dev)
         a.k_split, a.split_rows = k_split, rows_total
         a.split_partial, a.split_counter = partial.data_ptr(), counter.data_ptr()
     check(load().dmq_matmul_merged_gf(ctypes.byref(a), _stream(dev)), "matmul_merged_gf")
@@ -349,7 +360,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
 def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *, groups, n_out,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
-                  tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0):
+                  tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0, split_ws=None, nt=0):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -370,7 +381,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
                         dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total,
-                        item_tile_rows=item_tile_rows)
+                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt)
 
 
 def combine_slots(slots: torch.Tensor, top_k: int, add: torch.Tensor | None = None) -> torch.Tensor:

@@ -234,11 +234,14 @@ typedef struct {
   int post_scale_stride;
   /* k_split = 2 or 4 (0 / 1 = off): the groups of one (work item, feature block) are shared by
    * that many workgroups, for short work lists that leave most of the chip idle.  tt == 1,
-   * ks <= 1, a SILU epilogue, groups % k_split == 0; nbl is ignored.  Each workgroup parks its
-   * fp32 sums in split_partial (fp32 [k_split, split_rows, 2 * n_out], split_rows >= every routed
-   * row index + 1) and the last to arrive adds them in a fixed order and runs the epilogue.
-   * split_counter: int32 [max_items * n_out / 128], zero before the launch; the launch leaves it
-   * zero. */
+   * ks <= 1, groups % k_split == 0; nbl is ignored.  With a SILU epilogue: 1/2/4-bit pools,
+   * n_out a multiple of 128, split_partial fp32 [k_split, split_rows, 2 * n_out].  With
+   * DMQ_EPI_STORE (a Linear with a handful of rows): k_split may also be 8 or 16, any bit width,
+   * split_partial fp32 [k_split, split_rows, n_out].  split_rows >= every routed row index + 1.
+   * Each workgroup parks its fp32 sums in its plane of split_partial and the last to arrive adds
+   * the planes in a fixed order and runs the epilogue, so the result does not depend on the order
+   * of arrival.  split_counter: int32 [max_items * ceil(n_out / 128)], zero before the launch;
+   * the launch leaves it zero. */
   int k_split;
   int split_rows;
   void* split_partial;
@@ -247,6 +250,11 @@ typedef struct {
    * the launch walks every item as item_tile_rows / (16*tt) row tiles.  Lets one work-item list
    * serve launches of different tile sizes.  Not with k_split. */
   int item_tile_rows;
+  /* n-tiles of 16 output features per wave: 0 or 4 = the normal launch; 1 = the launch of a Linear
+   * with a handful of rows: DMQ_EPI_STORE, tt == 1, ks == 4 (the four waves of a workgroup split K
+   * and the workgroup covers 16 features, so a 4096-feature matrix gives 256 workgroups), any bit
+   * width, not WxFP4, not with k_split or dbg_acc; n_out a multiple of 16. */
+  int nt;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

@@ -149,6 +149,37 @@ def test_unsliced_callables_by_reference_names():
     assert relerr(of8.float().cpu(), _dataflow(packed, x, "wxfp8")) < 2e-2
 
 
+@pytest.mark.parametrize("cls,mode,tol", [("WxA16Linear", "wxa16", 1.5e-3), ("WxA8Linear", "wxa8", 6e-3),
+                                          ("WxFP8Linear", "wxfp8", 2e-2)])
+@pytest.mark.parametrize("bit", [1, 2, 4, 8])
+@pytest.mark.parametrize("rows", [1, 16, 17, 64])
+def test_linears_with_a_handful_of_rows(cls, mode, tol, bit, rows):
+    """The small-batch launches of a Linear: one n-tile per wave with K split over the waves (up
+    to 16 rows), K split over the waves of four n-tiles or shared between workgroups (up to 64);
+    16 groups, so every wave and every workgroup gets several."""
+    import dartmoq_hip
+    n, k = 320, 2048
+    packed = (turboquant.quantize_packed((torch.randn(n, k, generator=torch.Generator().manual_seed(bit)) * 0.02).half(),
+                                         bit, 128, seed=11, uniform_codebook=True)
+              if bit == 8 else _packed(n, k, bit, seed=bit))
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed)
+    if cls != "WxA16Linear":
+        lin = getattr(dartmoq_hip, cls).from_wxa16(lin)
+    x = torch.randn(rows, k, generator=torch.Generator().manual_seed(rows)).half()
+    out = lin(x.cuda())
+    assert torch.equal(out, lin(x.cuda()))                        # same bits on every call
+    out = out.float().cpu()
+    assert out.shape == (rows, n)
+    assert relerr(out, _dataflow(packed, x, mode)) < tol
+    if mode == "wxa16":
+        ref = x.float() @ turboquant.dequantize_packed(packed).T
+        assert max_rel(out, ref) <= 1e-2 and cosine(out, ref) >= 0.9999
+    # a row's result does not depend on the rows batched with it (same launch shape)
+    if rows == 16:
+        alone = lin(x[:5].cuda()).float().cpu()
+        assert torch.equal(alone, out[:5])
+
+
 # ----------------------------------------------------------------------------- 8-bit codebooks
 
 def _packed8(n, k, seed, uniform):

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/dartmoq_hip.h but not exported"
     assert set(declared) == set(_lib.PROTOTYPES), "ctypes prototypes and header disagree"
-    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 11
+    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 12
     assert lib.dmq_status_string(0) == b"ok"
     assert b"bit width" in lib.dmq_status_string(1)
 
@@ -181,8 +181,9 @@ def test_argument_validation_of_later_entry_points():
 
 
 def test_k_sharing_argument_validation():
-    """k_split of the merged GEMM: 2 or 4 workgroups per block, 16-row tiles, SiLU epilogues,
-    groups divisible, scratch present (all rejected before any launch)."""
+    """k_split of the merged GEMM: 2 or 4 workgroups per block (8 and 16 with the plain-store
+    epilogue only), 16-row tiles, never the scatter epilogue, groups divisible, scratch present
+    (all rejected before any launch)."""
     from dartmoq_hip import _lib
     lib = _lib.load()
     buf = ctypes.create_string_buffer(64)
@@ -202,7 +203,19 @@ def test_k_sharing_argument_validation():
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 3           # split_rows missing
     a.split_rows, a.tt = 16, 2
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # 16-row tiles only
-    a.tt, a.epi = 1, _lib.EPI_STORE
-    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # SiLU epilogues only
+    a.tt, a.epi = 1, _lib.EPI_SCATTER
+    a.row_weight = a.row_slot = p
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # not the scatter epilogue
+    a.epi, a.k_split = _lib.EPI_SILU, 8
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # 8 only with the plain store
+    a.epi = _lib.EPI_STORE
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 2           # 4 groups, 8 workgroups
+    a.k_split, a.nt = 0, 1
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # one n-tile per wave: ks = 4 only
+    a.ks, a.tt = 4, 2
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # ... and 16-row tiles
+    a.tt, a.nt = 1, 3
+    assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5           # 0, 1 or 4
+    a.nt, a.ks = 0, 0
     a.epi, a.k_split, a.groups, a.act_row_bytes = _lib.EPI_SILU, 4, 6, 2048
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 2           # 6 groups, 4 workgroups

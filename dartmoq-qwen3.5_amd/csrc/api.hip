@@ -427,6 +427,126 @@ int dmq_quantize_weights(const void* w_f16, long w_row_stride, const void* rot_f
                                      (uint8_t*)indices_packed, (__half*)norms_f16, (hipStream_t)stream);
 }
 
+// ------------------------------------------------------------------------------ Linear forward
+static inline size_t align_up(size_t v);
+
+struct LinearWs {
+  int *counter, *info, *n_items, *items;
+  uint8_t *codes, *scale;
+  float* partial;
+  int tiles, counters, k_split;
+  long code_row_bytes;
+  int scale_stride;
+  size_t bytes;
+};
+
+// Launch shape of a stand-alone Linear by batch size: up to 16 rows one n-tile per wave with K split
+// over the waves; up to 64 rows K split over the waves of four n-tiles (8-bit weights: K shared by
+// workgroups instead); beyond, 32- or 64-row tiles.
+struct LinearShape { int tt, ks, nt, k_split, rot_tt; };
+static LinearShape linear_shape(const dmq_linear_desc* L, int rows) {
+  const int groups = L->in_features / DMQ_GS;
+  LinearShape s{1, 0, 0, 0, rows >= 1024 ? 4 : 1};
+  if (rows <= 16) { s.ks = 4; s.nt = 1; }
+  else if (rows <= 64) {
+    if (L->bit != 8) s.ks = 4;
+    else s.k_split = groups % 4 == 0 ? 4 : (groups % 2 == 0 ? 2 : 0);
+  } else s.tt = rows <= 160 ? 2 : 4;
+  return s;
+}
+
+static LinearWs carve_linear(const dmq_linear_desc* L, int rows, uint8_t* base) {
+  LinearWs w{};
+  const LinearShape sh = linear_shape(L, rows);
+  const int groups = L->in_features / DMQ_GS;
+  w.tiles = (rows + 16 * sh.tt - 1) / (16 * sh.tt);
+  w.k_split = sh.k_split;
+  w.counters = (w.tiles + 1) * ((L->out_features + 127) / 128);
+  w.code_row_bytes = (long)groups * act_bytes_per_group(L->mode);
+  w.scale_stride = groups;
+  size_t off = 0;
+  auto take = [&](size_t n) { uint8_t* p = base ? base + off : nullptr; off += align_up(n); return p; };
+  w.counter = (int*)take((size_t)w.counters * 4);
+  w.info = (int*)take(16);
+  w.n_items = (int*)take(16);
+  w.items = (int*)take((size_t)(w.tiles + 1) * DMQ_ITEM_WORDS * 4);
+  w.codes = take((size_t)rows * w.code_row_bytes);
+  w.scale = take(L->mode == DMQ_MODE_A16 ? 0 : (size_t)rows * groups * 2);
+  w.partial = (float*)take(sh.k_split > 1 ? (size_t)sh.k_split * rows * L->out_features * 4 : 0);
+  w.bytes = off;
+  return w;
+}
+
+static int linear_desc_ok(const dmq_linear_desc* L) {
+  if (!L) return DMQ_ERR_NULL;
+  if (L->mode != DMQ_MODE_A16 && L->mode != DMQ_MODE_A8 && L->mode != DMQ_MODE_FP8) return DMQ_ERR_MODE;
+  if (!dmq_valid_bit_wide(L->bit)) return DMQ_ERR_BIT;
+  if (L->in_features <= 0 || L->out_features <= 0) return DMQ_ERR_SHAPE;
+  if (L->in_features % DMQ_GS || L->out_features % 64) return DMQ_ERR_ALIGN;
+  return DMQ_OK;
+}
+
+size_t dmq_linear_workspace_bytes(const dmq_linear_desc* L, int max_rows) {
+  if (linear_desc_ok(L) != DMQ_OK || max_rows <= 0) return 0;
+  // the carve of any batch up to max_rows fits the largest of the shapes
+  size_t best = 0;
+  const int probes[] = {max_rows, max_rows < 64 ? max_rows : 64, max_rows < 16 ? max_rows : 16};
+  for (int r : probes) {
+    const size_t b = carve_linear(L, r, nullptr).bytes;
+    if (b > best) best = b;
+  }
+  return best;
+}
+
+int dmq_linear_forward(const dmq_linear_desc* L, const void* x_f16, long x_stride, int rows,
+                       void* out_f16, long out_stride, void* workspace, size_t workspace_bytes,
+                       void* stream) {
+  int rc = linear_desc_ok(L);
+  if (rc) return rc;
+  if (rows <= 0) return DMQ_OK;
+  if (!x_f16 || !out_f16 || !workspace) return DMQ_ERR_NULL;
+  if (!L->indices_gf || !L->norms_gf || !L->rot) return DMQ_ERR_NULL;
+  if (!L->lut && !(L->mode == DMQ_MODE_A8 && L->bit == 8)) return DMQ_ERR_NULL;
+  if (x_stride < L->in_features || out_stride < L->out_features) return DMQ_ERR_SHAPE;
+  if (x_stride % 8 || out_stride % 4) return DMQ_ERR_ALIGN;
+  if ((uintptr_t)workspace % 256) return DMQ_ERR_ALIGN;
+  const LinearWs w = carve_linear(L, rows, (uint8_t*)workspace);
+  if (w.bytes > workspace_bytes) return DMQ_ERR_LIMIT;
+  const LinearShape sh = linear_shape(L, rows);
+  const int groups = L->in_features / DMQ_GS;
+
+  // launch 1: rotation (+ quantization) of the rows; its first workgroup also writes the work
+  // items of launch 2 and clears the arrival counters
+  RotParams p{};
+  p.pool[0] = RotPool{(const __half*)L->rot, w.codes, w.code_row_bytes, w.scale, w.scale_stride, nullptr,
+                      L->extra_scale, L->mode, 1, 0};
+  p.x = (const __half*)x_f16; p.x_stride = x_stride; p.row_index = nullptr;
+  p.rows = rows; p.groups = groups;
+  p.n_hoisted = 1; p.hoisted_pool[0] = 0;
+  p.items = nullptr; p.n_items = nullptr; p.tile_rows = 16 * sh.rot_tt; p.scale_fp32 = 0;
+  p.prep = LinearPrep{w.info, w.n_items, w.items, w.tiles, rows, L->out_features, w.counter,
+                      sh.k_split > 1 ? w.counters : 0};
+  rc = dmq_rotate_dispatch(L->mode, p, 0, sh.rot_tt, (hipStream_t)stream);
+  if (rc) return rc;
+
+  // launch 2: dequant GEMM, plain store
+  dmq_gemm_args a{};
+  a.mode = L->mode; a.epi = DMQ_EPI_STORE; a.tt = sh.tt; a.ks = sh.ks; a.nt = sh.nt; a.n_pools = 1;
+  dmq_gemm_pool& q = a.pool[0];
+  q.w = L->indices_gf; q.norms = L->norms_gf; q.lut = L->lut; q.expert_info = w.info;
+  q.act = w.codes; q.act_scale = L->mode == DMQ_MODE_A16 ? nullptr : w.scale; q.row_index = nullptr;
+  q.n_total = L->out_features; q.bit = L->bit; q.mode = L->mode; q.w_scale_byte = 127;
+  a.act_row_bytes = w.code_row_bytes; a.act_scale_stride = w.scale_stride;
+  a.groups = groups; a.n_out = L->out_features; a.half_width = 0; a.slice_is_groups = 0;
+  a.items = w.items; a.n_items = w.n_items; a.max_items = w.tiles;
+  a.out = out_f16; a.out_stride = out_stride;
+  if (sh.k_split > 1) {
+    a.k_split = sh.k_split; a.split_rows = rows;
+    a.split_partial = w.partial; a.split_counter = w.counter;
+  }
+  return dmq_matmul_merged_gf(&a, stream);
+}
+
 int dmq_rms_norm(const void* x, int x_bf16, const void* weight, int weight_fp32, long rows, int n,
                  long x_row_stride, long out_row_stride, float eps, void* out, void* stream) {
   if (rows <= 0) return DMQ_OK;

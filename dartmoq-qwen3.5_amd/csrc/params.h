@@ -18,6 +18,17 @@ struct RotPool {
   int rot_use_slice;       // tiled: 1 = matrices start at the expert's slice_start (down), 0 = at 0
 };
 
+// Side job of a rotation launch in front of a stand-alone Linear GEMM: workgroup 0 also writes the
+// work-item list of the GEMM (row tiles of one matrix) and clears its arrival counters.
+struct LinearPrep {
+  int* info;               // [4] expert_info of the one matrix; NULL = no side job
+  int* n_items;            // [1]
+  int* items;              // [tiles, DMQ_ITEM_WORDS]
+  int tiles, rows, n_out;
+  int* zero;               // optional int32 words to clear
+  int zero_count;
+};
+
 struct RotParams {
   RotPool pool[DMQ_MAX_POOLS];
   const __half* x;         // [*, x_stride] fp16
@@ -35,6 +46,7 @@ struct RotParams {
   int tile_rows;           // rows per work item (multiple of 16*TT)
   int scale_fp32;
   int items_prefix;        // 1: only the first n_items[1] items belong to tiled pools
+  LinearPrep prep;
 };
 
 struct QuantParams {

@@ -265,6 +265,20 @@ template <int MODE, int TT>
 __global__ __launch_bounds__(256)
 void dmq_rotate_kernel(RotParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
+  if (p.prep.info && blockIdx.x == 0) {
+    // the records dmq_items_from_info_kernel would write for expert_info = [0, rows, 0, n_out]
+    const LinearPrep& lp = p.prep;
+    for (int i = threadIdx.x; i < lp.tiles; i += 256) {
+      int4_t* it = (int4_t*)(lp.items + (long)DMQ_ITEM_WORDS * i);
+      it[0] = (int4_t){0, 0, i, 0};
+      it[1] = (int4_t){lp.rows, 0, 0, 0};
+    }
+    for (int i = threadIdx.x; i < lp.zero_count; i += 256) lp.zero[i] = 0;
+    if (threadIdx.x == 0) {
+      lp.n_items[0] = lp.tiles;
+      *(int4_t*)lp.info = (int4_t){0, lp.rows, 0, lp.n_out};
+    }
+  }
   dmq_rotate_wg<MODE, TT>(p, blockIdx.x, mat);
 }
 

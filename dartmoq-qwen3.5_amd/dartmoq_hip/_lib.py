@@ -64,6 +64,14 @@ class PoolDesc(Structure):
     ]
 
 
+class LinearDesc(Structure):
+    _fields_ = [
+        ("mode", c_int), ("bit", c_int), ("in_features", c_int), ("out_features", c_int),
+        ("indices_gf", c_void_p), ("norms_gf", c_void_p), ("lut", c_void_p), ("rot", c_void_p),
+        ("extra_scale", c_float),
+    ]
+
+
 class LayerDesc(Structure):
     _fields_ = [
         ("hidden", c_int), ("inter", c_int), ("experts", c_int), ("top_k", c_int), ("pools", c_int),
@@ -112,6 +120,9 @@ PROTOTYPES = {
                                      c_void_p, c_void_p]),
     "dmq_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_long, c_long, c_float,
                              c_void_p, c_void_p]),
+    "dmq_linear_workspace_bytes": (c_size_t, [POINTER(LinearDesc), c_int]),
+    "dmq_linear_forward": (c_int, [POINTER(LinearDesc), c_void_p, c_long, c_int, c_void_p, c_long,
+                                   c_void_p, c_size_t, c_void_p]),
     "dmq_moe_workspace_bytes": (c_size_t, [POINTER(LayerDesc), c_int]),
     "dmq_moe_ffn_forward": (c_int, [POINTER(LayerDesc), c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                     c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_void_p]),

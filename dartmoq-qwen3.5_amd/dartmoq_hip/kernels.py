@@ -81,9 +81,13 @@ def _gemm(mode, bit, x_codes, x_scale, w_gf, norms, lut, info, *, groups, n_out,
     if cfg is not None:                       # (BLOCK_B, ...) of the reference: rows per tile
         tt = max(1, min(4, int(cfg[0]) // 16))
         tt = 4 if tt >= 4 else (2 if tt >= 2 else 1)
+    small = {}
+    if tt is None and rows_total <= 16 and info.shape[0] == 1 and mode != MODE_FP4 and n_out % 16 == 0:
+        # one matrix, a handful of rows: a workgroup per 16 features, its four waves splitting K
+        tt, small = 1, {"ks": 4, "nt": 1}
     return ops.matmul_merged(mode, bit, EPI_STORE, x_codes, x_scale, w_gf, norms, lut, info,
                              groups=groups, n_out=n_out, slice_is_groups=slice_is_groups,
-                             rows_total=rows_total, w_scale_byte=w_scale_byte, tt=tt)
+                             rows_total=rows_total, w_scale_byte=w_scale_byte, tt=tt, **small)
 
 
 # ----------------------------------------------------------------------------- norm

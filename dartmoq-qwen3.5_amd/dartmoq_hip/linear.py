@@ -6,8 +6,9 @@ quantization/wxa8/linear.py:79-159 (fused rotate + int8 quantize, integer GEMM) 
 quantization/wxfp8/linear.py:37-100 (e4m3 activations and look-up table).  These are the Linears
 of the shared expert of the MoE layer.  Like the reference's WxA8Linear._ensure_gf the module
 converts the checkpoint layout to group-first once (norms divided by sqrt(128)) and keeps the
-rotation matrices and the per-mode look-up table resident; a forward is two launches (rotate
-(+quantize), dequant GEMM) on the current stream, the GEMM tiled by batch size (_tiling).
+rotation matrices and the per-mode look-up table resident; a forward is one call of
+dmq_linear_forward: two launches (rotate (+quantize), dequant GEMM) on the current stream, the
+GEMM shaped by batch size.
 
 Bit widths 1, 2, 4 and 8 are built, all through a codebook look-up.  8-bit weights run on the int8
 path only with a uniform codebook (then the table is the identity w = idx - 128 and the step rides
@@ -18,14 +19,33 @@ from __future__ import annotations
 
 import torch
 
+import ctypes
+
 from . import hostprep, ops
-from ._lib import EPI_STORE, MODE_A16, MODE_A8, MODE_FP8
+from ._lib import EPI_STORE, MODE_A16, MODE_A8, MODE_FP8, LinearDesc, check, load
 
 GROUP_SIZE = ops.GROUP_SIZE
 SPLIT_MAX_ROWS = 64          # batches up to this size split K between waves or workgroups
 
 
 _SPLIT_WS: dict = {}
+_WORKSPACE: dict = {}
+
+
+def _workspace(device, desc, rows: int) -> torch.Tensor:
+    """Scratch of dmq_linear_forward, shared by the Linears of a (device, stream): launches on one
+    stream run one after the other.  Grows to the largest request."""
+    dev = torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(dev).cuda_stream)
+    need = load().dmq_linear_workspace_bytes(ctypes.byref(desc), rows)
+    if need == 0:
+        raise ValueError("dmq_linear_workspace_bytes refused the Linear descriptor")
+    ws = _WORKSPACE.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        _WORKSPACE[key] = ws
+    return ws
 
 
 def _split_workspace(device, k: int, rows: int, n_out: int, items: int):
@@ -84,6 +104,7 @@ class WxA16Linear:
         self._ctx: dict[int, tuple] = {}
         self._info: dict[int, torch.Tensor] = {}
         self._tile_cache: dict = {}
+        self._desc: dict = {}
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -173,8 +194,48 @@ class WxA16Linear:
             self._tile_cache[key] = t
         return t
 
+    def _descriptor(self) -> LinearDesc:
+        d = self._desc.get(self.MODE)
+        if d is None:
+            lut, extra = self._mode_ctx()
+            d = LinearDesc()
+            d.mode, d.bit = self.MODE, self.bit_width
+            d.in_features, d.out_features = self.in_features, self.out_features
+            d.indices_gf, d.norms_gf = self.indices_gf.data_ptr(), self.norms_gf.data_ptr()
+            d.lut = lut.data_ptr() if lut is not None else None
+            d.rot, d.extra_scale = self.rot.data_ptr(), float(extra)
+            self._desc[self.MODE] = d
+        return d
+
     @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """One call of dmq_linear_forward: the rotation (+ quantization) launch and the GEMM launch."""
+        if not x.is_cuda:
+            raise RuntimeError("dartmoq_hip layers run on the GPU only (no CPU fallback)")
+        shape = x.shape
+        if shape[-1] != self.in_features:
+            raise ValueError(f"expected {self.in_features} input features, got {shape[-1]}")
+        x2 = x.reshape(-1, self.in_features)
+        src = x2 if x2.dtype == torch.float16 else x2.half()
+        if src.stride(1) != 1 or src.stride(0) % 8:
+            src = src.contiguous()
+        rows = src.shape[0]
+        out = torch.empty((rows, self.out_features), dtype=torch.float16, device=x.device)
+        if rows:
+            desc = self._descriptor()
+            ws = _workspace(self.device, desc, rows)
+            check(load().dmq_linear_forward(ctypes.byref(desc), src.data_ptr(), src.stride(0), rows,
+                                            out.data_ptr(), self.out_features, ws.data_ptr(), ws.numel(),
+                                            ops._stream(x.device)), "linear_forward")
+        if self.bias is not None:
+            out = out + self.bias.to(out.dtype)
+        return out.reshape(*shape[:-1], self.out_features).to(x.dtype)
+
+    @torch.no_grad()
+    def forward_by_pieces(self, x: torch.Tensor) -> torch.Tensor:
+        """The same two launches issued through the generic entry points (dmq_rotate, then
+        dmq_matmul_merged_gf over a one-matrix work list): what forward does inside one C call,
+        kept as its cross-check."""
         if not x.is_cuda:
             raise RuntimeError("dartmoq_hip layers run on the GPU only (no CPU fallback)")
         shape = x.shape

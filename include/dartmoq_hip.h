@@ -274,6 +274,38 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* args, void* stream);
 int dmq_combine_slots(const void* slots_f16, int k, const void* add_f16, long tokens, int hidden,
                       void* out_f16, void* stream);
 
+/* A quantized Linear (the shared-expert and attention Linears of a checkpoint): out = x @ W^T with W
+ * in the packed format.  Replaces WxA16Linear.forward (quantization/wxa16/linear.py:224-260, which
+ * calls triton_fused_matmul_grouped, triton_kernels.py:600-684), WxA8Linear.forward
+ * (quantization/wxa8/linear.py:130-159: rotate_quantize_fused + wxa8_matmul_grouped_gf) and
+ * WxFP8Linear.forward (quantization/wxfp8/linear.py): two launches, the rotation (+ quantization)
+ * of the rows and the dequant GEMM with its launch shape chosen by batch size.  The bias, if any,
+ * is the caller's add. */
+typedef struct {
+  int mode;                 /* DMQ_MODE_A16 / _A8 / _FP8 */
+  int bit;                  /* 1 / 2 / 4 / 8 */
+  int in_features;          /* multiple of 128 */
+  int out_features;         /* multiple of 64 */
+  const void* indices_gf;   /* u8 [G, out_features, 128*bit/8]: group-first packed indices */
+  const void* norms_gf;     /* fp16 [G, out_features], already divided by sqrt(128) */
+  const void* lut;          /* table of the mode: fp16 / int8 / e4m3 [2^bit]; NULL = identity
+                               (int8 path, 8-bit uniform codebook: w = idx - 128) */
+  const void* rot;          /* fp16 [G, 128, 128] rotation matrices of the input groups */
+  float extra_scale;        /* factor folded into the activation scales (int8 codebook step,
+                               e4m3 table scale); 1 for DMQ_MODE_A16 */
+} dmq_linear_desc;
+
+/* Bytes of scratch dmq_linear_forward needs for batches of up to max_rows rows (0: bad descriptor). */
+size_t dmq_linear_workspace_bytes(const dmq_linear_desc* linear, int max_rows);
+
+/* x fp16 [rows, x_stride >= in_features] -> out fp16 [rows, out_stride >= out_features] (strides in
+ * elements, x_stride % 8 == 0, out_stride % 4 == 0).  workspace: device memory, 256-byte aligned,
+ * at least dmq_linear_workspace_bytes(linear, rows) bytes, any contents; calls that overlap on the
+ * GPU need separate workspaces.  Allocates nothing, never synchronizes. */
+int dmq_linear_forward(const dmq_linear_desc* linear, const void* x_f16, long x_stride, int rows,
+                       void* out_f16, long out_stride, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
 /* rms_norm of turboquant_utils/norm_kernels.py:79-117, :183-209 (Qwen3_5MoeRMSNorm.forward: the
  * norm in front of the MoE block): out = x * rsqrt(mean(x^2) + eps) * (1 + weight) in fp32, one
  * rounding to the activation type.  x / out fp16 (x_bf16 == 0) or bf16 [rows, n] with the given

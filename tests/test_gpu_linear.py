@@ -168,6 +168,7 @@ def test_linears_with_a_handful_of_rows(cls, mode, tol, bit, rows):
     x = torch.randn(rows, k, generator=torch.Generator().manual_seed(rows)).half()
     out = lin(x.cuda())
     assert torch.equal(out, lin(x.cuda()))                        # same bits on every call
+    assert torch.equal(out, lin.forward_by_pieces(x.cuda()))      # the C entry = its two launches
     out = out.float().cpu()
     assert out.shape == (rows, n)
     assert relerr(out, _dataflow(packed, x, mode)) < tol
@@ -178,6 +179,23 @@ def test_linears_with_a_handful_of_rows(cls, mode, tol, bit, rows):
     if rows == 16:
         alone = lin(x[:5].cuda()).float().cpu()
         assert torch.equal(alone, out[:5])
+
+
+@pytest.mark.parametrize("cls", ["WxA16Linear", "WxA8Linear", "WxFP8Linear"])
+@pytest.mark.parametrize("rows", [65, 161, 1100])
+def test_linear_entry_point_equals_its_pieces(cls, rows):
+    """dmq_linear_forward against dmq_rotate + dmq_matmul_merged_gf issued one by one, on the
+    32- and 64-row tilings of bigger batches, with an input whose rows are strided."""
+    import dartmoq_hip
+    packed = _packed(192, 384, 4, seed=3)
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed)
+    if cls != "WxA16Linear":
+        lin = getattr(dartmoq_hip, cls).from_wxa16(lin)
+    wide = torch.randn(rows, 512, generator=torch.Generator().manual_seed(rows)).half().cuda()
+    x = wide[:, :384]                                             # row stride 512
+    out = lin(x)
+    assert torch.equal(out, lin.forward_by_pieces(x))
+    assert torch.equal(out, lin(x.contiguous()))
 
 
 # ----------------------------------------------------------------------------- 8-bit codebooks

@@ -180,6 +180,42 @@ def test_argument_validation_of_later_entry_points():
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 5                       # unknown epilogue
 
 
+def test_linear_entry_point_validation():
+    """dmq_linear_forward / dmq_linear_workspace_bytes reject bad descriptors before any launch."""
+    from dartmoq_hip import _lib
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096 + 256)
+    base = ctypes.addressof(buf)
+    p = ctypes.c_void_p((base + 255) // 256 * 256)
+    d = _lib.LinearDesc()
+    d.mode, d.bit, d.in_features, d.out_features, d.extra_scale = 0, 4, 256, 128, 1.0
+    assert lib.dmq_linear_workspace_bytes(ctypes.byref(d), 0) == 0
+    small = lib.dmq_linear_workspace_bytes(ctypes.byref(d), 16)
+    big = lib.dmq_linear_workspace_bytes(ctypes.byref(d), 4096)
+    assert 0 < small < big and big >= 4096 * 256 * 2              # the rotated fp16 rows at least
+    d8 = _lib.LinearDesc()
+    d8.mode, d8.bit, d8.in_features, d8.out_features = 1, 8, 512, 128
+    # 17 .. 64 rows of 8-bit weights add the fp32 planes of the shared K range
+    assert lib.dmq_linear_workspace_bytes(ctypes.byref(d8), 64) >= 64 * 512 + 4 * 64 * 128 * 4
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, p, 4096, None) == 6   # no weights
+    d.indices_gf = d.norms_gf = d.lut = d.rot = p
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 0, p, 128, p, 4096, None) == 0   # no rows
+    assert lib.dmq_linear_forward(ctypes.byref(d), None, 256, 4, p, 128, p, 4096, None) == 6
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 128, 4, p, 128, p, 4096, None) == 3   # x_stride < K
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 260, 4, p, 128, p, 4096, None) == 2   # x_stride % 8
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, p, 64, None) == 8     # workspace too small
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, ctypes.c_void_p(p.value + 4), 4096,
+                                  None) == 2                                                # unaligned
+    d.lut = None
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, p, 4096, None) == 6   # table missing
+    d.lut, d.mode = p, 3
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, p, 4096, None) == 5   # no WxFP4 Linear
+    d.mode, d.bit = 0, 3
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, p, 4096, None) == 1
+    d.bit, d.out_features = 4, 100
+    assert lib.dmq_linear_forward(ctypes.byref(d), p, 256, 4, p, 128, p, 4096, None) == 2
+
+
 def test_k_sharing_argument_validation():
     """k_split of the merged GEMM: 2 or 4 workgroups per block (8 and 16 with the plain-store
     epilogue only), 16-row tiles, never the scatter epilogue, groups divisible, scratch present

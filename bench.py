@@ -180,6 +180,49 @@ def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf, shared_cpu=Non
                       f"fp32 oracle (reference_forward), {torch.get_num_threads()} threads"}
 
 
+def bench_linear(spec, steps, warmup, seed):
+    """Side leg (--linear "bit,mode,rows[,out_features,in_features]"): one quantized Linear
+    (synthetic packed indices, the Lloyd-Max codebook of the width or the uniform 8-bit grid)
+    through dmq_linear_forward; wall time per call and, from events around the timed loop, GPU time."""
+    import torch
+    import dartmoq_hip
+    from dartmoq_hip import hostprep
+    f = spec.split(",")
+    bit, mode, rows = int(f[0]), f[1], int(f[2])
+    n, k = (int(f[3]), int(f[4])) if len(f) >= 5 else (4096, 4096)
+    g = torch.Generator().manual_seed(seed)
+    if bit == 8:
+        cb = ((torch.arange(256, dtype=torch.float32) - 128) * (3.5 / 128)).half()
+    else:
+        cb = hostprep.get_codebook(bit)[0].half()
+    groups = k // 128
+    idx = torch.randint(0, 256, (n, groups * 128 * bit // 8), dtype=torch.uint8, generator=g)
+    norms = (torch.rand(n, groups, generator=g) * 0.02 + 0.01).half()
+    lin = dartmoq_hip.WxA16Linear(k, n, bit, 128, idx, cb, norms, seed=seed)
+    cls = {"wxa16": None, "wxa8": dartmoq_hip.WxA8Linear, "wxfp8": dartmoq_hip.WxFP8Linear}[mode]
+    if cls is not None:
+        lin = cls.from_wxa16(lin)
+    x = torch.randn(rows, k, generator=g).half().cuda()
+    for _ in range(warmup):
+        lin(x)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        lin(x)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    packed = n * k * bit // 8 + n * groups * 2
+    print(json.dumps({"metric": "linear_forward_us", "value": wall * 1e6, "unit": "us",
+                      "higher_is_better": False, "steps": steps, "warmup": warmup, "n_gpus": 1,
+                      "gpu_us_between_events": e0.elapsed_time(e1) * 1e3 / steps, "dtype": "f16",
+                      "data": "synthetic",
+                      "config": {"workload": f"one {mode} Linear, {bit}-bit weights [{n}, {k}], {rows} rows",
+                                 "packed_weight_bytes": packed}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -196,6 +239,9 @@ def main():
                     help="also launch dmq_finalize_kernel on 64 Mi fp32 elements (256 MiB read, "
                          "128 MiB written): the known-size kernel that calibrates FETCH_SIZE / "
                          "WRITE_SIZE counter runs")
+    ap.add_argument("--linear", type=str, default="",
+                    help='side leg: time one quantized Linear instead of the layer, '
+                         '"bit,mode,rows[,out_features,in_features]" (mode wxa16 / wxa8 / wxfp8)')
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -208,6 +254,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(3)
+    if args.linear:
+        bench_linear(args.linear, args.steps, args.warmup, args.seed)
+        return
     spec = synthetic.CONFIGS[args.config]
     expert_bit = synthetic.assign_bits(spec["experts"], spec["fractions"], args.seed)
     pools = synthetic.build_pools(spec["hidden"], spec["inter"], spec["experts"], expert_bit,

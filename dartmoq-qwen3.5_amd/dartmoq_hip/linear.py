@@ -169,16 +169,26 @@ class WxA16Linear:
         16 features: 35 -> 10 us for an 8-bit 4096 x 4096 matrix, 15 -> 10 us for a 4-bit one).  Up
         to 64 rows the waves still split K over four n-tiles each, except for 8-bit weights, whose
         K range is shared between four workgroups instead (fp32 partial sums, added in a fixed
-        order by the last workgroup to arrive: 35 -> 21 us)."""
+        order by the last workgroup to arrive: 35 -> 21 us).  Bigger batches: see below.  The same
+        policy as linear_shape() of the library, which forward() runs."""
         if rows <= 16:
             return {"tt": 1, "ks": 4, "nt": 1}
-        if rows > SPLIT_MAX_ROWS:
-            return {}
-        if self.bit_width != 8:
-            return {"tt": 1, "ks": 4}
-        k = 4 if self.n_groups % 4 == 0 else (2 if self.n_groups % 2 == 0 else 1)
-        if k == 1:
-            return {"tt": 1}
+        k = 0
+        if rows <= SPLIT_MAX_ROWS:
+            if self.bit_width != 8:
+                return {"tt": 1, "ks": 4}
+            tt = 1
+            k = 4 if self.n_groups % 4 == 0 else (2 if self.n_groups % 2 == 0 else 0)
+        else:
+            # the largest row tile that still gives every CU a workgroup (8-bit: at most 32 rows);
+            # 16-row tiles on less than half the CUs: two workgroups share K
+            blocks = (self.out_features + 255) // 256
+            wgs = lambda t: ((rows + 16 * t - 1) // (16 * t)) * blocks
+            tt = next((t for t in ((2,) if self.bit_width == 8 else (4, 2)) if wgs(t) >= 256), 1)
+            if tt == 1 and wgs(1) <= 128 and self.n_groups % 2 == 0:
+                k = 2
+        if k <= 1:
+            return {"tt": tt}
         # counters: one per (work item, feature block); the item list has rows // 16 + 1 slots
         partial, counter = _split_workspace(self.device, k, rows, self.out_features, rows // 16 + 1)
         return {"tt": 1, "ks": 1, "k_split": k, "split_ws": (partial, counter)}

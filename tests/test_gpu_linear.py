@@ -181,21 +181,35 @@ def test_linears_with_a_handful_of_rows(cls, mode, tol, bit, rows):
         assert torch.equal(alone, out[:5])
 
 
-@pytest.mark.parametrize("cls", ["WxA16Linear", "WxA8Linear", "WxFP8Linear"])
-@pytest.mark.parametrize("rows", [65, 161, 1100])
-def test_linear_entry_point_equals_its_pieces(cls, rows):
-    """dmq_linear_forward against dmq_rotate + dmq_matmul_merged_gf issued one by one, on the
-    32- and 64-row tilings of bigger batches, with an input whose rows are strided."""
+_BIG = {}
+
+
+def _big_packed(bit):
+    if bit not in _BIG:
+        _BIG[bit] = _packed8(1024, 512, seed=3, uniform=True) if bit == 8 else _packed(1024, 512, bit, seed=3)
+    return _BIG[bit]
+
+
+@pytest.mark.parametrize("cls,mode,tol", [("WxA16Linear", "wxa16", 1.5e-3), ("WxA8Linear", "wxa8", 6e-3),
+                                          ("WxFP8Linear", "wxfp8", 2e-2)])
+@pytest.mark.parametrize("bit", [4, 8])
+@pytest.mark.parametrize("rows", [65, 1100, 2100, 4200])
+def test_linear_entry_point_equals_its_pieces(cls, mode, tol, bit, rows):
+    """dmq_linear_forward against dmq_rotate + dmq_matmul_merged_gf issued one by one, over the
+    launch shapes of bigger batches (1024 features = 4 blocks: 16-row tiles with K shared by two
+    workgroups at 65 and 1100 rows, 32-row tiles at 2100, 64-row tiles at 4200 unless the weights
+    are 8-bit), with an input whose rows are strided; and against the oracle's dataflow."""
     import dartmoq_hip
-    packed = _packed(192, 384, 4, seed=3)
+    packed = _big_packed(bit)
     lin = dartmoq_hip.WxA16Linear.from_packed(packed)
     if cls != "WxA16Linear":
         lin = getattr(dartmoq_hip, cls).from_wxa16(lin)
-    wide = torch.randn(rows, 512, generator=torch.Generator().manual_seed(rows)).half().cuda()
-    x = wide[:, :384]                                             # row stride 512
+    wide = torch.randn(rows, 640, generator=torch.Generator().manual_seed(rows)).half()
+    x = wide.cuda()[:, :512]                                      # row stride 640
     out = lin(x)
     assert torch.equal(out, lin.forward_by_pieces(x))
     assert torch.equal(out, lin(x.contiguous()))
+    assert relerr(out.float().cpu(), _dataflow(packed, wide[:, :512], mode)) < tol
 
 
 # ----------------------------------------------------------------------------- 8-bit codebooks
@@ -253,7 +267,9 @@ def test_wxa8_linear_8bit_identity_codebook():
     x_i8, x_s = K.rotate_quantize_fused(x.cuda(), rot, 128, 4, extra_scale=step)
     dummy = torch.zeros(256, dtype=torch.int8, device="cuda")
     o = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, dummy, norms_pre, 128, 4, 8, identity_cb=True)
-    assert torch.equal(o, lin(x.cuda()))
+    # (the class shares K between two workgroups at this size, the callable does not: the fp32
+    # group sums meet in another order, so the fp16 results agree to rounding, not bit for bit)
+    assert relerr(o.float().cpu(), out) < 5e-4
     # ... and the table-free kernel gives the bits of the look-up kernel fed the identity table
     table = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8).cuda()
     o_tab = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, table, norms_pre, 128, 4, 8, identity_cb=False)

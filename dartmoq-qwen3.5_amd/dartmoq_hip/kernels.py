@@ -85,6 +85,11 @@ def _gemm(mode, bit, x_codes, x_scale, w_gf, norms, lut, info, *, groups, n_out,
     if tt is None and rows_total <= 16 and info.shape[0] == 1 and mode != MODE_FP4 and n_out % 16 == 0:
         # one matrix, a handful of rows: a workgroup per 16 features, its four waves splitting K
         tt, small = 1, {"ks": 4, "nt": 1}
+    elif tt is None and rows_total > 64 and info.shape[0] == 1:
+        # one matrix: the largest row tile that still gives every CU a workgroup (8-bit: 32 rows)
+        blocks = (n_out + 255) // 256
+        tt = next((t for t in ((2,) if bit == 8 else (4, 2))
+                   if ((rows_total + 16 * t - 1) // (16 * t)) * blocks >= 256), 1)
     return ops.matmul_merged(mode, bit, EPI_STORE, x_codes, x_scale, w_gf, norms, lut, info,
                              groups=groups, n_out=n_out, slice_is_groups=slice_is_groups,
                              rows_total=rows_total, w_scale_byte=w_scale_byte, tt=tt, **small)

@@ -495,6 +495,38 @@ static int linear_desc_ok(const dmq_linear_desc* L) {
   return DMQ_OK;
 }
 
+int dmq_linear_gemm_i8(const void* x_i8, long x_row_bytes, const void* x_scale_f16, int scale_stride,
+                       const void* indices_gf, const void* norms_gf, int rows, int in_features,
+                       int out_features, void* out_f16, long out_stride, void* stream) {
+  if (rows <= 0) return DMQ_OK;
+  if (!x_i8 || !x_scale_f16 || !indices_gf || !norms_gf || !out_f16) return DMQ_ERR_NULL;
+  if (in_features <= 0 || out_features <= 0) return DMQ_ERR_SHAPE;
+  if (in_features % DMQ_GS || out_features % 4 || x_row_bytes % 16 || out_stride % 4) return DMQ_ERR_ALIGN;
+  const int groups = in_features / DMQ_GS;
+  if (x_row_bytes < in_features || scale_stride < groups || out_stride < out_features) return DMQ_ERR_SHAPE;
+  const LinearI8Params p{(const uint8_t*)x_i8, x_row_bytes, (const _Float16*)x_scale_f16, scale_stride,
+                         (const uint8_t*)indices_gf, (const _Float16*)norms_gf, rows, groups,
+                         out_features, (_Float16*)out_f16, out_stride};
+  return dmq_linear_i8_launch(p, (hipStream_t)stream);
+}
+
+// 8-bit weights on a uniform grid, int8 path, enough rows to fill the chip with 128 x 128 tiles:
+// the plain int8 GEMM instead of the look-up kernels.  4096 x 4096, forward time: 2048 rows
+// 146 -> 101 us, 4096 rows 290 -> 193 us; at 1024 rows (256 tiles) the two are equal, below that
+// the 32-row look-up tiles win.
+#ifndef DMQ_LINEAR_I8_MIN_WGS
+#define DMQ_LINEAR_I8_MIN_WGS 384
+#endif
+static bool linear_uses_i8_gemm(const dmq_linear_desc* L, int rows) {
+  if (L->mode != DMQ_MODE_A8 || L->bit != 8 || L->lut) return false;
+  const long wgs = (long)((L->out_features + 127) / 128) * ((rows + 127) / 128);
+  return wgs >= DMQ_LINEAR_I8_MIN_WGS;
+}
+
+int dmq_linear_uses_i8_gemm(const dmq_linear_desc* L, int rows) {
+  return (linear_desc_ok(L) == DMQ_OK && rows > 0 && linear_uses_i8_gemm(L, rows)) ? 1 : 0;
+}
+
 size_t dmq_linear_workspace_bytes(const dmq_linear_desc* L, int max_rows) {
   if (linear_desc_ok(L) != DMQ_OK || max_rows <= 0) return 0;
   // the carve of any batch up to max_rows fits the largest of the shapes
@@ -540,8 +572,14 @@ int dmq_linear_forward(const dmq_linear_desc* L, const void* x_f16, long x_strid
   p.items = nullptr; p.n_items = nullptr; p.tile_rows = 16 * sh.rot_tt; p.scale_fp32 = 0;
   p.prep = LinearPrep{w.info, w.n_items, w.items, w.tiles, rows, L->out_features, w.counter,
                       sh.k_split > 1 ? w.counters : 0};
+  const bool i8_gemm = linear_uses_i8_gemm(L, rows);
+  if (i8_gemm) p.prep = LinearPrep{};
   rc = dmq_rotate_dispatch(L->mode, p, 0, sh.rot_tt, (hipStream_t)stream);
   if (rc) return rc;
+  if (i8_gemm)
+    return dmq_linear_gemm_i8(w.codes, w.code_row_bytes, w.scale, w.scale_stride, L->indices_gf,
+                              L->norms_gf, rows, L->in_features, L->out_features, out_f16, out_stride,
+                              stream);
 
   // launch 2: dequant GEMM, plain store
   dmq_gemm_args a{};

@@ -137,6 +137,20 @@ struct TopkParams;
 int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream,
                         const TopkParams* tp = nullptr, int topk_fp16 = 0);
 int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
+
+// int8 GEMM of a Linear with 8-bit weights on a uniform grid (w = idx - 128), 128 x 128 tiles
+struct LinearI8Params {
+  const uint8_t* x;          // int8 codes [rows, x_row_bytes]
+  long x_row_bytes;
+  const _Float16* x_scale;   // fp16 [rows, scale_stride]
+  int scale_stride;
+  const uint8_t* w;          // u8 [groups, n_out, 128] group-first indices
+  const _Float16* norms;     // fp16 [groups, n_out]
+  int rows, groups, n_out;   // n_out % 4 == 0
+  _Float16* out;             // fp16 [rows, out_stride]
+  long out_stride;
+};
+int dmq_linear_i8_launch(const LinearI8Params& p, hipStream_t stream);
 int dmq_route_topk_launch(const void* logits, int logits_fp16, const int* in_idx, const float* in_w,
                           int tokens, int experts, int k, int renorm, float* out_w, int* out_idx,
                           const SharedGate& sg, hipStream_t stream);

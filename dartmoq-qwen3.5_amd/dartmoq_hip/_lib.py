@@ -121,6 +121,9 @@ PROTOTYPES = {
     "dmq_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_long, c_long, c_float,
                              c_void_p, c_void_p]),
     "dmq_linear_workspace_bytes": (c_size_t, [POINTER(LinearDesc), c_int]),
+    "dmq_linear_uses_i8_gemm": (c_int, [POINTER(LinearDesc), c_int]),
+    "dmq_linear_gemm_i8": (c_int, [c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
+                                   c_int, c_void_p, c_long, c_void_p]),
     "dmq_linear_forward": (c_int, [POINTER(LinearDesc), c_void_p, c_long, c_int, c_void_p, c_long,
                                    c_void_p, c_size_t, c_void_p]),
     "dmq_moe_workspace_bytes": (c_size_t, [POINTER(LayerDesc), c_int]),

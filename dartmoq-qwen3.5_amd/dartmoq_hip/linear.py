@@ -258,6 +258,12 @@ class WxA16Linear:
             return torch.empty(*shape[:-1], self.out_features, dtype=x.dtype, device=x.device)
         lut, extra = self._mode_ctx()
         codes, scale = ops.rotate(self.MODE, src, self.rot, extra_scale=extra, scale_fp32=False)
+        if load().dmq_linear_uses_i8_gemm(ctypes.byref(self._descriptor()), rows):
+            # 8-bit uniform weights, int8 path, a big batch: the plain int8 GEMM
+            out = ops.linear_gemm_i8(codes, scale, self.indices_gf, self.norms_gf)
+            if self.bias is not None:
+                out = out + self.bias.to(out.dtype)
+            return out.reshape(*shape[:-1], self.out_features).to(x.dtype)
         tiling = self._tiling(rows)
         tt = tiling.get("tt") or ops.pick_tt(rows, 1)
         tiling["tt"] = tt

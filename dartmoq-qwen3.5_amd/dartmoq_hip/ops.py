@@ -384,6 +384,23 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt)
 
 
+def linear_gemm_i8(x_i8: torch.Tensor, x_scale: torch.Tensor, indices_gf: torch.Tensor,
+                   norms_gf: torch.Tensor) -> torch.Tensor:
+    """int8 GEMM of a Linear whose 8-bit weights are idx - 128 (uniform codebook): x_i8 [rows, K]
+    int8 with fp16 scales [rows, K/128] (codebook step folded in), indices_gf u8 [G, N, 128],
+    norms_gf fp16 [G, N] pre-scaled -> fp16 [rows, N]."""
+    _need_cuda(x_i8, x_scale, indices_gf, norms_gf)
+    rows, k = x_i8.shape
+    g, n, _ = indices_gf.shape
+    if x_scale.dtype != torch.float16 or norms_gf.dtype != torch.float16:
+        raise TypeError("x_scale and norms_gf must be fp16")
+    out = torch.empty((rows, n), dtype=torch.float16, device=x_i8.device)
+    check(load().dmq_linear_gemm_i8(_ptr(x_i8), x_i8.stride(0), _ptr(x_scale), x_scale.stride(0),
+                                    _ptr(indices_gf), _ptr(norms_gf), rows, k, n, _ptr(out), n,
+                                    _stream(x_i8.device)), "linear_gemm_i8")
+    return out
+
+
 def combine_slots(slots: torch.Tensor, top_k: int, add: torch.Tensor | None = None) -> torch.Tensor:
     """out[t] = fp16(sum_j slots[t*k + j] (+ add[t])), slots fp16 [T*k, H], summed in fp32."""
     _need_cuda(slots)

@@ -295,6 +295,20 @@ typedef struct {
                                e4m3 table scale); 1 for DMQ_MODE_A16 */
 } dmq_linear_desc;
 
+/* The int8 GEMM behind dmq_linear_forward for 8-bit weights on a uniform grid and big batches
+ * (wxa8_matmul_grouped_gf with IDENTITY_CB, triton_kernels_a8.py:769-799: w = idx - 128):
+ * out[r, n] = sum_g x_scale[r, g] * norms_gf[g, n] * sum_k x_i8[r, g, k] * (idx[g, n, k] - 128),
+ * 128 x 128 output tiles, both operands through LDS.  x_i8 [rows, x_row_bytes >= in_features]
+ * (x_row_bytes % 16 == 0), x_scale fp16 [rows, scale_stride] with the codebook step folded in,
+ * indices_gf u8 [G, out_features, 128], norms_gf fp16 [G, out_features] pre-scaled,
+ * out fp16 [rows, out_stride]; out_features % 4 == 0, out_stride % 4 == 0. */
+int dmq_linear_gemm_i8(const void* x_i8, long x_row_bytes, const void* x_scale_f16, int scale_stride,
+                       const void* indices_gf, const void* norms_gf, int rows, int in_features,
+                       int out_features, void* out_f16, long out_stride, void* stream);
+
+/* 1 when dmq_linear_forward runs this Linear at this batch size through dmq_linear_gemm_i8. */
+int dmq_linear_uses_i8_gemm(const dmq_linear_desc* linear, int rows);
+
 /* Bytes of scratch dmq_linear_forward needs for batches of up to max_rows rows (0: bad descriptor). */
 size_t dmq_linear_workspace_bytes(const dmq_linear_desc* linear, int max_rows);
 

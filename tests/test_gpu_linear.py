@@ -193,12 +193,13 @@ def _big_packed(bit):
 @pytest.mark.parametrize("cls,mode,tol", [("WxA16Linear", "wxa16", 1.5e-3), ("WxA8Linear", "wxa8", 6e-3),
                                           ("WxFP8Linear", "wxfp8", 2e-2)])
 @pytest.mark.parametrize("bit", [4, 8])
-@pytest.mark.parametrize("rows", [65, 1100, 2100, 4200])
+@pytest.mark.parametrize("rows", [65, 1100, 2100, 4200, 6200])
 def test_linear_entry_point_equals_its_pieces(cls, mode, tol, bit, rows):
     """dmq_linear_forward against dmq_rotate + dmq_matmul_merged_gf issued one by one, over the
     launch shapes of bigger batches (1024 features = 4 blocks: 16-row tiles with K shared by two
     workgroups at 65 and 1100 rows, 32-row tiles at 2100, 64-row tiles at 4200 unless the weights
-    are 8-bit), with an input whose rows are strided; and against the oracle's dataflow."""
+    are 8-bit; 6200 rows of 8-bit weights on the int8 path: the 128 x 128-tile int8 GEMM), with an
+    input whose rows are strided; and against the oracle's dataflow."""
     import dartmoq_hip
     packed = _big_packed(bit)
     lin = dartmoq_hip.WxA16Linear.from_packed(packed)
@@ -210,6 +211,27 @@ def test_linear_entry_point_equals_its_pieces(cls, mode, tol, bit, rows):
     assert torch.equal(out, lin.forward_by_pieces(x))
     assert torch.equal(out, lin(x.contiguous()))
     assert relerr(out.float().cpu(), _dataflow(packed, wide[:, :512], mode)) < tol
+
+
+def test_int8_gemm_of_uniform_8bit_weights():
+    """dmq_linear_gemm_i8 (128 x 128 tiles, weights idx - 128 as a plain MFMA operand) on ragged
+    shapes (300 rows, 320 features: partial tiles both ways) against the look-up kernel's
+    table-free path and the oracle's int8 dataflow; the group sums are exact integers in both
+    kernels and are scaled and added in the same order."""
+    from dartmoq_hip import kernels as K, ops
+    packed = _packed8(320, 512, seed=6, uniform=True)
+    x = torch.randn(300, 512, generator=torch.Generator().manual_seed(2)).half()
+    idx_gf, norms_gf = K.convert_to_group_first(packed["indices_packed"].cuda(), packed["norms"].cuda(), 128, 8)
+    norms_pre = (norms_gf.float() / 128 ** 0.5).half()
+    rot = K.generate_batch_rotation_matrices(128, packed["seed"], 4, 128, device="cuda")
+    x_i8, x_s = K.rotate_quantize_fused(x.cuda(), rot, 128, 4, extra_scale=K.uniform_codebook_step(packed["codebook"]))
+    out = ops.linear_gemm_i8(x_i8, x_s, idx_gf, norms_pre)
+    dummy = torch.zeros(256, dtype=torch.int8, device="cuda")
+    lut_path = K.wxa8_matmul_grouped_gf(x_i8, x_s, idx_gf, dummy, norms_pre, 128, 4, 8, identity_cb=True)
+    assert out.shape == (300, 320)
+    assert relerr(out.float().cpu(), lut_path.float().cpu()) < 5e-4
+    assert relerr(out.float().cpu(), _dataflow(packed, x, "wxa8")) < 6e-3
+    assert torch.equal(out, ops.linear_gemm_i8(x_i8, x_s, idx_gf, norms_pre))
 
 
 # ----------------------------------------------------------------------------- 8-bit codebooks

@@ -512,10 +512,10 @@ int dmq_linear_gemm_i8(const void* x_i8, long x_row_bytes, const void* x_scale_f
 
 // 8-bit weights on a uniform grid, int8 path, enough rows to fill the chip with 128 x 128 tiles:
 // the plain int8 GEMM instead of the look-up kernels.  4096 x 4096, forward time: 2048 rows
-// 146 -> 101 us, 4096 rows 290 -> 193 us; at 1024 rows (256 tiles) the two are equal, below that
+// 146 -> 80 us, 4096 rows 290 -> 150 us, 768 rows 79 -> 61 us; with fewer tiles (640 rows: 160)
 // the 32-row look-up tiles win.
 #ifndef DMQ_LINEAR_I8_MIN_WGS
-#define DMQ_LINEAR_I8_MIN_WGS 384
+#define DMQ_LINEAR_I8_MIN_WGS 192
 #endif
 static bool linear_uses_i8_gemm(const dmq_linear_desc* L, int rows) {
   if (L->mode != DMQ_MODE_A8 || L->bit != 8 || L->lut) return false;

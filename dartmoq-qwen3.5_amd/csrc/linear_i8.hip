@@ -98,35 +98,35 @@ void dmq_linear_i8_kernel(LinearI8Params p) {
       nrm[j] = *(const half4_t*)(p.norms + (long)g * p.n_out + nidx[j]);
       xs[j] = (float)p.x_scale[(long)ridx[j] * p.scale_stride + g];
     }
-    int4_t acc[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int t = 0; t < 4; ++t) acc[j][t] = (int4_t){0, 0, 0, 0};
     const int wl = (wave & 1) * 64, xl = (wave >> 1) * 64;   // the wave's rows inside the slots
+    // the activation operands of both MFMA steps stay in registers; the feature tiles go one
+    // after the other, so the scaling of tile row j overlaps the matrix work of tile row j + 1
+    int4_t b[2][4];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      int4_t a[4], b[4];
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        a[j] = *(const int4_t*)(wbuf[buf] + lds_off(wl + 16 * j + l16, 4 * s + q));
-        b[j] = *(const int4_t*)(xbuf[buf] + lds_off(xl + 16 * j + l16, 4 * s + q));
-      }
+      for (int t = 0; t < 4; ++t)
+        b[s][t] = *(const int4_t*)(xbuf[buf] + lds_off(xl + 16 * t + l16, 4 * s + q));
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 4; ++j) {
+      int4_t acc[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[t] = (int4_t){0, 0, 0, 0};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int4_t a = *(const int4_t*)(wbuf[buf] + lds_off(wl + 16 * j + l16, 4 * s + q));
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-          acc[j][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], b[t], acc[j][t], 0, 0, 0);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
+          acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[s][t], acc[t], 0, 0, 0);
+      }
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float v = (float)acc[j][t][r] * xs[t];
+          const float v = (float)acc[t][r] * xs[t];
           total[j][t][r] += v * (float)nrm[j][r];
         }
+    }
     if (g + 1 < p.groups) store(buf ^ 1);               // the other slot: last read one step ago
     __syncthreads();
   }

@@ -531,31 +531,44 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     // Loads retire in order, so each iteration requests slot data before weights: the wait
     // for the slot of group g + 1 then never covers weights younger than group g + 1.
     constexpr int NC = AB / 16;                       // chunks per row
-    constexpr int CPT = (TT * NC >= 16) ? TT * NC / 16 : 1;   // chunks per thread
-    constexpr int TPR = NC / CPT;                     // threads per row
+    constexpr int NCHUNK = 16 * TT * NC;              // chunks of the tile
+    constexpr int CPT = (NCHUNK + 255) / 256;         // chunks per thread
     constexpr int ACT_BYTES = 16 * TT * AB;
     constexpr int NORM_OFF = ACT_BYTES;
     constexpr int SCALE_OFF = NORM_OFF + 128 * NT;
     constexpr int SLOT = GG::SLOT;
     constexpr bool SCALED = (MODE != DMQ_MODE_A16);
     static_assert(NT <= 4, "a wave stages the norms of at most four n-tiles");
-    const int srow = threadIdx.x / TPR;               // >= 16*TT for threads without a chunk
-    const int sc0 = (threadIdx.x % TPR) * CPT;
-    const int s_rlog = r_first + srow;
-    const bool s_active = srow < 16 * TT;
-    const bool s_valid = s_active && s_rlog < r_end;
-    const int s_phys = s_valid ? (pw.row_index ? pw.row_index[s_rlog] : s_rlog) : 0;
-    const uint32_t s_off = (uint32_t)s_phys * (uint32_t)p.act_row_bytes + sc0 * 16;
+    // Thread t stages chunks t, t + 256, ... of the tile (chunk L = row L / NC, position L % NC), so
+    // the lanes of a load cover whole rows: 64 contiguous 16-byte pieces per row group, every
+    // cache line it touches is used in full.  Rows past the item's last row stage a copy of that
+    // last row: the loads stay unconditional (a predicated load is a branch and splits the loop
+    // into blocks whose wait counters are taken conservatively), and nothing computed from such
+    // a row is ever stored.
+    bool s_active[CPT];
+    uint32_t s_off[CPT], s_dst[CPT];
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+      const int L0 = c * 256 + (int)threadIdx.x;
+      s_active[c] = (NCHUNK % 256 == 0) || L0 < NCHUNK;     // threads past the tile reload its last chunk
+      const int L = (NCHUNK % 256 == 0) ? L0 : min(L0, NCHUNK - 1);
+      const int srow = L / NC, sc = L % NC;
+      const int s_rlog = min(r_first + srow, r_end - 1);
+      const int s_phys = pw.row_index ? pw.row_index[s_rlog] : s_rlog;
+      s_off[c] = (uint32_t)s_phys * (uint32_t)p.act_row_bytes + sc * 16;
+      s_dst[c] = (uint32_t)(srow * AB + ((sc ^ (srow & (NC - 1))) * 16));
+    }
     // lane (l16, q) stages the norm of row l16 of its wave's n-tile q
     const bool n_active = q < NT;
     const uint32_t n_off = 2u * (uint32_t)(SILU
         ? slice_start + ((q & 1) ? p.half_width : 0) + featw + (q >> 1) * 16 + l16
         : (p.slice_is_groups ? 0 : slice_start) + featw + q * 16 + l16);
     // thread t < 16*TT stages the scale word of tile row t
-    const int c_rlog = r_first + (int)threadIdx.x;
+    // (threads past the tile and rows past the item's last row read a valid row's scale: the load
+    // is unconditional, like the activation loads; only tile rows are stored)
+    const int c_rlog = min(r_first + min((int)threadIdx.x, 16 * TT - 1), r_end - 1);
     const bool c_active = SCALED && threadIdx.x < 16 * TT;
-    const bool c_valid = c_active && c_rlog < r_end;
-    const int c_phys = c_valid ? (pw.row_index ? pw.row_index[c_rlog] : c_rlog) : 0;
+    const int c_phys = SCALED ? (pw.row_index ? pw.row_index[c_rlog] : c_rlog) : 0;
     const uint32_t c_off = (uint32_t)c_phys * (uint32_t)p.act_scale_stride * (MODE == DMQ_MODE_FP4 ? 1u : 2u);
     uint32_t w_off[NT];
 #pragma unroll
@@ -575,28 +588,25 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     auto stage_load = [&](int k, int g, Staged& sr) {
       const uint8_t* abase = act_p + (long)g * AB;
 #pragma unroll
-      for (int c = 0; c < CPT; ++c)
-        sr.a[c] = s_valid ? *(const uint4_t*)(abase + lane_off(s_off) + c * 16) : (uint4_t){0u, 0u, 0u, 0u};
+      for (int c = 0; c < CPT; ++c) {
+        sr.a[c] = *(const uint4_t*)(abase + lane_off(s_off[c]));
+      }
       const uint8_t* nbase = norms_p + ((long)(g_base + g) * group_rows + (long)k * FPB) * 2;
       sr.nrm = n_active ? *(const uint16_t*)(nbase + lane_off(n_off)) : 0u;
       sr.sc = 0u;
       if constexpr (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
         const uint8_t* sbase = scale_p + (long)g * 2;
-        if (c_valid) sr.sc = *(const uint16_t*)(sbase + lane_off(c_off));
+        sr.sc = *(const uint16_t*)(sbase + lane_off(c_off));
       } else if constexpr (MODE == DMQ_MODE_FP4) {
         const uint8_t* sbase = scale_p + (long)g * 4;
-        sr.sc = 0x7f7f7f7fu;
-        if (c_valid) sr.sc = *(const uint32_t*)(sbase + lane_off(c_off));
+        sr.sc = *(const uint32_t*)(sbase + lane_off(c_off));
       }
     };
     auto stage_store = [&](int buf, const Staged& sr) {
       uint8_t* slot = stage + buf * SLOT;
-      if (s_active) {
-        uint8_t* base = slot + srow * AB;
 #pragma unroll
-        for (int c = 0; c < CPT; ++c)
-          *(uint4_t*)(base + (((sc0 + c) ^ (srow & (NC - 1))) * 16)) = sr.a[c];
-      }
+      for (int c = 0; c < CPT; ++c)
+        if (NCHUNK % 256 == 0 || s_active[c]) *(uint4_t*)(slot + s_dst[c]) = sr.a[c];
       if (n_active) *(uint16_t*)(slot + NORM_OFF + ((wave * NT + q) * 16 + l16) * 2) = (uint16_t)sr.nrm;
       if (c_active) *(uint32_t*)(slot + SCALE_OFF + threadIdx.x * 4) = sr.sc;
     };

@@ -61,7 +61,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 12; }
+int dmq_abi_version(void) { return 13; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -189,6 +189,47 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
                                tile_rows, max_items, counts, offsets, sorted_tokens, sorted_weights,
                                sorted_rows, gu_info, dn_info, n_items, items, scratch, scratch_bytes,
                                nullptr, -1, stream);
+}
+
+// Scratch of dmq_route_permute_static: the per-chunk expert histograms of the counting sort at their
+// largest (DMQ_SORT_MAX_CHUNKS chunks x DMQ_SORT_MAX_EXPERTS experts), one copy per GPU, held until the
+// process ends.  Host code never uses the array's name as an address: the device address is looked
+// up once per device (with that device current) and cached.
+#define DMQ_STATIC_SCRATCH_BYTES (DMQ_SORT_MAX_CHUNKS * DMQ_SORT_MAX_EXPERTS * 4)
+#define DMQ_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char dmq_static_scratch[DMQ_STATIC_SCRATCH_BYTES];
+static void* dmq_static_scratch_ptr[DMQ_STATIC_MAX_DEVICES];
+
+static int static_scratch_address(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return DMQ_ERR_HIP;
+  if (dev < 0 || dev >= DMQ_STATIC_MAX_DEVICES) return DMQ_ERR_LIMIT;
+  if (!dmq_static_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(dmq_static_scratch)) != hipSuccess || !ptr) return DMQ_ERR_HIP;
+    dmq_static_scratch_ptr[dev] = ptr;
+  }
+  *out = dmq_static_scratch_ptr[dev];
+  return DMQ_OK;
+}
+
+int dmq_route_permute_static(const void* topk_idx, const void* topk_w, int tokens, int k, int experts,
+                             int pools, const void* slice_start, const void* slice_count,
+                             int tile_rows, int max_items, void* counts, void* offsets,
+                             void* sorted_tokens, void* sorted_weights, void* sorted_rows,
+                             void* gu_info, void* dn_info, void* n_items, void* items, void* stream) {
+  if (tokens <= 0 || k <= 0 || experts <= 0) return DMQ_ERR_SHAPE;
+  if (experts > DMQ_SORT_MAX_EXPERTS) return DMQ_ERR_LIMIT;          // histograms would not fit
+  if (dmq_route_scratch_bytes(tokens, k, experts) > (size_t)DMQ_STATIC_SCRATCH_BYTES) return DMQ_ERR_LIMIT;
+  void* scratch = nullptr;
+  const int rc = static_scratch_address(&scratch);
+  if (rc) return rc;
+  // every (chunk, expert) cell the launch reads is written by its counting pass first: nothing
+  // has to start at zero
+  return route_permute_ordered(topk_idx, topk_w, tokens, k, experts, pools, slice_start, slice_count,
+                               tile_rows, max_items, counts, offsets, sorted_tokens, sorted_weights,
+                               sorted_rows, gu_info, dn_info, n_items, items, scratch,
+                               DMQ_STATIC_SCRATCH_BYTES, nullptr, -1, stream);
 }
 
 int dmq_build_tiles(const void* expert_info, int n_experts, int tile_rows, int max_items, int pool,

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 12
+ABI_VERSION = 13
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER, EPI_SILU_ROT = 0, 1, 2, 3
@@ -104,6 +104,8 @@ PROTOTYPES = {
     "dmq_route_permute": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                   c_int, c_int] + [c_void_p] * 10 + [c_size_t, c_void_p]),
     "dmq_route_scratch_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "dmq_route_permute_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                                         c_int, c_int] + [c_void_p] * 10),
     "dmq_build_tiles": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "dmq_rotate": (c_int, [c_int, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p,
                            c_long, c_void_p, c_int, c_int, c_float, c_int, c_void_p]),

@@ -150,8 +150,12 @@ def route_topk_shared(logits, topk_idx, topk_w, top_k: int, renormalize: bool, x
     return w, idx
 
 
-def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_rows=16):
-    """Device-side sort + pool partition.  Returns a dict of int32/fp32 device tensors."""
+def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_rows=16,
+                  static_scratch=False):
+    """Device-side sort + pool partition.  Returns a dict of int32/fp32 device tensors.
+    ``static_scratch``: go through dmq_route_permute_static, whose histograms live in the library's
+    static device array instead of a scratch tensor (the entry point for callers that cannot
+    allocate; calls that overlap on one GPU would race on that array)."""
     _need_cuda(topk_idx, topk_w, slice_start, slice_count)
     t, k = topk_idx.shape
     dev = topk_idx.device
@@ -171,6 +175,15 @@ def route_permute(topk_idx, topk_w, num_experts, slice_start, slice_count, tile_
         "items": torch.zeros((max_items, ITEM_WORDS), **i32),
         "max_items": max_items, "tile_rows": tile_rows,
     }
+    if static_scratch:
+        check(load().dmq_route_permute_static(
+            _ptr(topk_idx.to(torch.int32).contiguous()), _ptr(topk_w.float().contiguous()), t, k,
+            num_experts, pools, _ptr(slice_start.contiguous()), _ptr(slice_count.contiguous()),
+            tile_rows, max_items, _ptr(res["counts"]), _ptr(res["offsets"]), _ptr(res["sorted_tokens"]),
+            _ptr(res["sorted_weights"]), _ptr(res["sorted_rows"]), _ptr(res["gu_info"]),
+            _ptr(res["dn_info"]), _ptr(res["n_items"]), _ptr(res["items"]), _stream(dev)),
+            "route_permute_static")
+        return res
     scratch = torch.empty(max(1, load().dmq_route_scratch_bytes(t, k, num_experts)),
                           dtype=torch.uint8, device=dev)
     check(load().dmq_route_permute(

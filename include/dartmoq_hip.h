@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 9). */
+/* Library / build identification: returns the ABI version (currently 13). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -139,6 +139,21 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
                       void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
                       void* n_items, void* items, void* scratch, size_t scratch_bytes,
                       void* stream);
+
+/* dmq_route_permute for callers that cannot allocate or bring a scratch buffer (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The scratch (per-chunk expert histograms) lives in a static device array of 512 KiB inside the
+ * library, one copy per GPU, held until the process ends; its size covers every accepted call
+ * (any number of tokens, experts <= 2048; larger problems return DMQ_ERR_LIMIT).  The call
+ * allocates nothing.  All calls on one GPU share that array: calls that overlap on a GPU (two
+ * streams, two threads) race; calls ordered on one stream do not.  Arguments and outputs as
+ * dmq_route_permute. */
+int dmq_route_permute_static(const void* topk_idx, const void* topk_w, int tokens, int k,
+                             int experts, int pools, const void* slice_start,
+                             const void* slice_count, int tile_rows, int max_items, void* counts,
+                             void* offsets, void* sorted_tokens, void* sorted_weights,
+                             void* sorted_rows, void* gu_info, void* dn_info, void* n_items,
+                             void* items, void* stream);
 
 /* Work items for a caller-built expert_info: n_items int32[1], items int32 [max_items, 4]
  * with the given pool id. */

@@ -1,0 +1,73 @@
+"""GPU test of the entry point that allocates nothing: dmq_route_permute_static.
+
+Its scratch (the per-chunk expert histograms of the counting sort) is a static device array inside
+the library, shared by every call on a GPU and holding whatever the last call left.  Two calls in a
+row, the second on a smaller input, must each reproduce dmq_route_permute (caller-provided scratch)
+exactly: integer outputs and the gathered fp32 weights bit for bit.
+"""
+
+import pytest
+import torch
+
+from oracle import routing
+
+pytestmark = pytest.mark.gpu
+
+KEYS = ("counts", "offsets", "sorted_tokens", "sorted_weights", "sorted_rows", "gu_info", "dn_info")
+
+
+def _slices(expert_bit, inter, bits):
+    e = len(expert_bit)
+    start = torch.full((len(bits), e), -1, dtype=torch.int32)
+    count = torch.zeros((len(bits), e), dtype=torch.int32)
+    for pi, b in enumerate(bits):
+        cur = 0
+        for ex in range(e):
+            if expert_bit[ex] == b:
+                start[pi, ex] = 2 * cur
+                count[pi, ex] = 2 * inter
+                cur += inter
+    return start, count
+
+
+def _compare(tokens, experts, k, tile_rows, seed):
+    from dartmoq_hip import ops
+    inter = 256
+    expert_bit = [4 if e % 9 == 0 else (1 if e % 13 == 5 else 2) for e in range(experts)]
+    start, count = _slices(expert_bit, inter, [4, 2, 1])
+    w, idx = routing.route_topk(routing.zipf_logits(tokens, experts, seed=seed), k)
+    args = (idx.int().cuda(), w.cuda(), experts, start.cuda(), count.cuda(), tile_rows)
+    want = ops.route_permute(*args)
+    got = ops.route_permute(*args, static_scratch=True)
+    torch.cuda.synchronize()
+    for key in KEYS:
+        assert torch.equal(got[key].view(torch.int32), want[key].view(torch.int32)), key
+    n = int(want["n_items"][0])
+    assert int(got["n_items"][0]) == n and n > 0
+    assert torch.equal(got["items"][:n], want["items"][:n])
+    # and the permutation itself is right (stable sort by expert), not merely equal
+    toks, _wts, _slots, offs = routing.sort_by_expert(idx, w, experts)
+    assert torch.equal(got["sorted_tokens"].cpu().long(), toks)
+    assert got["offsets"].cpu().tolist() == offs.tolist()
+
+
+def test_static_scratch_two_calls_in_a_row():
+    # 4096 tokens x 8: the three-launch path whose histograms live in the scratch (64 chunks)
+    _compare(4096, 256, 8, 32, seed=1)
+    # a smaller input right after: fewer chunks, fewer experts; the array still holds the first
+    # call's histograms
+    _compare(600, 48, 4, 16, seed=2)
+    # and a batch small enough for the one-launch path, which never touches the scratch
+    _compare(16, 48, 4, 16, seed=3)
+
+
+def test_static_scratch_rejects_what_does_not_fit():
+    from dartmoq_hip import ops
+    experts, k = 2049, 2                                     # the histograms hold 2048 experts
+    idx = torch.zeros((700, k), dtype=torch.int32, device="cuda")
+    idx[:, 1] = 1
+    w = torch.ones((700, k), device="cuda")
+    start = torch.zeros((1, experts), dtype=torch.int32, device="cuda")
+    count = torch.full((1, experts), 512, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        ops.route_permute(idx, w, experts, start, count, 16, static_scratch=True)

@@ -61,7 +61,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 13; }
+int dmq_abi_version(void) { return 14; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -370,7 +370,8 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     const int qi = i < a->n_pools ? i : 0;
     p.pool[i] = PoolW{(const uint8_t*)q.w, (const __half*)q.norms, q.lut, (const int*)q.expert_info,
                       (const uint8_t*)q.act, q.act_scale, (const int*)q.row_index, q.n_total, q.bit,
-                      q.mode, q.w_scale_byte, (const __half*)a->post_rot[qi], a->post_extra_scale[qi]};
+                      q.mode, q.w_scale_byte, (const __half*)a->post_rot[qi], a->post_extra_scale[qi],
+                      (const int*)q.col_start, (const int*)q.home};
   }
   p.act_row_bytes = a->act_row_bytes;
   p.act_scale_stride = a->act_scale_stride;
@@ -390,6 +391,10 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.post_row_bytes = a->post_row_bytes;
   p.post_scale = a->post_scale;
   p.post_scale_stride = a->post_scale_stride;
+  if (a->width_filter != 0 && wsplit > 1) return DMQ_ERR_MODE;
+  p.width_filter = a->width_filter;
+  p.home_filter = a->width_filter != 0 ? a->home_filter : -1;
+  p.accumulate = (a->epi == DMQ_EPI_SCATTER && a->accumulate) ? 1 : 0;
   p.wsplit = wsplit;
   p.subs = subs;
   p.split_rows = a->split_rows;
@@ -697,7 +702,9 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   const size_t R = (size_t)tokens * L->top_k;
   const size_t E = L->experts, P = L->pools, H = L->hidden, I = L->inter;
   w.tile_rows = 16 * tt;
-  w.max_items = (int)(R / w.tile_rows + E);
+  // an expert of a sub-expert layer has work items in every pool that holds a share of it
+  const size_t homes = L->n_widths > 0 && L->max_homes > 1 ? (size_t)L->max_homes : 1;
+  w.max_items = (int)((R / w.tile_rows + E) * homes);
   size_t off = 0;
   auto take = [&](size_t n) { uint8_t* p = base + off; off += align_up(n); return p; };
   w.counts = (int*)take(E * 4);
@@ -723,7 +730,9 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.xq_rows_scale = take(R * (H / DMQ_GS) * 4);
   w.act = take(R * I * 2);
   w.actq = take(R * I * 2);
-  w.actq_scale = take(R * (I / DMQ_GS) * 4);
+  // two areas: the second holds the block scales of the FP4 pools of a sub-expert layer, whose
+  // rows may also carry the int8 share of another pool
+  w.actq_scale = take(2 * R * (I / DMQ_GS) * 4);
   w.split_rows = (int)(R < DMQ_SPLIT_MAX_ROWS ? R : DMQ_SPLIT_MAX_ROWS);
   w.split_partial = (float*)take((size_t)4 * w.split_rows * 2 * I * 4);
   w.split_counters = (int)((R / 16 + E) * (I / DMQ_GS));
@@ -785,17 +794,37 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if ((long)tokens * K > DMQ_SPLIT_MAX_ROWS) return DMQ_ERR_LIMIT;
     ks = 1;
   }
+  // Sub-expert layers (experts spread over several pools, shares of several widths): one gate_up
+  // launch per width and one down launch per (rank, width); no K sharing between workgroups or
+  // waves, every pool rotated by token (a routed row may feed several pools)
+  const bool sub = layer->n_widths > 0;
+  if (sub) {
+    if (layer->n_widths > 8 || layer->max_homes <= 0 || layer->max_homes > P) return DMQ_ERR_LIMIT;
+    if (!layer->col_start || !layer->home) return DMQ_ERR_NULL;
+    for (int i = 0; i < layer->n_widths; ++i)
+      if (layer->widths[i] <= 0 || layer->widths[i] % DMQ_GS || layer->widths[i] > I) return DMQ_ERR_ALIGN;
+    ks = 1;
+  }
+  const int wsplit_eff = sub ? 1 : wsplit;
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   if (nbl <= 0) nbl = pick_nbl((long)tokens * K, tt);
   // a rotation wave covers 16 or 32 rows: 64-row work items are rotated by two waves each
   const int rot_tt = tt > 2 ? 2 : tt;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
   if (w.bytes > workspace_bytes) return DMQ_ERR_LIMIT;
+  // Rotated down-projection input.  In a sub-expert layer one routed row may hold the shares of
+  // pools of two precision modes (wxfp4: 4-bit pools run FP4, 2-bit pools int8), whose codes and
+  // scales are laid out by column at different densities: the FP4 codes go to the upper half of the
+  // row (bytes [I, 1.5 I); int8 / fp8 codes fill [0, I)) and the FP4 scales to an area of their own.
+  auto actq_of = [&](int m) { return (sub && m == DMQ_MODE_FP4) ? w.actq + I : w.actq; };
+  auto actq_scale_of = [&](int m) {
+    return (sub && m == DMQ_MODE_FP4) ? w.actq_scale + (size_t)tokens * K * (I / DMQ_GS) * 4 : w.actq_scale;
+  };
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (aux_out) {
     long* aux = (long*)aux_out;
-    aux[0] = tt; aux[1] = wsplit > 1 ? -wsplit : ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
+    aux[0] = tt; aux[1] = wsplit_eff > 1 ? -wsplit_eff : ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
     aux[3] = w.max_items; aux[4] = (long)((uint8_t*)w.n_items - (uint8_t*)workspace);
     aux[5] = nbl;
   }
@@ -827,7 +856,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   // few dozen tokens for a pool that ends up using a handful is cheaper than the dependent
   // per-work-item pass (same values either way).
   bool whole_batch[DMQ_MAX_POOLS] = {false, false, false, false};
-  for (int i = 0; i < P; ++i) whole_batch[i] = layer->pool[i].major != 0 || tokens <= DMQ_HOIST_ALL_TOKENS;
+  for (int i = 0; i < P; ++i)
+    whole_batch[i] = sub || layer->pool[i].major != 0 || tokens <= DMQ_HOIST_ALL_TOKENS;
 
   // The pools whose rows are rotated per work item come first in the item list, so that the
   // rotation launch knows their items as a prefix (n_items[1]) and touches no other record.
@@ -913,7 +943,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       plan.lead_pools = lead_pools;
       sp.sorted_tokens = w.sorted_tokens; sp.sorted_weights = w.sorted_weights;
       sp.sorted_rows = w.sorted_rows;
-      if (wsplit > 1) { sp.clear_words = w.split_counter; sp.clear_count = w.split_counters; }
+      if (wsplit_eff > 1) { sp.clear_words = w.split_counter; sp.clear_count = w.split_counters; }
       rc = dmq_route_small_launch(sp, st);
     } else {
       const void* tk_idx = router->topk_idx;
@@ -932,7 +962,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
                                  w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items,
                                  w.items, w.sort_scratch, w.sort_scratch_bytes, pool_order,
                                  lead_pools, stream);
-      if (!rc && wsplit > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
+      if (!rc && wsplit_eff > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
     }
   }
   if (rc) return rc;
@@ -966,21 +996,35 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
                                 hoisted ? w.sorted_tokens : nullptr, pd.n_gate_up, pd.bit, pd.mode,
                                 pd.gu_w_scale_byte};
     }
+    if (sub)
+      for (int i = 0; i < P; ++i) {
+        g.pool[i].col_start = (const int*)layer->col_start + (size_t)i * E;
+        g.pool[i].home = (const int*)layer->home + (size_t)i * E;
+      }
     g.act_row_bytes = (long)H * 2;
     g.act_scale_stride = scale_stride_for(mode, H);
     g.groups = H / DMQ_GS; g.n_out = I; g.half_width = I; g.slice_is_groups = 0;
     g.items = w.items; g.n_items = w.n_items; g.max_items = w.max_items;
     g.out = w.act; g.out_stride = I;
-    g.post_out = w.actq; g.post_row_bytes = (long)I * 2;
-    g.post_scale = w.actq_scale; g.post_scale_stride = scale_stride_for(mode, I);
+    g.post_out = actq_of(mode); g.post_row_bytes = (long)I * 2;
+    g.post_scale = actq_scale_of(mode); g.post_scale_stride = scale_stride_for(mode, I);
     bool mode_wide = false;
     for (int i = 0; i < P; ++i) mode_wide |= (layer->pool[i].mode == mode && layer->pool[i].bit == 8);
-    if (wsplit > 1 && !mode_wide) {
-      g.k_split = wsplit; g.split_rows = w.split_rows;
+    if (wsplit_eff > 1 && !mode_wide) {
+      g.k_split = wsplit_eff; g.split_rows = w.split_rows;
       g.split_partial = w.split_partial; g.split_counter = w.split_counter;
     }
-    rc = dmq_matmul_merged_gf(&g, stream);
-    if (rc) return rc;
+    if (!sub) {
+      rc = dmq_matmul_merged_gf(&g, stream);
+      if (rc) return rc;
+    } else {
+      for (int wi = 0; wi < layer->n_widths; ++wi) {     // one launch per share width
+        const int W = layer->widths[wi];
+        g.n_out = W; g.half_width = W; g.width_filter = 2 * W; g.home_filter = -1;
+        rc = dmq_matmul_merged_gf(&g, stream);
+        if (rc) return rc;
+      }
+    }
   }
 
   mark(3);
@@ -997,10 +1041,11 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       const int pi = i < P ? i : 0;
       const dmq_pool_desc& pd = layer->pool[pi];
       const bool live = i < P && pd.mode == mode;
-      rp.pool[i] = RotPool{(const __half*)pd.dn_rot, w.actq,
-                           (long)I * 2, w.actq_scale,
+      rp.pool[i] = RotPool{(const __half*)pd.dn_rot, actq_of(pd.mode),
+                           (long)I * 2, actq_scale_of(pd.mode),
                            scale_stride_for(pd.mode, I), w.dn_info + (size_t)pi * E * 4,
-                           pd.dn_extra_scale, live ? pd.mode : -1, 0, 1};
+                           pd.dn_extra_scale, live ? pd.mode : -1, 0, 1,
+                           sub ? (const int*)layer->col_start + (size_t)pi * E : nullptr};
     }
     const long n = (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
     rc = dmq_rotate_dispatch(mode, rp, n, rot_tt, st);
@@ -1031,8 +1076,39 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     d.items = w.items; d.n_items = w.n_items; d.max_items = w.max_items;
     d.out = w.slots; d.out_stride = H;
     d.row_weight = w.sorted_weights; d.row_slot = w.sorted_rows;
-    rc = dmq_matmul_merged_gf(&d, stream);
-    if (rc) return rc;
+    if (!sub) {
+      rc = dmq_matmul_merged_gf(&d, stream);
+      if (rc) return rc;
+    }
+  }
+  if (sub) {
+    // rank 0 stores every slot row (every routed expert has a first share), the following ranks
+    // add theirs in rank order: the sum over the pools of bit_partitioned_moe.py:818-822
+    for (int h = 0; h < layer->max_homes; ++h)
+      for (int mi = 0; mi < n_modes; ++mi)
+        for (int wi = 0; wi < layer->n_widths; ++wi) {
+          const int mode = modes[mi], W = layer->widths[wi];
+          dmq_gemm_args d{};
+          d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt == 4 ? 2 : tt; d.item_tile_rows = 16 * tt;
+          d.ks = 1; d.nbl = nbl; d.n_pools = P;
+          for (int i = 0; i < P; ++i) {
+            const dmq_pool_desc& pd = layer->pool[i];
+            d.pool[i] = dmq_gemm_pool{pd.dn_w, pd.dn_norms, pd.dn_lut, w.dn_info + (size_t)i * E * 4,
+                                      actq_of(pd.mode), actq_scale_of(pd.mode), nullptr, H, pd.bit,
+                                      pd.mode, pd.dn_w_scale_byte,
+                                      (const int*)layer->col_start + (size_t)i * E,
+                                      (const int*)layer->home + (size_t)i * E};
+          }
+          d.act_row_bytes = (long)I * 2;
+          d.act_scale_stride = scale_stride_for(mode, I);
+          d.groups = W / DMQ_GS; d.n_out = H; d.half_width = 0; d.slice_is_groups = 1;
+          d.items = w.items; d.n_items = w.n_items; d.max_items = w.max_items;
+          d.out = w.slots; d.out_stride = H;
+          d.row_weight = w.sorted_weights; d.row_slot = w.sorted_rows;
+          d.width_filter = W / DMQ_GS; d.home_filter = h; d.accumulate = h > 0;
+          rc = dmq_matmul_merged_gf(&d, stream);
+          if (rc) return rc;
+        }
   }
 
   mark(5);

@@ -40,7 +40,7 @@ template <int MODE, int TT, int KS>
 static int dmq_gemm_launch_epi(const GemmLaunch& L) {
   switch (L.epi) {
     case DMQ_EPI_STORE:
-      if constexpr (MODE == DMQ_MODE_A8 && TT == 1 && KS == 1) {
+      if constexpr (MODE == DMQ_MODE_A8 && KS == 1) {      // 16-, 32- and 64-row tiles
         if (L.dbg) return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_STORE, true>(L);
       }
       return dmq_gemm_launch_one<MODE, TT, KS, DMQ_EPI_STORE, false>(L);
@@ -74,7 +74,7 @@ static int dmq_gemm_launch_mode(const GemmLaunch& L) {
     if (L.tt != 1 || L.ks != 4 || L.epi != DMQ_EPI_STORE || L.dbg) return DMQ_ERR_MODE;
     return dmq_gemm_launch_narrow<MODE>(L);
   }
-  if (L.dbg && !(MODE == DMQ_MODE_A8 && L.tt == 1 && L.ks == 1 && L.epi == DMQ_EPI_STORE))
+  if (L.dbg && !(MODE == DMQ_MODE_A8 && L.ks == 1 && L.epi == DMQ_EPI_STORE))
     return DMQ_ERR_MODE;
   if (L.tt == 1 && L.ks == 4) return dmq_gemm_launch_epi<MODE, 1, 4>(L);
   if (L.tt == 1 && L.ks == 1) return dmq_gemm_launch_epi<MODE, 1, 1>(L);

@@ -68,6 +68,12 @@ struct PoolW {
   // into the stored activation scale
   const __half* post_rot;
   float post_extra;
+  // layers whose experts are cut into sub-experts living in several pools (width_filter != 0):
+  // first activation column of the pool's share of each expert (act / post_out columns of the
+  // gate_up launch, contracted columns of the down launch) and the expert's rank among the pools
+  // that hold a share of it
+  const int* col_start;        // [n_experts] or NULL (0)
+  const int* home;             // [n_experts] or NULL (0)
 };
 
 struct GemmParams {
@@ -101,6 +107,13 @@ struct GemmParams {
   // K range of one (item, block) shared by wsplit workgroups (16-row tiles, SiLU and plain-store
   // epilogues): each parks its fp32 sums in its plane of split_partial and takes a ticket; the
   // last one adds the planes in plane order and runs the epilogue
+  // Sub-expert layers: a launch serves the (pool, expert) shares of one width (and, for the down
+  // projection, of one home rank); it skips work items whose slice count (expert_info[e][3]) differs
+  // from width_filter (0 = take all) or whose rank differs from home_filter (< 0 = take all).
+  // accumulate (SCATTER): add to the slot row instead of storing it (ranks above 0).
+  int width_filter;
+  int home_filter;
+  int accumulate;
   int wsplit;                  // 1, 2, 4, 8 or 16
   int split_rows;              // rows of one plane
   float* split_partial;        // fp32 [wsplit, split_rows, 2 * n_out (SiLU) or n_out (store)]
@@ -242,7 +255,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
                                               uint8_t* smem2, uint8_t* smem_post, int token_start,
                                               int token_count, int slice_start, int post_slice,
                                               int ttile, int nb, int nbc, int split, int* ticket,
-                                              int* wg_flag) {
+                                              int* wg_flag, int col0) {
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   using GG = GemmGeom<MODE, NT, TT, KS>;
@@ -283,6 +296,10 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     else wrow[j] = (p.slice_is_groups ? 0 : slice_start) + featw + j * 16;
   }
   const int g_base = p.slice_is_groups ? slice_start : 0;
+  // sub-expert layers: the down launch contracts the expert's columns from col0 on (whole groups),
+  // the gate_up launch writes its SiLU*up columns from col0 on
+  const int in_group0 = p.slice_is_groups ? col0 / DMQ_GS : 0;
+  const int out_col0 = p.slice_is_groups ? 0 : col0;
   const int g_lo = (p.groups * kpart) / KS;
   const int g_hi = (p.groups * (kpart + 1)) / KS;
 
@@ -298,7 +315,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     rlog[t] = r_first + t * 16 + l16;
     avalid[t] = rlog[t] < r_end;
     rphys[t] = avalid[t] ? (pw.row_index ? pw.row_index[rlog[t]] : rlog[t]) : 0;
-    arow[t] = pw.act + (long)rphys[t] * p.act_row_bytes + q * (AW * 4);
+    arow[t] = pw.act + (long)rphys[t] * p.act_row_bytes + q * (AW * 4) + in_group0 * AB;
   }
 
   float4_t total_acc[NT][TT];
@@ -321,11 +338,11 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     for (int t = 0; t < TT; ++t) {
       xs[t] = 1.0f; xsb[t] = 127;
       if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
-        xs[t] = avalid[t] ? (float)((const __half*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g]
+        xs[t] = avalid[t] ? (float)((const __half*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + in_group0 + g]
                           : 0.f;
       } else if (MODE == DMQ_MODE_FP4) {
         if (avalid[t])
-          xsb[t] = ((const uint8_t*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + g * 4 + q];
+          xsb[t] = ((const uint8_t*)pw.act_scale)[(long)rphys[t] * p.act_scale_stride + (in_group0 + g) * 4 + q];
       }
     }
   };
@@ -484,12 +501,17 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 #pragma unroll
           for (int r = 0; r < 4; ++r)
             h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
-          *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + feat_k + (j >> 1) * 16 + 4 * q) = h;
+          *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + out_col0 + feat_k + (j >> 1) * 16 + 4 * q) = h;
         } else {
           const float rw = p.row_weight[rlog[t]];
-          const float4_t v = total_acc[j][t] * rw;
+          float4_t v = total_acc[j][t] * rw;
+          half4_t* dst = (half4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat_k + j * 16 + 4 * q);
+          if (p.accumulate) {                  // a further share of the expert: add to what is there
+            const half4_t prev = *dst;
+            v += (float4_t){(float)prev[0], (float)prev[1], (float)prev[2], (float)prev[3]};
+          }
           const half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-          *(half4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat_k + j * 16 + 4 * q) = h;
+          *dst = h;
         }
       }
     }
@@ -555,7 +577,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       const int srow = L / NC, sc = L % NC;
       const int s_rlog = min(r_first + srow, r_end - 1);
       const int s_phys = pw.row_index ? pw.row_index[s_rlog] : s_rlog;
-      s_off[c] = (uint32_t)s_phys * (uint32_t)p.act_row_bytes + sc * 16;
+      s_off[c] = (uint32_t)s_phys * (uint32_t)p.act_row_bytes + sc * 16 + (uint32_t)in_group0 * AB;
       s_dst[c] = (uint32_t)(srow * AB + ((sc ^ (srow & (NC - 1))) * 16));
     }
     // lane (l16, q) stages the norm of row l16 of its wave's n-tile q
@@ -569,7 +591,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     const int c_rlog = min(r_first + min((int)threadIdx.x, 16 * TT - 1), r_end - 1);
     const bool c_active = SCALED && threadIdx.x < 16 * TT;
     const int c_phys = SCALED ? (pw.row_index ? pw.row_index[c_rlog] : c_rlog) : 0;
-    const uint32_t c_off = (uint32_t)c_phys * (uint32_t)p.act_scale_stride * (MODE == DMQ_MODE_FP4 ? 1u : 2u);
+    const uint32_t c_off = ((uint32_t)c_phys * (uint32_t)p.act_scale_stride) * (MODE == DMQ_MODE_FP4 ? 1u : 2u) +
+                           (uint32_t)in_group0 * (MODE == DMQ_MODE_FP4 ? 4u : 2u);
     uint32_t w_off[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) w_off[j] = (uint32_t)(wrow[j] + l16) * PPG + q * (WW * 4);
@@ -701,7 +724,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
                                                                    racc[jt][t], 0, 0, 0);
           }
         }
-        const int col0 = blk + 32 * wave + 4 * q;                  // + 16*jt: first of the lane's 4 outputs
+        const int col0 = out_col0 + blk + 32 * wave + 4 * q;       // + 16*jt: first of the lane's 4 outputs
+        const int out_group = (out_col0 + blk) / DMQ_GS;           // group of the down projection's input
         if constexpr (MODE == DMQ_MODE_A16) {
 #pragma unroll
           for (int t = 0; t < TT; ++t) {
@@ -757,7 +781,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
               *(uint32_t*)(orow + col0 + 16 * jt) = word;
             }
             if (wave == 0 && q == 0)
-              ((__half*)p.post_scale)[(long)rlog[t] * p.post_scale_stride + blk / DMQ_GS] =
+              ((__half*)p.post_scale)[(long)rlog[t] * p.post_scale_stride + out_group] =
                   __float2half_rn(sc * pw.post_extra);
           }
         } else {   // FP4: the wave's 32 outputs are one MX block
@@ -787,7 +811,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
               *(uint16_t*)(orow + (col0 + 16 * jt) / 2) = (uint16_t)half_word;
             }
             if (q == 0)
-              ((uint8_t*)p.post_scale)[(long)rlog[t] * p.post_scale_stride + (blk / DMQ_GS) * 4 + wave] =
+              ((uint8_t*)p.post_scale)[(long)rlog[t] * p.post_scale_stride + out_group * 4 + wave] =
                   (uint8_t)fminf(fmaxf(e + 127.0f, 0.f), 254.f);
           }
         }
@@ -1114,18 +1138,25 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE) return;
   if (WIDE != (pw.bit == 8)) return;
+  int col0 = 0;
+  if (p.width_filter != 0) {                             // sub-expert layers: one width (and rank) per launch
+    const int e = r0[1];
+    if (pw.expert_info[e * 4 + 3] != p.width_filter) return;
+    if (p.home_filter >= 0 && (pw.home ? pw.home[e] : 0) != p.home_filter) return;
+    col0 = pw.col_start ? pw.col_start[e] : 0;
+  }
   if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
+    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
   } else if constexpr (WIDE) {
     if (MODE == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
-      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG, MODE == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
+      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG, MODE == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
     else
-      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag);
+      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
   } else {
     switch (pw.bit) {
-      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;
-      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;
-      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag); break;
+      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
     }
   }
 }

@@ -16,6 +16,9 @@ struct RotPool {
   int mode;                // pools whose mode differs from the kernel's are skipped
   int hoisted;             // 1: every input row is rotated once; 0: rows follow the work items
   int rot_use_slice;       // tiled: 1 = matrices start at the expert's slice_start (down), 0 = at 0
+  const int* col_start;    // sub-expert layers (per-work-item pools whose matrix depends on the slice):
+                           // first column of the pool's share of each expert [n_experts]; NULL = 0 and
+                           // every item spans all `groups`
 };
 
 // Side job of a rotation launch in front of a stand-alone Linear GEMM: workgroup 0 also writes the

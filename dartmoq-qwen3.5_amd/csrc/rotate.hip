@@ -43,6 +43,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
   // once.  The remaining workgroups take one work item per wave and read their matrices (one
   // per expert with rot_use_slice) straight from memory.
   int pool, g, r_first, r_end, rot_g;
+  int cg = -1;                                          // column group of the rows; -1: the group g
   int stage_pool = -1;                                  // tiled workgroups: pool whose matrix is staged
   const int* row_index = nullptr;
   const long hoisted_wgs = (long)p.n_hoisted * p.hoisted_wgs_per_pool;
@@ -105,7 +106,15 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
     r_end = ts + tc;
     rot_g = (p.pool[pool].rot_use_slice ? it[6] : 0) + g;
     row_index = p.row_index;
+    if (p.pool[pool].col_start) {
+      // sub-expert layers: the pool's share of the expert is expert_info[e][3] groups wide and
+      // starts at column col_start[e] of the row
+      const int e = it[1];
+      if (g >= p.pool[pool].expert_info[e * 4 + 3]) return;
+      cg = p.pool[pool].col_start[e] / DMQ_GS + g;
+    }
   }
+  if (cg < 0) cg = g;
   const RotPool& rp = p.pool[pool];
   const bool tiled_wg = !hoisted && p.tiled_staged;
   if (!tiled_wg && rp.mode != MODE) return;
@@ -118,7 +127,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
     rlog[t] = r_first + t * 16 + l16;
     valid[t] = rlog[t] < r_end;
     int phys = valid[t] ? (row_index ? row_index[rlog[t]] : rlog[t]) : 0;
-    xrow[t] = p.x + (long)phys * p.x_stride + g * DMQ_GS + 8 * q;
+    xrow[t] = p.x + (long)phys * p.x_stride + cg * DMQ_GS + 8 * q;
   }
   // the rows of the tile are requested before the matrix is staged, so both are in flight together
   uint4_t xraw[4][TT];
@@ -190,7 +199,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
       for (int j = 0; j < 8; ++j) {
         half4_t h = {(_Float16)acc[j][t][0], (_Float16)acc[j][t][1], (_Float16)acc[j][t][2],
                      (_Float16)acc[j][t][3]};
-        *(half4_t*)(orow + (g * DMQ_GS + j * 16 + 4 * q) * 2) = h;
+        *(half4_t*)(orow + (cg * DMQ_GS + j * 16 + 4 * q) * 2) = h;
       }
     } else if (MODE == DMQ_MODE_A8 || MODE == DMQ_MODE_FP8) {
       float amax = 0.f;
@@ -218,12 +227,12 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
           }
           word |= code << (8 * r);
         }
-        *(uint32_t*)(orow + g * DMQ_GS + j * 16 + 4 * q) = word;
+        *(uint32_t*)(orow + cg * DMQ_GS + j * 16 + 4 * q) = word;
       }
       if (q == 0) {
         const float stored = sc * rp.extra_scale;
-        if (p.scale_fp32) ((float*)rp.scale)[(long)rlog[t] * rp.scale_stride + g] = stored;
-        else ((__half*)rp.scale)[(long)rlog[t] * rp.scale_stride + g] = __float2half_rn(stored);
+        if (p.scale_fp32) ((float*)rp.scale)[(long)rlog[t] * rp.scale_stride + cg] = stored;
+        else ((__half*)rp.scale)[(long)rlog[t] * rp.scale_stride + cg] = __float2half_rn(stored);
       }
     } else {   // FP4: four MX blocks of 32 per group
       uint32_t sbytes = 0;
@@ -250,12 +259,12 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
               uint32_t nib = dmq_e2m1_mag(fabsf(y)) | ((y < 0.f) ? 8u : 0u);
               half_word |= nib << (4 * r);
             }
-            *(uint16_t*)(orow + (g * DMQ_GS + (2 * b + jj) * 16 + 4 * q) / 2) = (uint16_t)half_word;
+            *(uint16_t*)(orow + (cg * DMQ_GS + (2 * b + jj) * 16 + 4 * q) / 2) = (uint16_t)half_word;
           }
         }
       }
       if (valid[t] && q == 0)
-        *(uint32_t*)((uint8_t*)rp.scale + (long)rlog[t] * rp.scale_stride + g * 4) = sbytes;
+        *(uint32_t*)((uint8_t*)rp.scale + (long)rlog[t] * rp.scale_stride + cg * 4) = sbytes;
     }
   }
 }

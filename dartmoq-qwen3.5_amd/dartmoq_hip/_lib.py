@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 13
+ABI_VERSION = 14
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER, EPI_SILU_ROT = 0, 1, 2, 3
@@ -31,6 +31,7 @@ class GemmPool(Structure):
         ("w", c_void_p), ("norms", c_void_p), ("lut", c_void_p), ("expert_info", c_void_p),
         ("act", c_void_p), ("act_scale", c_void_p), ("row_index", c_void_p),
         ("n_total", c_int), ("bit", c_int), ("mode", c_int), ("w_scale_byte", c_int),
+        ("col_start", c_void_p), ("home", c_void_p),
     ]
 
 
@@ -50,6 +51,7 @@ class GemmArgs(Structure):
         ("k_split", c_int), ("split_rows", c_int), ("split_partial", c_void_p), ("split_counter", c_void_p),
         ("item_tile_rows", c_int),
         ("nt", c_int),
+        ("width_filter", c_int), ("home_filter", c_int), ("accumulate", c_int),
     ]
 
 
@@ -76,6 +78,8 @@ class LayerDesc(Structure):
     _fields_ = [
         ("hidden", c_int), ("inter", c_int), ("experts", c_int), ("top_k", c_int), ("pools", c_int),
         ("pool", POINTER(PoolDesc)), ("slice_start", c_void_p), ("slice_count", c_void_p),
+        ("n_widths", c_int), ("widths", c_int * 8), ("max_homes", c_int),
+        ("col_start", c_void_p), ("home", c_void_p),
     ]
 
 

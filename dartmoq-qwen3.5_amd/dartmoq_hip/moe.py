@@ -146,19 +146,22 @@ class WxA16BitPartitionedGroupMoE:
             if len(offs) != num_experts + 1:
                 raise ValueError("expert_offsets must have num_experts + 1 entries")
             widths = {b - a for a, b in zip(offs[:-1], offs[1:]) if b > a}
-            if widths and widths != {intermediate_size}:
-                raise ValueError(f"every member of a pool must own {intermediate_size} neurons, "
-                                 f"got widths {sorted(widths)}")
+            if any(w_ % GROUP_SIZE or w_ > intermediate_size for w_ in widths):
+                raise ValueError(f"the share of an expert in a pool must be a multiple of {GROUP_SIZE} "
+                                 f"neurons and at most {intermediate_size}, got widths {sorted(widths)}")
             moe.bit_weights[bit_str] = BitPoolWeights(bit, p["gate_up"], p["down"], offs, moe.device)
             moe.expert_offsets[bit_str] = offs
             moe.bit_list.append(bit)
         if len(moe.bit_weights) > _lib_max_pools():
             raise ValueError(f"at most {_lib_max_pools()} bit pools per layer")
+        # An expert may be cut into sub-experts that live in several pools (the --slices layout,
+        # quantization/wxa16/bit_partitioned_moe.py:499-521): its shares must add up to the
+        # expert's intermediate size, its output is the sum over its pools (:818-822).
         for ex in range(num_experts):
-            homes = sum(1 for o in moe.expert_offsets.values() if o[ex + 1] > o[ex])
-            if homes != 1:
-                raise ValueError(f"expert {ex} belongs to {homes} bit pools; this build handles "
-                                 "layers whose experts live in exactly one pool")
+            total = sum(o[ex + 1] - o[ex] for o in moe.expert_offsets.values())
+            if total != intermediate_size:
+                raise ValueError(f"the shares of expert {ex} add up to {total} neurons, "
+                                 f"expected {intermediate_size}")
         if shared_expert is not None:
             moe.attach_shared_expert(shared_expert)
         return moe
@@ -184,8 +187,11 @@ class WxA16BitPartitionedGroupMoE:
         i_s, h = (int(v) for v in gate["shape"])
         if h != self.hidden_size or tuple(up["shape"]) != (i_s, h) or tuple(down["shape"]) != (h, i_s):
             raise ValueError("shared expert shapes must be gate/up [I_s, H], down [H, I_s]")
-        if i_s % inter:
-            raise ValueError(f"shared intermediate size {i_s} must be a multiple of {inter}")
+        if i_s % GROUP_SIZE:
+            raise ValueError(f"shared intermediate size {i_s} must be a multiple of {GROUP_SIZE}")
+        # slices of the routed experts' width when that divides the shared width, else the widest
+        # multiple of 128 that does (the layer then runs as a sub-expert layer: shares of several widths)
+        inter = max(w_ for w_ in range(GROUP_SIZE, inter + 1, GROUP_SIZE) if i_s % w_ == 0)
         bit = int(gate["bit_width"])
         if bit not in (1, 2, 4, 8) or int(up["bit_width"]) != bit or int(down["bit_width"]) != bit:
             raise ValueError(f"shared expert bit_width must be 1/2/4/8 and equal for gate/up/down, got {bit}")
@@ -274,6 +280,26 @@ class WxA16BitPartitionedGroupMoE:
             return MODE_A8
         return mode
 
+    # How the Linears of the shared expert run when the layer is switched to an activation-quantized
+    # mode: "wxa8" (the reference's default, also for wxfp8 / wxfp4 layers), "wxfp8" (its opt-in
+    # attn="wxfp8" of convert_model_to_wxfp8) or "wxa16".
+    shared_attn = "wxa8"
+
+    def shared_pool_mode(self, bw: "BitPoolWeights") -> int:
+        """Precision mode of the shared expert's pool.  The reference converts these Linears on
+        their own rule (qwen35_quant_io.py:416-532): a WxA16 layer keeps them fp16; the other
+        modes move an 8-bit Linear to int8 only when its codebook is the uniform grid (a Lloyd-Max
+        codebook would lose levels on the int8 grid) and never to fp8 unless asked to
+        (attn="wxfp8"); anything else stays on the fp16 path."""
+        mode = MODE_BY_NAME[self.MODE]
+        if mode == MODE_A16 or self.shared_attn == "wxa16" or bw.bit != 8:
+            return MODE_A16
+        if mode == MODE_FP8 and self.shared_attn == "wxfp8":
+            return MODE_FP8
+        uniform = hostprep.is_uniform_codebook(bw.gu_codebook.cpu()) and \
+            hostprep.is_uniform_codebook(bw.dn_codebook.cpu())
+        return MODE_A8 if uniform else MODE_A16
+
     def _descriptor(self):
         if self._desc is not None:
             return self._desc
@@ -292,7 +318,7 @@ class WxA16BitPartitionedGroupMoE:
                     start[pi, ex] = 2 * s
                     count[pi, ex] = 2 * (t - s)
                     members += 1
-            mode = self.pool_mode(bw.bit)
+            mode = self.shared_pool_mode(bw) if bit_str == self.SHARED_KEY else self.pool_mode(bw.bit)
             ctx = bw.context(mode)
             keep.append(ctx)
             d = pool_arr[pi]
@@ -317,7 +343,34 @@ class WxA16BitPartitionedGroupMoE:
         desc.experts, desc.top_k, desc.pools = e, top_k, n_pools
         desc.pool = ctypes.cast(pool_arr, ctypes.POINTER(PoolDesc))
         desc.slice_start, desc.slice_count = slice_start.data_ptr(), slice_count.data_ptr()
-        self._desc = (desc, pool_arr, slice_start, slice_count, keep)
+        # Sub-expert layers: per (pool, expert) the first column of the pool's share inside the
+        # expert's SiLU*up row (shares packed in pool order) and the rank of the pool among the
+        # expert's pools; the distinct share widths; the largest number of pools per expert.
+        widths_all = (count // 2)
+        homes_per_expert = (count > 0).sum(0)
+        sub = bool((homes_per_expert > 1).any()) or bool(((count > 0) & (widths_all != self.intermediate_size)).any())
+        col_start = home = None
+        if sub:
+            col = torch.zeros((n_pools, e), dtype=torch.int32)
+            rank = torch.zeros((n_pools, e), dtype=torch.int32)
+            run_col = torch.zeros(e, dtype=torch.int32)
+            run_rank = torch.zeros(e, dtype=torch.int32)
+            for pi in range(n_pools):
+                member = count[pi] > 0
+                col[pi] = torch.where(member, run_col, torch.zeros_like(run_col))
+                rank[pi] = torch.where(member, run_rank, torch.zeros_like(run_rank))
+                run_col = run_col + widths_all[pi]
+                run_rank = run_rank + member.int()
+            widths = sorted({int(v) for v in widths_all[count > 0].tolist()})
+            if len(widths) > 8:
+                raise ValueError(f"at most 8 distinct share widths per layer, got {widths}")
+            desc.n_widths = len(widths)
+            for i, w_ in enumerate(widths):
+                desc.widths[i] = w_
+            desc.max_homes = int(homes_per_expert.max())
+            col_start, home = col.to(self.device), rank.to(self.device)
+            desc.col_start, desc.home = col_start.data_ptr(), home.data_ptr()
+        self._desc = (desc, pool_arr, slice_start, slice_count, keep, col_start, home)
         return self._desc
 
     def _get_workspace(self, tokens: int) -> torch.Tensor:

@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 13). */
+/* Library / build identification: returns the ABI version (currently 14). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -209,6 +209,13 @@ typedef struct {
   int bit;                  /* index width of idx_gf (FP4 reads folded e2m1: pass the pool bit) */
   int mode;                 /* must equal the launch mode; other pools are skipped */
   int w_scale_byte;         /* FP4: 127 + E0 */
+  /* Layers whose experts are cut into sub-experts that live in several pools (width_filter of
+   * dmq_gemm_args != 0), both int32 [n_experts] in device memory, NULL = all zero:
+   * col_start: first column of this pool's share inside the expert's SiLU*up row (gate_up: where
+   * the launch writes; down: where it starts contracting); home: rank of this pool among the pools
+   * that hold a share of the expert. */
+  const void* col_start;
+  const void* home;
 } dmq_gemm_pool;
 
 typedef struct {
@@ -234,7 +241,7 @@ typedef struct {
   long out_stride;
   const void* row_weight;   /* SCATTER: fp32 routing weight per row */
   const void* row_slot;     /* SCATTER: int32 destination slot row per row */
-  void* dbg_acc;            /* A8, tt == 1, ks == 1, STORE only: int32 [rows, groups, n_out] or NULL */
+  void* dbg_acc;            /* A8, ks == 1, STORE only: int32 [rows, groups, n_out] or NULL */
   /* DMQ_EPI_SILU_ROT (ks == 1, n_out % 128 == 0): per pool the rotation matrices fp16
    * [groups_total, 128, 128] (the matrix of group g of an expert is post_rot[slice_g + g], slice_g
    * the expert's first down group = gate_up slice_start / 256) and the factor folded into the
@@ -270,6 +277,16 @@ typedef struct {
    * and the workgroup covers 16 features, so a 4096-feature matrix gives 256 workgroups), any bit
    * width, not WxFP4, not with k_split or dbg_acc; n_out a multiple of 16. */
   int nt;
+  /* Sub-expert layers (the reference's --slices checkpoints: an expert's neurons are spread over
+   * several bit pools, quantization/wxa16/bit_partitioned_moe.py:499-521; its output is the sum
+   * over its pools, :818-822).  A launch serves the shares of one width: work items whose
+   * expert_info slice_count differs from width_filter are skipped (0 = no filter); n_out /
+   * half_width / groups describe that width.  home_filter >= 0 further restricts the launch to the
+   * shares of that rank (the down projection runs rank after rank); accumulate != 0 makes
+   * DMQ_EPI_SCATTER add to the slot row instead of storing it (ranks above 0).  Not with k_split. */
+  int width_filter;
+  int home_filter;
+  int accumulate;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more
@@ -365,7 +382,16 @@ typedef struct {
   int hidden, inter, experts, top_k, pools;    /* pools <= DMQ_MAX_POOLS */
   const dmq_pool_desc* pool;      /* host array [pools] */
   const void* slice_start;        /* device int32 [pools, experts] (2*start or -1) */
-  const void* slice_count;        /* device int32 [pools, experts] (2*I) */
+  const void* slice_count;        /* device int32 [pools, experts] (2*width of the pool's share) */
+  /* Sub-expert layers (experts spread over several pools, shares of different widths): n_widths > 0
+   * lists the distinct share widths (multiples of 128, at most 8), max_homes the largest number of
+   * pools one expert lives in, col_start / home device int32 [pools, experts] as in dmq_gemm_pool.
+   * n_widths == 0: every expert lives in exactly one pool with width `inter`. */
+  int n_widths;
+  int widths[8];
+  int max_homes;
+  const void* col_start;
+  const void* home;
 } dmq_layer_desc;
 
 /* Bytes of workspace dmq_moe_ffn_forward needs for `tokens` tokens. */
@@ -375,7 +401,7 @@ size_t dmq_moe_workspace_bytes(const dmq_layer_desc* layer, int tokens);
  * and its WxA8 / WxFP8 / WxFP4 subclasses, routed experts only:
  *   x fp16 [tokens, hidden]; topk_idx int32 / topk_w fp32 [tokens, top_k];
  *   out fp16 [tokens, hidden] = sum_k w * down_e(silu(gate_e(x)) * up_e(x)) (+ add_f16).
- * Every expert must belong to exactly one pool.  tt <= 0 / ks == 0 / nbl <= 0 pick the tiling
+ * tt <= 0 / ks == 0 / nbl <= 0 pick the tiling
  * (rows per tile, K split, feature blocks per workgroup) from tokens.  ks > 0 splits K over the
  * waves of a workgroup (1 or 4); ks = -2 / -4 shares the K range of the gate_up GEMM between
  * that many workgroups instead (k_split of dmq_gemm_args: tt == 1, at most 1024 routed rows). */

@@ -118,11 +118,13 @@ def test_merged_in_features_down(mode, bit):
     torch.testing.assert_close(out, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
 
 
+@pytest.mark.parametrize("tt", [1, 2, 4])
 @pytest.mark.parametrize("bit", [1, 2, 4])
-def test_wxa8_int32_accumulators_exact(bit):
-    """Per-group int32 accumulators of the i8 matrix cores equal an int64 numpy matmul."""
+def test_wxa8_int32_accumulators_exact(bit, tt):
+    """Per-group int32 accumulators of the i8 matrix cores equal an int64 numpy matmul, in the
+    16-, 32- and 64-row kernels (the last two serve the prefill batches); full-range int8 codes."""
     from dartmoq_hip import ops
-    counts = [7, 20, 1]
+    counts = [7, 20, 1, 70, 0, 130]
     k, n_slice = 384, 128
     starts, rows_total = _expert_rows(counts)
     idx_gf, norms_gf, cb = _pool(bit, n_slice * len(counts), k, 300 + bit)
@@ -133,10 +135,12 @@ def test_wxa8_int32_accumulators_exact(bit):
     dbg = torch.zeros(rows_total, k // 128, n_slice, dtype=torch.int32, device="cuda")
     ops.matmul_merged(A8, bit, STORE, codes.cuda(), s.half().cuda(), idx_gf.cuda(), norms_gf.cuda(),
                       q_lut.cuda(), torch.tensor(info, dtype=torch.int32).cuda(), groups=k // 128,
-                      n_out=n_slice, slice_is_groups=False, rows_total=rows_total, tt=1, ks=1, dbg_acc=dbg)
+                      n_out=n_slice, slice_is_groups=False, rows_total=rows_total, tt=tt, ks=1, dbg_acc=dbg)
     torch.cuda.synchronize()
     w = q_lut.long()[packing.unpack_nbit(idx_gf, bit, 128).long()]          # [G, N, 128]
     for e, (ts, cnt, ss, sc) in enumerate(info):
+        if cnt == 0:
+            continue
         a = codes[ts:ts + cnt].long().reshape(cnt, k // 128, 128)
         ref = torch.einsum("bgk,gnk->bgn", a, w[:, ss:ss + sc])
         assert torch.equal(dbg[ts:ts + cnt].cpu().long(), ref)

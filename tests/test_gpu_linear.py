@@ -234,6 +234,36 @@ def test_int8_gemm_of_uniform_8bit_weights():
     assert torch.equal(out, ops.linear_gemm_i8(x_i8, x_s, idx_gf, norms_pre))
 
 
+def test_int8_gemm_exact_integers():
+    """dmq_linear_gemm_i8 on operands whose result is an exact small integer: activation codes in
+    [-3, 3], weights idx - 128 in [-2, 2], unit scales and norms.  Every group sum is an int32 the
+    matrix cores must deliver exactly, their fp32 scaling and sum are exact, and the fp16 store of
+    an integer below 2048 is exact, so the output must equal an int64 matmul bit for bit (ragged
+    shape: partial tiles in rows and features)."""
+    from dartmoq_hip import ops
+    rows, k, n = 203, 384, 200
+    g = torch.Generator().manual_seed(11)
+    x = torch.randint(-3, 4, (rows, k), generator=g, dtype=torch.int8)
+    w = torch.randint(-2, 3, (n, k), generator=g, dtype=torch.int64)
+    idx_gf = (w + 128).to(torch.uint8).reshape(n, k // 128, 128).permute(1, 0, 2).contiguous()
+    ones_s = torch.ones(rows, k // 128, dtype=torch.float16)
+    ones_n = torch.ones(k // 128, n, dtype=torch.float16)
+    out = ops.linear_gemm_i8(x.cuda(), ones_s.cuda(), idx_gf.cuda(), ones_n.cuda())
+    ref = x.long() @ w.t()
+    assert ref.abs().max() < 2048 and ref.abs().max() > 100
+    assert torch.equal(out.cpu().long(), ref)
+    # power-of-two scales and norms keep everything exact: the scale and norm factors reach the
+    # right row and feature
+    s2 = (2.0 ** torch.randint(-2, 3, (rows, k // 128), generator=g)).half()
+    n2 = (2.0 ** torch.randint(-3, 2, (k // 128, n), generator=g)).half()
+    out2 = ops.linear_gemm_i8(x.cuda(), s2.cuda(), idx_gf.cuda(), n2.cuda()).cpu()
+    xg = x.double().reshape(rows, k // 128, 128)
+    wg = w.double().reshape(n, k // 128, 128)
+    ref2 = torch.einsum("rgk,ngk,rg,gn->rn", xg, wg, s2.double(), n2.double())
+    # the scaled sums (multiples of 2^-5 below 2^14) are exact in fp32; the fp16 store rounds once
+    assert torch.equal(out2, ref2.float().half())
+
+
 # ----------------------------------------------------------------------------- 8-bit codebooks
 
 def _packed8(n, k, seed, uniform):

@@ -138,6 +138,36 @@ def test_layer_with_8bit_shared_expert(small_layer, mode, tokens):
     assert relerr(out, ref) < MODE_BOUND[mode], (mode, relerr(out, ref))
 
 
+@pytest.mark.parametrize("mode", ["wxa8", "wxfp8", "wxfp4"])
+def test_lloydmax_8bit_shared_expert_stays_on_the_fp16_path(small_layer, mode):
+    """An 8-bit shared expert with a Lloyd-Max codebook cannot go to int8 (it would lose levels on
+    the int8 grid): like the reference's convert_model_to_wxa8 / _wxfp8 / _wxfp4
+    (qwen35_quant_io.py:416-532) the layer keeps it on the fp16 path, whatever its own mode."""
+    import dataclasses
+    from dartmoq_hip._lib import MODE_A16, MODE_A8, MODE_FP8
+    layer = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter,
+                                  seed=33, bit=8, uniform_codebook=False)
+    x, idx, w, out = _run(layer, mode, 40, seed=21)
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    tight = {"wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+    mod = make_module(layer, mode)
+    assert mod.shared_pool_mode(mod.bit_weights[mod.SHARED_KEY]) == MODE_A16
+    # the uniform grid moves to int8 in every activation-quantized mode, to fp8 only when asked
+    uni = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter,
+                                seed=31, bit=8, uniform_codebook=True)
+    mu = make_module(uni, mode)
+    assert mu.shared_pool_mode(mu.bit_weights[mu.SHARED_KEY]) == MODE_A8
+    if mode == "wxfp8":
+        mu.shared_attn = "wxfp8"
+        assert mu.shared_pool_mode(mu.bit_weights[mu.SHARED_KEY]) == MODE_FP8
+        mu._desc = None
+        xs = x.cuda()
+        o8 = mu.forward(xs, topk_idx=idx.int().cuda(), topk_w=w.cuda()).float().cpu()
+        ideal8 = moe.quantized_forward_with_attn(uni, x, idx, w, mode, "wxfp8")
+        assert relerr(o8, ideal8) < 2e-2
+
+
 def dataclasses_replace_shared(layer):
     import dataclasses
     return dataclasses.replace(layer, shared=None)
@@ -175,10 +205,54 @@ def test_shared_expert_from_logits_and_gate_columns(shared_layer):
 
 def test_shared_expert_shape_errors(small_layer):
     import dataclasses
-    bad = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter + 128,
-                                seed=3)
+    bad = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter, seed=3)
+    wrong = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter + 128,
+                                  seed=3)
+    bad.shared = dict(bad.shared, up=wrong.shared["up"])          # up [I + 128, H] beside gate [I, H]
     with pytest.raises(ValueError):
         make_module(bad, "wxa16")
+
+
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp4"])
+def test_shared_expert_width_not_a_multiple_of_the_routed_width(small_layer, mode):
+    """I_s = I + 128: the shared expert is cut into 128-wide slices, the layer runs with shares of
+    two widths (one gate_up launch per width)."""
+    import dataclasses
+    layer = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter + 128,
+                                  seed=3)
+    x, idx, w, out = _run(layer, mode, 40, seed=8)
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+
+
+@pytest.fixture(scope="module", params=["421+shared", "842"])
+def sliced_layer(request):
+    """12 experts, H=256, I=512, top-3: experts whole in one pool, cut in two (128 + 384,
+    256 + 256) and in three (128 + 256 + 128).  Either 4/2/1-bit pools plus a 4-bit shared expert
+    of 640 neurons (five 128-wide slices), or 8/4/2-bit pools (the 8-bit pool keeps the rotation
+    of the down input a launch of its own)."""
+    if request.param == "421+shared":
+        shapes = [{4: 512}, {4: 128, 2: 384}, {2: 256, 1: 256}, {4: 128, 2: 256, 1: 128}, {1: 512}]
+    else:
+        shapes = [{4: 512}, {8: 128, 2: 384}, {8: 256, 4: 256}, {8: 128, 4: 256, 2: 128}, {2: 512}]
+    layer = moe.build_sliced_layer(256, 512, 12, 3, [shapes[e % len(shapes)] for e in range(12)], seed=9)
+    return moe.add_shared_expert(layer, 640, seed=4) if request.param == "421+shared" else layer
+
+
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
+@pytest.mark.parametrize("tokens,tt", [(1, 0), (50, 0), (50, 2), (400, 2), (400, 4)])
+def test_sub_expert_layer_matches_oracles(sliced_layer, mode, tokens, tt):
+    """Experts spread over several bit pools (the reference's --slices layout): the output of an
+    expert is the sum over its pools."""
+    if "8" in sliced_layer.pools and mode in ("wxa8", "wxfp4"):
+        pytest.skip("a Lloyd-Max 8-bit pool has no int8 form (int8 takes the uniform 8-bit grid only)")
+    x, idx, w, out = _run(sliced_layer, mode, tokens, seed=tokens, tt=tt)
+    ideal = moe.quantized_forward(sliced_layer, x, idx, w, mode)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+    ref = moe.reference_forward(sliced_layer, x, idx, w)
+    assert relerr(out, ref) < MODE_BOUND[mode], (mode, relerr(out, ref))
 
 
 def test_cpu_input_fails_loudly(small_layer):

@@ -113,3 +113,126 @@ def test_loaded_layer_equals_in_memory_layer(tmp_path, shared_layer, mode):
     y = loaded.forward(x)
     ref_logits = (x @ gate.cuda().t())
     assert torch.equal(y, direct.forward(x, router_logits=ref_logits))
+
+
+# ----------------------------------------------------------------------------- reference-written fixture
+# tests/golden/ckpt_tiny was written by the reference's save_quantized_model over a tiny model
+# assembled from the reference's classes (tests/golden/make_ckpt_fixture.py); expected.json holds
+# outputs computed with the reference's own CPU dequantizers.
+
+CKPT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ckpt_tiny")
+FIX_LAYERS = ("model.layers.0.mlp", "model.layers.1.mlp")
+
+
+def _fixture_case(path):
+    exp = json.load(open(os.path.join(CKPT, "expected.json")))[path]
+    x = torch.tensor(exp["x_fp16_bits"], dtype=torch.int16).view(torch.float16).reshape(4, -1)
+    return (x, torch.tensor(exp["topk_idx"]), torch.tensor(exp["topk_w"], dtype=torch.float32),
+            torch.tensor(exp["y_routed"]), torch.tensor(exp["y_shared"]))
+
+
+def _oracle_layer(d):
+    layer = moe.MoELayer(d["hidden_size"], d["intermediate_size"], d["num_experts"], d["top_k"], 128)
+    for b, p in d["pools"].items():
+        layer.pools[b] = moe.BitPool(int(b), p["gate_up"], p["down"], p["expert_offsets"])
+    layer.shared = d["shared_expert"]
+    return layer
+
+
+def test_reads_checkpoint_written_by_the_reference():
+    from safetensors import safe_open
+    from dartmoq_hip import checkpoint
+    assert checkpoint.list_layers(CKPT) == list(FIX_LAYERS)
+    meta = json.load(open(os.path.join(CKPT, "meta.json")))
+    raw = safe_open(os.path.join(CKPT, "model.safetensors"), framework="pt", device="cpu")
+    for path in FIX_LAYERS:
+        d = checkpoint.read_layer(CKPT, path)
+        lm = meta["layers"][path]
+        assert (d["num_experts"], d["hidden_size"], d["top_k"]) == (4, 256, 2)
+        assert d["intermediate_size"] == lm["intermediate_size"]
+        assert list(d["pools"]) == [str(b) for b in lm["bit_list"]] == ["4", "2"]
+        for b, p in d["pools"].items():
+            assert p["expert_offsets"] == lm["expert_offsets"][b]
+            for which in ("gate_up", "down"):
+                assert p[which]["seed"] == 42 + int(b) + (1000 if which == "down" else 0)
+                assert p[which]["bit_width"] == int(b) and p[which]["group_size"] == 128
+                for k in ("indices_packed", "codebook", "norms"):
+                    assert torch.equal(p[which][k], raw.get_tensor(f"{path}.bit_weights.{b}.{which}_{k}"))
+            total = p["expert_offsets"][-1]
+            assert tuple(p["gate_up"]["shape"]) == (2 * total, 256)
+            assert tuple(p["down"]["shape"]) == (256, total)
+        assert torch.equal(d["gate_weight"], raw.get_tensor(f"{path}.gate.weight"))
+        sh = d["shared_expert"]
+        assert sh["gate"]["bit_width"] == (4 if path.endswith("0.mlp") else 8)
+        assert sh["down"]["codebook_type"] == ("lloydmax" if path.endswith("0.mlp") else "uniform")
+        assert torch.equal(sh["gate_row"], raw.get_tensor(f"{path}.shared_expert_gate.weight"))
+    # layer 1 is the --slices 2 layout: experts 0 and 2 live in both pools
+    offs = checkpoint.read_layer(CKPT, FIX_LAYERS[1])["pools"]
+    homes = [sum(1 for p in offs.values() if p["expert_offsets"][e + 1] > p["expert_offsets"][e])
+             for e in range(4)]
+    assert homes == [2, 1, 2, 1]
+
+
+@pytest.mark.parametrize("path", FIX_LAYERS)
+def test_oracle_on_reference_checkpoint_matches_reference_dequant_outputs(path):
+    """The oracle's dequantize-then-matmul forward over the tensors the reader returns equals what
+    the reference's own dequantizers give (routed part incl. the sum over the pools of a split
+    expert, and the gated shared expert)."""
+    from dartmoq_hip import checkpoint
+    layer = _oracle_layer(checkpoint.read_layer(CKPT, path))
+    x, idx, w, y_routed, y_shared = _fixture_case(path)
+    shared = layer.shared
+    layer.shared = None
+    routed = moe.reference_forward(layer, x, idx, w)
+    # the reference's dequantizers return the weight dtype (fp16: one rounding per weight, relative
+    # 2^-11), the oracle keeps fp32
+    from tests.helpers import relerr
+    assert relerr(routed, y_routed) < 5e-4
+    layer.shared = shared
+    assert relerr(moe.shared_expert_forward(layer, x.float()), y_shared) < 5e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
+@pytest.mark.parametrize("path", FIX_LAYERS)
+def test_gpu_forward_of_reference_checkpoint(path, mode):
+    """load_moe_layer on the reference-written checkpoint, router's own top-k handed over: output
+    against the reference-dequantizer expectation (fp32) within the mode's error."""
+    from dartmoq_hip import checkpoint
+    from tests.helpers import relerr
+    bound = {"wxa16": 2e-3, "wxa8": 0.03, "wxfp8": 0.09, "wxfp4": 0.35}[mode]
+    mod = checkpoint.load_moe_layer(CKPT, path, mode=mode)
+    x, idx, w, y_routed, y_shared = _fixture_case(path)
+    out = mod.forward(x.cuda(), topk_idx=idx.int().cuda(), topk_w=w.cuda()).float().cpu()
+    want = y_routed + y_shared
+    assert relerr(out, want) < bound, (mode, relerr(out, want))
+    # and the router weight of the checkpoint reproduces that top-k
+    out2 = mod.forward(x.cuda()).float().cpu()
+    assert relerr(out2, want) < bound
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
+@pytest.mark.parametrize("tokens,tt", [(1, 0), (37, 0), (300, 2), (300, 4)])
+def test_gpu_sub_expert_layer_matches_dataflow_oracle(mode, tokens, tt):
+    """model.layers.1.mlp of the fixture (experts cut into sub-experts over two pools, an 8-bit
+    uniform shared expert narrower than the routed experts) at several batch sizes and tilings,
+    against the oracle's kernel-dataflow forward on the tensors the reader returns."""
+    from dartmoq_hip import checkpoint
+    from tests.helpers import relerr
+    d = checkpoint.read_layer(CKPT, FIX_LAYERS[1])
+    layer = _oracle_layer(d)
+    mod = checkpoint.load_moe_layer(CKPT, FIX_LAYERS[1], mode=mode)
+    mod.tt_override = tt
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(tokens, layer.hidden, generator=g).half()
+    w, idx = routing.route_topk(routing.zipf_logits(tokens, layer.num_experts, tokens), layer.top_k)
+    out = mod.forward(x.cuda(), topk_idx=idx.int().cuda(), topk_w=w.cuda()).float().cpu()
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+    # splitting the batch leaves every row unchanged
+    if tokens > 100:
+        a = mod.forward(x[:111].cuda(), topk_idx=idx[:111].int().cuda(), topk_w=w[:111].cuda())
+        b = mod.forward(x[111:].cuda(), topk_idx=idx[111:].int().cuda(), topk_w=w[111:].cuda())
+        assert torch.equal(torch.cat([a, b]).float().cpu(), out)

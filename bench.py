@@ -11,8 +11,13 @@ the timed region starts.  The 2 bpw layer (~216 MB packed) fits in the 256 MB In
 the steps rotate through three independent copies of the layer.
 
 Defaults: 50 untimed warm-up steps and 500 timed ones (about 0.15 s of GPU work).  The GPU takes
-tens of milliseconds of sustained load to reach its working clocks: 30 steps after 5 warm-up
-steps read 0.26 ms per step on the same box that settles at 0.226 ms from 200 steps on.
+tens of milliseconds of sustained load to reach its working clocks, so every measurement starts
+with an untimed prelude of fixed length (`clock_prelude_s` in the JSON) of the same forwards:
+short and long runs then read the same time per step.
+
+`modes` holds the activation-quantized modes on the configurations named for them (configs[2]
+WxA8, configs[4] WxFP8 and WxFP4; the all-4-bit layer, uniform routing) at 2048 and 64 tokens, each
+with the roofline of its gate_up launch; `sweep` the decode sizes of the main configuration.
 
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the gate_up dequant-GEMM of the
 largest bit pool, which also rotates its output rows for the down projection), timed live with
@@ -55,9 +60,29 @@ def layer_bytes(mod, counts):
     return total, per_pool
 
 
+PRELUDE_S = 0.5
+
+
+def settle_clocks(mods, x, logits, seconds):
+    """Untimed load of fixed duration before a measurement: the GPU needs tens of milliseconds of
+    sustained work to reach its working clocks (and drops them again while the host is busy), so
+    without it a 20-step run reads 15 % slower than a 500-step run of the same thing."""
+    import torch
+    n = len(mods)
+    t0 = time.perf_counter()
+    s = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            mods[s % n].forward(x, router_logits=logits)
+            s += 1
+        torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
 def time_steps(mods, x, logits, steps, warmup):
     import torch
     n = len(mods)
+    settle_clocks(mods, x, logits, PRELUDE_S)
     for s in range(warmup):
         mods[s % n].forward(x, router_logits=logits)
     torch.cuda.synchronize()
@@ -158,8 +183,26 @@ def measured_traffic(config, mode, tokens):
     return None
 
 
-def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf, shared_cpu=None):
-    """The CPU oracle (dequantize per call, fp32 matmuls) on a bounded sample of the workload."""
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    return ln.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf, shared_cpu=None, warm=2, timed=5,
+                 budget_s=30.0):
+    """The CPU oracle (dequantize-then-matmul, fp32 matmuls, all host threads) on the same seeded
+    inputs as the GPU run at `tokens` tokens, the two variants of the reference's benchmark script
+    (test_triton_mp_moe_e2e_bench.py:135-164): weights dequantized once before the timed calls
+    ("cached") and dequantized inside every call ("per_call").  Each: `warm` untimed calls, then
+    `timed` calls, median.  `value` is the cached variant (the faster one).  The per-call variant
+    stops early (at least 3 timed calls) when its calls would pass `budget_s` seconds."""
+    import statistics
     import torch
     from oracle import moe as omoe, routing
     layer = omoe.MoELayer(spec["hidden"], spec["inter"], spec["experts"], spec["top_k"], 128,
@@ -167,17 +210,41 @@ def cpu_baseline(pools_cpu, spec, expert_bit, tokens, seed, zipf, shared_cpu=Non
     for b, p in pools_cpu.items():
         layer.pools[b] = omoe.BitPool(int(b), p["gate_up"], p["down"], p["expert_offsets"])
     layer.shared = shared_cpu
-    torch.set_num_threads(os.cpu_count() or 1)
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
     x = torch.randn(tokens, spec["hidden"], generator=torch.Generator().manual_seed(seed)).half()
     w, idx = routing.route_topk(routing.zipf_logits(tokens, spec["experts"], seed, skew=zipf),
                                 spec["top_k"])
+
+    def run(cache, n_warm, n_timed, budget):
+        times = []
+        t_start = time.perf_counter()
+        for i in range(n_warm + n_timed):
+            t0 = time.perf_counter()
+            omoe.reference_forward(layer, x, idx, w, weight_cache=cache)
+            dt = time.perf_counter() - t0
+            if i >= n_warm:
+                times.append(dt)
+            if budget and len(times) >= 3 and time.perf_counter() - t_start + dt > budget:
+                break
+        return statistics.median(times), len(times)
+
     t0 = time.perf_counter()
-    omoe.reference_forward(layer, x, idx, w)
-    sec = time.perf_counter() - t0
-    return {"value": tokens / sec, "unit": "tokens/s", "cores": torch.get_num_threads(),
-            "kind": "port", "seconds": sec,
-            "sample": f"one forward of {tokens} tokens of the same layer, dequantize-per-call "
-                      f"fp32 oracle (reference_forward), {torch.get_num_threads()} threads"}
+    cache = omoe.build_weight_cache(layer)
+    build_s = time.perf_counter() - t0
+    cached_s, cached_n = run(cache, warm, timed, 0.0)
+    del cache
+    per_call_s, per_call_n = run(None, warm, timed, budget_s)
+    return {"value": tokens / cached_s, "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port", "cpu_model": cpu_model_name(), "tokens": tokens,
+            "cached": {"tokens_per_s": tokens / cached_s, "median_s": cached_s, "timed_calls": cached_n,
+                       "warmup_calls": warm, "dequantize_once_s": build_s},
+            "per_call": {"tokens_per_s": tokens / per_call_s, "median_s": per_call_s,
+                         "timed_calls": per_call_n, "warmup_calls": warm},
+            "sample": f"forwards of {tokens} tokens of the same layer and the same seeded inputs as the "
+                      f"GPU sweep entry, fp32 dequantize-then-matmul oracle (reference_forward), "
+                      f"{torch.get_num_threads()} threads; value = weights dequantized once (cached), "
+                      f"per_call = dequantized inside every call; median of the timed calls"}
 
 
 def bench_linear(spec, steps, warmup, seed):
@@ -233,8 +300,11 @@ def main():
     ap.add_argument("--config", type=int, default=1)
     ap.add_argument("--mode", type=str, default="wxa16", choices=list(MFMA_PEAK))
     ap.add_argument("--seed", type=int, default=42)
-    ap.add_argument("--cpu-tokens", type=int, default=16)
+    ap.add_argument("--cpu-tokens", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--modes", type=str, default="2:wxa8:2048/64,4:wxfp8:2048/64,4:wxfp4:2048/64",
+                    help='extra entries of the "modes" array, "config:mode:tokens[/tokens...]" comma '
+                         'separated ("" for none)')
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch dmq_finalize_kernel on 64 Mi fp32 elements (256 MiB read, "
                          "128 MiB written): the known-size kernel that calibrates FETCH_SIZE / "
@@ -258,19 +328,36 @@ def main():
         bench_linear(args.linear, args.steps, args.warmup, args.seed)
         return
     spec = synthetic.CONFIGS[args.config]
-    expert_bit = synthetic.assign_bits(spec["experts"], spec["fractions"], args.seed)
-    pools = synthetic.build_pools(spec["hidden"], spec["inter"], spec["experts"], expert_bit,
-                                  seed=args.seed, device="cuda")
-    shared = None
-    if spec.get("shared_inter"):
-        shared = synthetic.build_shared_expert(spec["hidden"], spec["shared_inter"], args.seed,
-                                               spec.get("shared_bit", 4), device="cuda")
-    mods = []
-    for _ in range(N_COPIES):
-        m = dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
-            pools, spec["experts"], spec["hidden"], spec["inter"], spec["top_k"], device="cuda",
-            shared_expert=shared)
-        mods.append(dartmoq_hip.convert_moe(m, args.mode))
+    layers = {}
+
+    def build(cfg):
+        """Packed pools (and shared expert) of a config; configs with the same layer share them."""
+        sp = synthetic.CONFIGS[cfg]
+        key = json.dumps({k: v for k, v in sp.items() if k != "zipf"}, sort_keys=True)
+        if key not in layers:
+            eb = synthetic.assign_bits(sp["experts"], sp["fractions"], args.seed)
+            pl = synthetic.build_pools(sp["hidden"], sp["inter"], sp["experts"], eb, seed=args.seed,
+                                       device="cuda")
+            sh = None
+            if sp.get("shared_inter"):
+                sh = synthetic.build_shared_expert(sp["hidden"], sp["shared_inter"], args.seed,
+                                                   sp.get("shared_bit", 4), device="cuda")
+            layers[key] = (eb, pl, sh)
+        return layers[key]
+
+    def modules(cfg, mode):
+        sp = synthetic.CONFIGS[cfg]
+        _eb, pl, sh = build(cfg)
+        out = []
+        for _ in range(N_COPIES):
+            m = dartmoq_hip.WxA16BitPartitionedGroupMoE.from_packed(
+                pl, sp["experts"], sp["hidden"], sp["inter"], sp["top_k"], device="cuda",
+                shared_expert=sh)
+            out.append(dartmoq_hip.convert_moe(m, mode))
+        return out
+
+    expert_bit, pools, shared = build(args.config)
+    mods = modules(args.config, args.mode)
 
     if args.traffic_probe:
         from dartmoq_hip import ops
@@ -288,8 +375,29 @@ def main():
         if t == args.tokens:
             continue
         res, r = measure(mods, t, args.steps, args.warmup, args.seed, spec["zipf"], args.mode)
+        r["traffic"] = measured_traffic(args.config, args.mode, t)
         res["roofline"] = r
         sweep.append(res)
+    del mods
+
+    # the activation-quantized modes on the configurations BASELINE names for them
+    mode_results = []
+    for entry in [v for v in args.modes.split(",") if v]:
+        cfg_s, mode_s, tok_s = entry.split(":")
+        cfg_m = int(cfg_s)
+        sp = synthetic.CONFIGS[cfg_m]
+        mm = modules(cfg_m, mode_s)
+        for t in [int(v) for v in tok_s.split("/")]:
+            res, r = measure(mm, t, args.steps, args.warmup, args.seed, sp["zipf"], mode_s)
+            r["traffic"] = measured_traffic(cfg_m, mode_s, t)
+            mode_results.append({"config": cfg_m, "mode": mode_s, "dtype": DTYPE[mode_s], "tokens": t,
+                                 "value": res["tokens_per_s"], "unit": "tokens/s",
+                                 "ms_per_step": res["ms_per_step"], "eff_tflops": res["eff_tflops"],
+                                 "layer_hbm_frac": res["layer_hbm_frac"],
+                                 "layer_mfma_frac": res["layer_mfma_frac"],
+                                 "gpu_stage_ms": res["gpu_stage_ms"], "roofline": r})
+        del mm
+        torch.cuda.empty_cache()
 
     cpu = None
     if not args.no_cpu:
@@ -325,6 +433,8 @@ def main():
         "roofline": roof,
         "cpu_baseline": cpu,
         "sweep": sweep,
+        "modes": mode_results,
+        "clock_prelude_s": PRELUDE_S,
     }
     print(json.dumps(line))
 

@@ -39,18 +39,10 @@ static inline int pick_ks(int tt, long rows, int groups) {
 #define DMQ_SPLIT_MAX_ROWS 1024
 // single-block workgroups at the end of every XCD's share of a GEMM launch that otherwise walks
 // several blocks per workgroup: one round of resident workgroups (32 CUs x 3)
-#ifndef DMQ_DOWN_TT4_MIN_AVG
 #define DMQ_DOWN_TT4_MIN_AVG 512
-#endif
-#ifndef DMQ_TT4_MIN_AVG
 #define DMQ_TT4_MIN_AVG 112
-#endif
-#ifndef DMQ_HOIST_ALL_TOKENS
 #define DMQ_HOIST_ALL_TOKENS 1024
-#endif
-#ifndef DMQ_TAIL_SLOTS
 #define DMQ_TAIL_SLOTS 96
-#endif
 
 // Feature blocks one workgroup walks back to back.  With few row tiles every block gets its own
 // workgroup (parallelism); with many, a workgroup amortizes its start-up over several blocks.
@@ -560,9 +552,7 @@ int dmq_linear_gemm_i8(const void* x_i8, long x_row_bytes, const void* x_scale_f
 // the plain int8 GEMM instead of the look-up kernels.  4096 x 4096, forward time: 2048 rows
 // 146 -> 80 us, 4096 rows 290 -> 150 us, 768 rows 79 -> 61 us; with fewer tiles (640 rows: 160)
 // the 32-row look-up tiles win.
-#ifndef DMQ_LINEAR_I8_MIN_WGS
 #define DMQ_LINEAR_I8_MIN_WGS 192
-#endif
 static bool linear_uses_i8_gemm(const dmq_linear_desc* L, int rows) {
   if (L->mode != DMQ_MODE_A8 || L->bit != 8 || L->lut) return false;
   const long wgs = (long)((L->out_features + 127) / 128) * ((rows + 127) / 128);

@@ -32,24 +32,6 @@
 #include <type_traits>
 #include "lut.h"
 
-#ifdef DMQ_TRACE
-static __device__ long long dmq_trace_buf[256];
-#define DMQ_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x == 0) { \
-    dmq_trace_buf[2 * (i)] = __builtin_readcyclecounter(); \
-    dmq_trace_buf[2 * (i) + 1] = wall_clock64(); } } while (0)
-// per-workgroup wall-clock stamps (100 MHz): [0] entry, [1] table ready, [2] exit, [3] hardware id
-#define DMQ_WG_SLOTS 8192
-#ifndef DMQ_TRACE_EPI
-#define DMQ_TRACE_EPI DMQ_EPI_SILU
-#endif
-static __device__ long long dmq_wg_buf[DMQ_WG_SLOTS * 4];
-#define DMQ_WG_MARK(i) do { if (EPI == DMQ_TRACE_EPI && threadIdx.x == 0 && blockIdx.x < DMQ_WG_SLOTS) { \
-    dmq_wg_buf[blockIdx.x * 4 + (i)] = wall_clock64(); \
-    if ((i) == 0) dmq_wg_buf[blockIdx.x * 4 + 3] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)); } } while (0)
-#else
-#define DMQ_MARK(i)
-#define DMQ_WG_MARK(i)
-#endif
 
 struct PoolW {
   const uint8_t* w;            // [G_total, n_total, ppg] packed indices (FP4: folded e2m1, ppg = 64)
@@ -197,27 +179,12 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
 // weights.  Rings of 8 words (16-row tiles) and 4 words (32-row tiles) keep three resp. two
 // workgroups resident per CU; deeper rings cost a workgroup of occupancy and measured slower.
 #define DMQ_XCDS 8          // accelerator dies of an MI355X; the grid is a multiple of it
-#ifndef DMQ_SCHED
-#define DMQ_SCHED 1
-#endif
-#ifndef DMQ_KOUT
 #define DMQ_KOUT 1
-#endif
-#ifndef DMQ_KOUT_MIN_TT
 #define DMQ_KOUT_MIN_TT 2
-#endif
-#ifndef DMQ_FOLD_MIN_TT
 #define DMQ_FOLD_MIN_TT 2
-#endif
-#ifndef DMQ_RING_TT1
 #define DMQ_RING_TT1 8
-#endif
-#ifndef DMQ_RING_TT2
 #define DMQ_RING_TT2 4
-#endif
-#ifndef DMQ_RING_TT4
 #define DMQ_RING_TT4 4
-#endif
 template <int WW, int TT> constexpr int dmq_ring_depth() {
   constexpr int words = (TT == 1) ? DMQ_RING_TT1 : (TT == 2 ? DMQ_RING_TT2 : DMQ_RING_TT4);
   constexpr int d = words / WW;                     // words of packed weights per n-tile in flight
@@ -382,7 +349,6 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
                      const uint32_t (&xa)[TT][AW], const float (&xs)[TT], const int (&xsb)[TT]) {
     uint32_t wqb[2][WQ];
     dequant_tile(pk[0], wqb[0]);
-#if DMQ_SCHED
     if constexpr (FOLD) {
       // Explicit software pipeline, one fence per MFMA step: scale this step's operand, issue a
       // quarter of the next tile's look-ups, then the TT matrix instructions of the step.  The
@@ -413,7 +379,6 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       }
       return;
     }
-#endif
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       if (j + 1 < NT) dequant_tile(pk[j + 1], wqb[(j + 1) & 1]);
@@ -882,6 +847,16 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     // The planes are written and read with device-scope accesses, which go past the per-XCD L2
     // on their own: no cache-wide write-back or invalidate, only a wait for this wave's stores
     // to be acknowledged before the workgroup takes its ticket.
+    // Ordering without a release / acquire pair on the ticket: (1) every plane store is a
+    // device-scope store, performed at the memory side, and s_waitcnt vmcnt(0) returns only once
+    // each of this wave's stores has been acknowledged from there (stores count in vmcnt on this
+    // target); (2) the workgroup barrier orders all waves' waits before thread 0's ticket
+    // increment; (3) the increment is performed at the same memory side, so the workgroup that
+    // reads nsplit - 1 from it runs after all those acknowledgements; (4) its plane loads are
+    // device-scope loads issued after the barrier that publishes the ticket value, and are
+    // served from the memory side, never from a stale line of its own L2.  A release increment
+    // and acquire read (an L2 write-back and invalidate per workgroup) measured 1-3 us slower
+    // per layer at 1-16 tokens and changes no result.
     auto split_gather = [&](int nsplit_) -> bool {
       using u64 = unsigned long long;
       // one plane row holds the sums of a routed row: gate then up features (SiLU epilogues) or
@@ -972,13 +947,9 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       load_packed(lk, g_first + lg, pkb[u]);
       next_load();
     }
-    DMQ_MARK(1);
     if constexpr (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_store_wave<BIT, T::ES>(tbl, wave, lutw);
-    DMQ_MARK(2);
     stage_store(0, srb[0]);
     __syncthreads();
-    DMQ_MARK(3);
-    DMQ_WG_MARK(1);
     int cg = 0;                                        // group of the step being computed
     for (int sb = 0; sb < steps; sb += D) {
 #pragma unroll
@@ -1015,7 +986,6 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
           feat_k += FPB;
         }
         __syncthreads();
-        DMQ_MARK(4 + sb + u);
       }
     }
   }
@@ -1053,8 +1023,6 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     }
   }
   if constexpr (!STAGE) epilogue();
-  DMQ_MARK(120);
-  DMQ_WG_MARK(2);
 }
 
 // Waves per SIMD the register allocation aims for: three for tiles up to 32 rows (the 32-row
@@ -1069,15 +1037,9 @@ template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
-#ifndef DMQ_LDS_PAD
-#define DMQ_LDS_PAD 0
-#endif
-  __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2 + DMQ_LDS_PAD];
+  __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2];
   __shared__ __attribute__((aligned(16))) uint8_t smem_post[PostGeom<MODE, TT, EPI>::BYTES];
   static_assert(EPI != DMQ_EPI_SILU_ROT || KS == 1, "the fused rotation needs the whole block in one workgroup");
-
-  DMQ_MARK(0);
-  DMQ_WG_MARK(0);
   // Workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD gets a contiguous range of
   // the work list, so the workgroups that share an activation tile (the feature blocks of an
   // item) and those that share weights (the row tiles of an expert) meet in one L2.

@@ -12,9 +12,7 @@
 #pragma once
 #include "common.h"
 
-#ifndef DMQ_LUT_ROW
 #define DMQ_LUT_ROW 128
-#endif
 #define DMQ_LUT_BYTES (256 * DMQ_LUT_ROW)
 
 template <int BIT, int ES>   // ES = bytes per dequantized element (2: fp16, 1: int8 / e4m3)

@@ -113,10 +113,8 @@ struct PlanParams {
 // columns, the stable sort by expert and the work-item list in a single launch.
 #define DMQ_ROUTE_SMALL_ROWS 1024       // routed rows (tokens * (k + n_shared)) it handles
 #define DMQ_ROUTE_SMALL_EXPERTS 512     // experts including the shared slices
-#ifndef DMQ_ROUTE_SMALL_TOKENS
 #define DMQ_ROUTE_SMALL_TOKENS 4        // tokens when the top-k is computed inside (one per wave;
                                         // from 8 tokens on it rides the rotation launch instead)
-#endif
 struct RouteSmallParams {
   const void* logits;            // [tokens, router_experts] fp32 / fp16, or NULL
   int logits_fp16;

@@ -362,9 +362,7 @@ void dmq_quantize_kernel(QuantParams p) {
 }
 
 // --------------------------------------------------------------------------------------------
-#ifndef DMQ_ROT_STAGE_MIN_TILES
 #define DMQ_ROT_STAGE_MIN_TILES 1
-#endif
 // tiled_waves: waves of the per-work-item part (max_items * tile_rows / (16*tt) * groups); the
 // whole-batch pools add n_hoisted * ceil(row tiles / 4) * groups workgroups in front
 template <int MODE>

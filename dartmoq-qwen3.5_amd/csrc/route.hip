@@ -13,18 +13,6 @@
 #include "topk.h"
 #include <type_traits>
 
-// developer instrumentation of the one-workgroup routing kernel: wall-clock stamps (100 MHz) of
-// thread 0 at the phase boundaries, read back with dmq_route_trace_read
-#ifdef DMQ_TRACE
-static __device__ long long dmq_route_marks[32];
-#define DMQ_RMARK(i) do { if (threadIdx.x == 0) dmq_route_marks[i] = wall_clock64(); } while (0)
-extern "C" int dmq_route_trace_read(long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(dmq_route_marks), sizeof(long long) * 32);
-}
-#else
-#define DMQ_RMARK(i)
-#endif
-
 // Widen caller-made top-k arrays [tokens, k] by the shared columns.
 __global__ __launch_bounds__(256)
 void dmq_topk_widen_kernel(const int* in_idx, const float* in_w, int tokens, int experts, int k,
@@ -280,7 +268,6 @@ void dmq_plan_kernel(PlanParams p) {
   __shared__ int item_first[DMQ_MAX_POOLS * 1024];
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
-  DMQ_RMARK(8);
   const PlanSlices slices = plan_load_slices(p);       // in flight during the counting phases
   // The chunk axis of the histogram is split over `parts` threads per expert so that all 1024
   // threads load; a thread keeps at most 16 loads in flight and its values stay in registers
@@ -323,7 +310,6 @@ void dmq_plan_kernel(PlanParams p) {
     if (!one_pass) __syncthreads();                    // partial[] is reused by the next pass
   }
   __syncthreads();
-  DMQ_RMARK(9);
   // expert offsets: exclusive scan of counts, 1024 experts per pass
   for (int base = 0; base < p.experts; base += 1024) {
     const int e = base + tid;
@@ -336,7 +322,6 @@ void dmq_plan_kernel(PlanParams p) {
   }
   if (tid == 0) { s_off[0] = 0; p.offsets[0] = 0; }
   __syncthreads();
-  DMQ_RMARK(10);
   // hist[c, e] <- position of the first row of chunk c routed to expert e
   for (int ebase = 0; ebase < p.experts; ebase += epad) {
     const int e = ebase + el;
@@ -358,9 +343,7 @@ void dmq_plan_kernel(PlanParams p) {
     }
     if (!one_pass) __syncthreads();
   }
-  DMQ_RMARK(11);
   plan_emit_items(p, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices, item_first);
-  DMQ_RMARK(12);
 }
 
 // Stable scatter of one chunk.  The rows of one token name distinct experts, so the lanes of a
@@ -423,11 +406,9 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   const int kt = k + p.sg.n_shared;
   const int rows = p.tokens * kt;
   const int experts = p.plan.experts;
-  DMQ_RMARK(0);
   const PlanSlices slices = plan_load_slices(p.plan);  // in flight during the top-k
   for (int i = tid; i < 16 * experts; i += 1024) s_hist[i] = 0;
   for (int i = tid; i < p.clear_count; i += 1024) p.clear_words[i] = 0;
-  DMQ_RMARK(1);
   // top-k (or the caller's), shared columns: the rows of the next token of the wave are requested
   // before the current token is worked on
   auto tokens_of_wave = [&](auto nv_tag) {
@@ -463,9 +444,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   if (!p.logits || p.router_experts <= 256) tokens_of_wave(std::integral_constant<int, 4>{});
   else if (p.router_experts <= 512) tokens_of_wave(std::integral_constant<int, 8>{});
   else tokens_of_wave(std::integral_constant<int, 16>{});
-  DMQ_RMARK(2);
   __syncthreads();
-  DMQ_RMARK(3);
   // rows per (wave chunk, expert)
   const int r = tid;
   const int e_r = (r < rows) ? s_idx[r] : -1;
@@ -488,7 +467,6 @@ void dmq_route_small_kernel(RouteSmallParams p) {
     if (tid == 0) { s_off[0] = 0; p.plan.offsets[0] = 0; }
   }
   __syncthreads();
-  DMQ_RMARK(4);
   // s_hist[w, e] <- sorted position of the first row of wave chunk w routed to expert e
   if (tid < experts) {
     int at = s_off[tid];
@@ -500,9 +478,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
     }
   }
   __syncthreads();
-  DMQ_RMARK(5);
   plan_emit_items(p.plan, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices);
-  DMQ_RMARK(6);
   // stable scatter of the wave's chunk: tokens one after the other, the rows of a token name
   // distinct experts
   const int base = wave * 64;
@@ -520,7 +496,6 @@ void dmq_route_small_kernel(RouteSmallParams p) {
       p.sorted_rows[at] = r;
     }
   }
-  DMQ_RMARK(7);
 }
 
 // Work items for a caller-supplied expert_info (merged-GEMM entry points): one workgroup.

@@ -96,15 +96,20 @@ def dequantize_packed(packed: dict, row_start: int = 0, row_end: int | None = No
     norms = packed["norms"].float()
     if norms.dim() == 1:
         norms = norms.unsqueeze(1)
-    idx = unpack_nbit(packed["indices_packed"][row_start:row_end], bit, k).long()
+    # only the bytes of the groups that overlap the column window are unpacked (the reference
+    # unpacks the whole matrix first, :733: same values, a pool-sized temporary per call)
+    g_first = (col_start // gs) * gs
+    g_last = min(-(-col_end // gs) * gs, k)
+    epb = 8 // bit
+    idx = unpack_nbit(packed["indices_packed"][row_start:row_end, g_first // epb:-(-g_last // epb)],
+                      bit, g_last - g_first).long()
     norms = norms[row_start:row_end]
     out = torch.zeros((row_end - row_start, col_end - col_start), dtype=torch.float32)
-    g_first = (col_start // gs) * gs
     for g0 in range(g_first, col_end, gs):
         g1 = min(g0 + gs, k)
         d = g1 - g0
         p = rotation_matrix(d, seed + g0)
-        wg = (cb[idx[:, g0:g1]] / math.sqrt(d)) @ p * norms[:, g0 // gs].unsqueeze(1)
+        wg = (cb[idx[:, g0 - g_first:g1 - g_first]] / math.sqrt(d)) @ p * norms[:, g0 // gs].unsqueeze(1)
         lo, hi = max(col_start, g0), min(col_end, g1)
         out[:, lo - col_start:hi - col_start] = wg[:, lo - g0:hi - g0]
     return out if out_dtype is None else out.to(out_dtype)

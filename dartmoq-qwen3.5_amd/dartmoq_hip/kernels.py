@@ -224,16 +224,35 @@ def _group_first_cached(indices_packed, norms, group_size, bit_width):
     return hit
 
 
+_RAGGED_CACHE: dict = {}
+
+
+def _ragged_linear(indices_packed, codebook, norms, seed, group_size, in_features, bit_width):
+    """A WxA16Linear over a row-major packed matrix whose last group is short; kept per
+    (tensor, shape) like the group-first copies, since it pads and re-lays the weights out."""
+    from .linear import WxA16Linear
+    key = (indices_packed.data_ptr(), tuple(indices_packed.shape), norms.data_ptr(), _seed(seed),
+           int(in_features), int(bit_width), indices_packed._version, norms._version)
+    hit = _RAGGED_CACHE.get(key)
+    if hit is None:
+        hit = WxA16Linear(in_features, indices_packed.shape[0], bit_width, group_size, indices_packed,
+                          codebook, norms, _seed(seed), device=indices_packed.device)
+        if len(_RAGGED_CACHE) >= 64:
+            _RAGGED_CACHE.pop(next(iter(_RAGGED_CACHE)))
+        _RAGGED_CACHE[key] = hit
+    return hit
+
+
 def triton_fused_matmul_grouped(x, indices_packed, codebook, norms, seed, group_size, in_features,
                                 bit_width: int = 4):
     """triton_kernels.py:600-684, the kernel of WxA16Linear.forward: x[B, K] times the whole packed
     matrix [N, K*bit/8] (row-major, bit 1/2/4/8), group g rotated with seed + g*group_size.
-    in_features must be a multiple of the group size (the reference's per-group fallback for ragged
-    K is not built)."""
+    A ragged last group (in_features % group_size != 0, the reference's per-group path :652-684)
+    runs through a WxA16Linear, which pads that group once."""
     _check_bit(bit_width, {1, 2, 4, 8}, "matmul_grouped")
     _check_gs(group_size)
     if in_features % group_size:
-        raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
+        return _ragged_linear(indices_packed, codebook, norms, seed, group_size, in_features, bit_width)(x)
     idx_gf, norms_gf = _group_first_cached(indices_packed, norms, group_size, bit_width)
     return triton_fused_matmul_grouped_slice_rows_gf(
         x, idx_gf, codebook, norms_gf, seed, group_size, in_features, 0, indices_packed.shape[0],
@@ -246,7 +265,9 @@ def triton_fused_matmul_grouped_slice_rows(x, indices_packed, codebook, norms, s
     _check_bit(bit_width, {1, 2, 4, 8}, "slice_rows")
     _check_gs(group_size)
     if in_features % group_size:
-        raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
+        n2 = norms if norms.dim() == 2 else norms.unsqueeze(1)
+        return _ragged_linear(indices_packed[row_start:row_end], codebook, n2[row_start:row_end], seed,
+                              group_size, in_features, bit_width)(x)
     idx_gf, norms_gf = _group_first_cached(indices_packed, norms, group_size, bit_width)
     return triton_fused_matmul_grouped_slice_rows_gf(
         x, idx_gf, codebook, norms_gf, seed, group_size, in_features, row_start, row_end, bit_width,

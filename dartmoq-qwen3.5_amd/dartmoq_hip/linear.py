@@ -75,8 +75,8 @@ class WxA16Linear:
             raise ValueError(f"bit_width must be 1/2/4/8, got {bit_width}")
         if group_size != GROUP_SIZE:
             raise ValueError(f"group_size must be {GROUP_SIZE}, got {group_size}")
-        if in_features % group_size:
-            raise ValueError(f"in_features ({in_features}) must be a multiple of group_size ({group_size})")
+        if in_features % (8 // bit_width):
+            raise ValueError(f"in_features ({in_features}) must fill whole bytes of {bit_width}-bit indices")
         if rotation != "qr":
             raise ValueError(f"rotation must be 'qr', got {rotation!r}")
         self.in_features, self.out_features = int(in_features), int(out_features)
@@ -84,10 +84,18 @@ class WxA16Linear:
         self.seed = int(seed.item()) if isinstance(seed, torch.Tensor) else int(seed)
         self.rotation, self.orig_dtype, self.codebook_type = rotation, orig_dtype, codebook_type
         self.device = torch.device(device)
-        self.n_groups = self.in_features // self.group_size
+        self.n_groups = -(-self.in_features // self.group_size)
+        # A ragged last group (in_features % 128 = d > 0: the reference's per-group path,
+        # turboquant_utils/triton_kernels.py:618-650, rotates it with a d x d matrix seeded
+        # seed + g_start and scales by 1 / sqrt(d)) is widened to a full group once, here: index
+        # bytes and activation columns padded with zeros, the d x d rotation in the corner of a
+        # 128 x 128 matrix of zeros, the group's norm times sqrt(128 / d).
+        self.k_padded = self.n_groups * self.group_size
+        self.last_dim = self.in_features - (self.n_groups - 1) * self.group_size
         ppg = self.group_size * self.bit_width // 8
-        if tuple(packed_indices.shape) != (self.out_features, self.n_groups * ppg):
-            raise ValueError(f"packed_indices must be {(self.out_features, self.n_groups * ppg)}, "
+        row_bytes = self.in_features * self.bit_width // 8
+        if tuple(packed_indices.shape) != (self.out_features, row_bytes):
+            raise ValueError(f"packed_indices must be {(self.out_features, row_bytes)}, "
                              f"got {tuple(packed_indices.shape)}")
         if norms.dim() == 1:
             norms = norms.unsqueeze(1)
@@ -96,11 +104,24 @@ class WxA16Linear:
         self.codebook = codebook.to(self.device, torch.float16).contiguous()
         self.bias = None if bias is None else bias.to(self.device)
         # group-first relayout, norms / sqrt(gs): the row-major originals are not kept on the device
+        packed_indices = packed_indices.to(self.device)
+        norms = norms.to(self.device).half()
+        full_groups = self.n_groups
+        if self.k_padded != self.in_features:
+            full_groups -= 1
+            packed_indices = torch.nn.functional.pad(packed_indices, (0, self.n_groups * ppg - row_bytes))
+            norms = norms.float()
+            norms[:, -1] *= (self.group_size / self.last_dim) ** 0.5
+            norms = norms.half()
         self.indices_gf, self.norms_gf = ops.convert_to_group_first(
-            packed_indices.to(self.device).contiguous(), norms.to(self.device).half().contiguous(),
-            self.group_size, self.bit_width, prescale=True)
-        self.rot = hostprep.generate_batch_rotation_matrices(self.group_size, self.seed, self.n_groups,
+            packed_indices.contiguous(), norms.contiguous(), self.group_size, self.bit_width, prescale=True)
+        self.rot = hostprep.generate_batch_rotation_matrices(self.group_size, self.seed, full_groups,
                                                              self.group_size, self.device)
+        if full_groups != self.n_groups:
+            last = torch.zeros((1, self.group_size, self.group_size), dtype=torch.float16, device=self.device)
+            small = hostprep.generate_rotation_matrix(self.last_dim, self.seed + full_groups * self.group_size)
+            last[0, :self.last_dim, :self.last_dim] = small.to(self.device, torch.float16)
+            self.rot = torch.cat([self.rot, last], 0).contiguous()
         self._ctx: dict[int, tuple] = {}
         self._info: dict[int, torch.Tensor] = {}
         self._tile_cache: dict = {}
@@ -210,7 +231,7 @@ class WxA16Linear:
             lut, extra = self._mode_ctx()
             d = LinearDesc()
             d.mode, d.bit = self.MODE, self.bit_width
-            d.in_features, d.out_features = self.in_features, self.out_features
+            d.in_features, d.out_features = self.k_padded, self.out_features
             d.indices_gf, d.norms_gf = self.indices_gf.data_ptr(), self.norms_gf.data_ptr()
             d.lut = lut.data_ptr() if lut is not None else None
             d.rot, d.extra_scale = self.rot.data_ptr(), float(extra)
@@ -227,6 +248,8 @@ class WxA16Linear:
             raise ValueError(f"expected {self.in_features} input features, got {shape[-1]}")
         x2 = x.reshape(-1, self.in_features)
         src = x2 if x2.dtype == torch.float16 else x2.half()
+        if self.k_padded != self.in_features:
+            src = torch.nn.functional.pad(src, (0, self.k_padded - self.in_features))
         if src.stride(1) != 1 or src.stride(0) % 8:
             src = src.contiguous()
         rows = src.shape[0]
@@ -253,6 +276,8 @@ class WxA16Linear:
             raise ValueError(f"expected {self.in_features} input features, got {shape[-1]}")
         x2 = x.reshape(-1, self.in_features)
         src = x2 if x2.dtype == torch.float16 else x2.half()
+        if self.k_padded != self.in_features:
+            src = torch.nn.functional.pad(src, (0, self.k_padded - self.in_features))
         rows = src.shape[0]
         if rows == 0:
             return torch.empty(*shape[:-1], self.out_features, dtype=x.dtype, device=x.device)

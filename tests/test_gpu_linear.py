@@ -58,6 +58,35 @@ def test_quantized_activation_linears(mode, cls, tight):
     assert relerr(out, ref) < {"wxa8": 0.02, "wxfp8": 0.075}[mode]
 
 
+@pytest.mark.parametrize("k", [200, 448])
+@pytest.mark.parametrize("bit,mode", [(4, "wxa16"), (2, "wxa16"), (1, "wxa16"), (4, "wxa8"), (4, "wxfp8")])
+def test_ragged_in_features(k, bit, mode):
+    """in_features not a multiple of the group size: the last group has d = k % 128 columns, its own
+    d x d rotation (seed + g_start) and scale 1 / sqrt(d), the reference's per-group path
+    (turboquant_utils/triton_kernels.py:618-650); here the group is padded to 128 once at load."""
+    import dartmoq_hip
+    packed = _packed(192, k, bit, seed=k + bit)
+    assert packed["indices_packed"].shape == (192, k * bit // 8) and packed["norms"].shape == (192, -(-k // 128))
+    lin = dartmoq_hip.WxA16Linear.from_packed(packed)
+    if mode != "wxa16":
+        lin = {"wxa8": dartmoq_hip.WxA8Linear, "wxfp8": dartmoq_hip.WxFP8Linear}[mode].from_wxa16(lin)
+    x = torch.randn(45, k, generator=torch.Generator().manual_seed(k)).half()
+    out = lin(x.cuda()).float().cpu()
+    ref = x.float() @ turboquant.dequantize_packed(packed).T
+    assert relerr(out, ref) < {"wxa16": 2e-3, "wxa8": 0.02, "wxfp8": 0.075}[mode], relerr(out, ref)
+    if mode == "wxa16":
+        assert max_rel(out, ref) <= 1e-2 and cosine(out, ref) >= 0.9999
+    assert torch.equal(lin.forward_by_pieces(x.cuda()).float().cpu(), out)
+    if mode == "wxa16":
+        # the reference's un-sliced callables take the same route
+        from dartmoq_hip import kernels as K
+        ip, cb, nm = packed["indices_packed"].cuda(), packed["codebook"].cuda(), packed["norms"].cuda()
+        full = K.triton_fused_matmul_grouped(x.cuda(), ip, cb, nm, packed["seed"], 128, k, bit)
+        assert torch.equal(full.float().cpu(), out)
+        part = K.triton_fused_matmul_grouped_slice_rows(x.cuda(), ip, cb, nm, packed["seed"], 128, k, 64, 192, bit)
+        assert relerr(part.float().cpu(), ref[:, 64:192]) < 2e-3
+
+
 def test_linear_bias_shapes_and_dtypes():
     import dartmoq_hip
     packed = _packed(128, 256, 2, seed=3)

@@ -53,7 +53,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 14; }
+int dmq_abi_version(void) { return 15; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -396,6 +396,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   L.tt = a->tt;
   L.nt = one_tile ? 1 : 4;
   L.dbg = a->dbg_acc != nullptr;
+  L.roomy = (a->roomy != 0 && a->tt == 1 && ks == 1 && !L.dbg) ? 1 : 0;
   L.stream = (hipStream_t)stream;
   // the 1/2/4-bit pools and the 8-bit pools of the mode are separate launches over the same work
   // list (each skips the items of the other kind); 8-bit pools never split K over the waves
@@ -832,6 +833,20 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if (!seen) modes[n_modes++] = m;
   }
 
+  // 16-row tiles: which kernel instance (see dmq_gemm_args.roomy).  The two-per-CU instance wins
+  // while the gate_up launch has few workgroups (routed rows x feature blocks; measured: H=2048
+  // I=512 up to 128 tokens, H=3072 I=1024 up to 32) and whenever most rows go to 4-bit weights.
+  bool roomy = false;
+  if (tt == 1) {
+    roomy = (long)tokens * K * (I / DMQ_GS) <= 4096;
+    long w4 = 0, w_all = 0;                            // gate_up rows held by 4-bit pools / by all pools
+    for (int i = 0; i < P; ++i) {
+      w_all += layer->pool[i].n_gate_up;
+      if (layer->pool[i].bit == 4 && layer->pool[i].mode != DMQ_MODE_FP4) w4 += layer->pool[i].n_gate_up;
+    }
+    if (2 * w4 > w_all) roomy = true;
+  }
+
   // The gate_up GEMM rotates (and quantizes) its SiLU*up rows for the down projection itself when
   // a workgroup owns whole blocks of 128 features: no K split, no 8-bit pools in the mode.
   bool fuse_rot[DMQ_MAX_POOLS];
@@ -974,7 +989,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     g.mode = mode; g.epi = fuse_rot[mi] ? DMQ_EPI_SILU_ROT : DMQ_EPI_SILU;
     // the gate_up blocks are four times as long as the down blocks (K = H against K = I) and end in
     // the rotation epilogue: more than two per workgroup costs more in balance than it saves
-    g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P;
+    g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P; g.roomy = roomy;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = whole_batch[i];
@@ -1052,7 +1067,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     // until the experts are big enough for its 64-row kernel to pay
     const long avg_rows = (long)tokens * K / E;
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
-    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt;
+    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
     d.ks = ks; d.nbl = nbl; d.n_pools = P;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
@@ -1079,7 +1094,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
         for (int wi = 0; wi < layer->n_widths; ++wi) {
           const int mode = modes[mi], W = layer->widths[wi];
           dmq_gemm_args d{};
-          d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt == 4 ? 2 : tt; d.item_tile_rows = 16 * tt;
+          d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = tt == 4 ? 2 : tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
           d.ks = 1; d.nbl = nbl; d.n_pools = P;
           for (int i = 0; i < P; ++i) {
             const dmq_pool_desc& pd = layer->pool[i];

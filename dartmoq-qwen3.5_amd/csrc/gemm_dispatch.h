@@ -11,6 +11,7 @@ struct GemmLaunch {
   int dbg;
   int wide;        // 1: the pools of 8-bit indices (ks must be 1 unless nt == 1), 0: the 1/2/4-bit pools
   int nt;          // n-tiles per wave: 4, or 1 (plain store, tt == 1, ks == 4 only)
+  int roomy;       // tt == 1, ks == 1: the two-waves-per-SIMD instance (see ROOMY)
   int grid;
   hipStream_t stream;
 };
@@ -31,6 +32,13 @@ static int dmq_gemm_launch_one(const GemmLaunch& L) {
     }
   }
   if (L.wide) return DMQ_ERR_MODE;
+  if constexpr (MODE != DMQ_MODE_FP4 && TT == 1 && KS == 1 && !DBG) {
+    if (L.roomy) {
+      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, true>), dim3(L.grid),
+                         dim3(256), 0, L.stream, L.p);
+      return dmq_check_launch();
+    }
+  }
   hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false>), dim3(L.grid), dim3(256), 0,
                      L.stream, L.p);
   return dmq_check_launch();

@@ -1033,8 +1033,12 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 // NT: n-tiles of 16 features per wave.  Four everywhere except the instances for a Linear with a
 // handful of rows (NT = 1, K split over the four waves: a workgroup covers 16 features, so a
 // 4096-feature matrix gives 256 workgroups instead of 64).
-template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT = 4>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2) ? 3 : 2)))
+// ROOMY (16-row tiles, 1/2/4-bit pools): two waves per SIMD instead of three.  At three the body
+// of the 4-bit weights keeps part of its weight ring in scratch memory inside the K loop; a
+// launch that fills at most two workgroups per CU anyway, or one with 4-bit pools, runs the
+// instance that has the registers.
+template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT = 4, bool ROOMY = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2 && !ROOMY) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
   __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2];

@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 14). */
+/* Library / build identification: returns the ABI version (currently 15). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -287,6 +287,11 @@ typedef struct {
   int width_filter;
   int home_filter;
   int accumulate;
+  /* tt == 1, ks == 1, 1/2/4-bit pools (not WxFP4): != 0 selects the kernel instance that keeps two
+   * workgroups per CU instead of three and in exchange holds the weight ring of 4-bit pools in
+   * registers (the three-per-CU instance keeps part of it in scratch memory).  Pays for launches
+   * of at most two workgroups per CU and for layers with 4-bit pools; same results either way. */
+  int roomy;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

@@ -255,6 +255,51 @@ def test_sub_expert_layer_matches_oracles(sliced_layer, mode, tokens, tt):
     assert relerr(out, ref) < MODE_BOUND[mode], (mode, relerr(out, ref))
 
 
+@pytest.mark.parametrize("tokens", [1, 3, 40, 200])
+def test_sub_expert_layer_from_logits_split_and_graph(sliced_layer, tokens):
+    """A sub-expert layer through the other routing shapes (top-k inside the fused routing launch,
+    top-k on the rotation launch, chunked sort): the forward from logits equals the forward from
+    the same top-k, batch splitting leaves every row unchanged, and a captured graph replays the
+    eager bits."""
+    from dartmoq_hip import ops
+    layer = sliced_layer
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(tokens, layer.hidden, generator=g).half().cuda()
+    logits = routing.zipf_logits(tokens, layer.num_experts, tokens).cuda()
+    mod = make_module(layer, "wxa16")
+    w, idx = ops.route_topk(logits, layer.top_k)
+    a = mod.forward(x, router_logits=logits).clone()
+    b = mod.forward(x, topk_idx=idx, topk_w=w).clone()
+    assert torch.equal(a, b)
+    ideal = moe.quantized_forward(layer, x.cpu(), idx.cpu().long(), w.cpu(), "wxa16")
+    assert relerr(a.float().cpu(), ideal) < 3e-3
+    if tokens >= 40:
+        cut = tokens // 3
+        mod.tt_override = 2
+        full = mod.forward(x, topk_idx=idx, topk_w=w).clone()
+        lo = mod.forward(x[:cut].contiguous(), topk_idx=idx[:cut].contiguous(), topk_w=w[:cut].contiguous()).clone()
+        hi = mod.forward(x[cut:].contiguous(), topk_idx=idx[cut:].contiguous(), topk_w=w[cut:].contiguous()).clone()
+        assert torch.equal(torch.cat([lo, hi]), full)
+        mod.tt_override = 0
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            mod.forward(x, router_logits=logits)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = mod.forward(x, router_logits=logits)
+    for _ in range(3):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, a)
+        mod.forward(x.flip(0).contiguous(), router_logits=logits.flip(0).contiguous())
+        torch.cuda.synchronize()
+
+
 def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):

@@ -910,14 +910,33 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   // whole-batch rotation of the first mode: neither needs the other, both are short.
   bool whole_done[DMQ_MAX_POOLS] = {false, false, false, false};   // per mode
   bool topk_done = false;
-  if (!route_small && router->logits) {
+  // Up to four tokens with logits: no sort at all.  The top-k workgroup of that launch writes one
+  // work item per routed row (see DirectPlan); the routing launch below is skipped.
+  const long R = (long)tokens * K;
+  bool direct = !sub && router->logits && tokens <= DMQ_DIRECT_MAX_TOKENS && R <= DMQ_DIRECT_MAX_ROWS &&
+                R <= w.max_items && K <= 64 &&
+                (wsplit_eff == 1 || R * (I / DMQ_GS) <= w.split_counters);
+  bool direct_done = false;
+  if ((direct || !route_small) && router->logits) {
     bool any_whole = false;
     for (int i = 0; i < P; ++i) any_whole |= (whole_batch[i] && layer->pool[i].mode == modes[0]);
     const int rk = K - n_shared, re = E - n_shared;
     if (any_whole && re <= 1024 && rk <= 64 && rk <= re && rk > 0 && n_shared <= 64) {
       const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
-      const TopkParams tp{router->logits, tokens, re, rk, router->renorm, w.topk_w, w.topk_idx, sg,
-                          (tokens + 3) / 4};
+      TopkParams tp{router->logits, tokens, re, rk, router->renorm, w.topk_w, w.topk_idx, sg,
+                    (tokens + 3) / 4, DirectPlan{}};
+      if (direct) {
+        tp.blocks = 1;
+        DirectPlan& dp = tp.dp;
+        dp.on = 1; dp.pools = P; dp.experts = E;
+        dp.slice_start_rows = (const int*)layer->slice_start;
+        dp.slice_count_rows = (const int*)layer->slice_count;
+        dp.items = w.items; dp.n_items = w.n_items; dp.counts = w.counts;
+        dp.sorted_tokens = w.sorted_tokens; dp.sorted_weights = w.sorted_weights;
+        dp.sorted_rows = w.sorted_rows;
+        if (wsplit_eff > 1) { dp.clear_words = w.split_counter; dp.clear_count = w.split_counters; }
+        direct_done = true;
+      }
       rc = rotate_gate_up_input(modes[0], true, false, &tp, router->logits_fp16);
       if (rc) return rc;
       whole_done[0] = true;
@@ -930,7 +949,9 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   {
     const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
     const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
-    if (route_small) {
+    if (direct_done) {
+      rc = DMQ_OK;
+    } else if (route_small) {
       RouteSmallParams sp{};
       sp.logits = router->logits; sp.logits_fp16 = router->logits_fp16;
       sp.in_idx = (const int*)router->topk_idx; sp.in_w = (const float*)router->topk_w;

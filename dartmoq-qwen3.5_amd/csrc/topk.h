@@ -130,6 +130,31 @@ __device__ __forceinline__ void dmq_topk_token(const T* row, int experts, int k,
   }
 }
 
+// A handful of tokens: the routing step inside one top-k workgroup.  With a few dozen routed rows the
+// stable sort by expert is a brute-force ranking (every row counts the rows that come before it),
+// and the work items (one per routed expert: at most four rows each) follow from the same scan:
+// the record at the sorted position of an expert's first row carries the item, the positions of
+// its other rows hold empty records.  Same permutation and counts as the chunked sort.  Measured
+// with more tokens per wave (8 and 16 tokens): the serial top-k rounds cost more than the routing
+// launch they replace, so four tokens (one per wave) is the limit.  It saves the routing
+// launch (~9 us of a 37 us forward at one token).
+#define DMQ_DIRECT_MAX_TOKENS 4
+#define DMQ_DIRECT_MAX_ROWS 256
+struct DirectPlan {
+  int on;
+  int pools, experts;            // experts including the shared slices
+  const int* slice_start_rows;   // [pools, experts] first gate_up row of the expert's slice, -1: not a member
+  const int* slice_count_rows;   // [pools, experts]
+  int* items;                    // [rows, DMQ_ITEM_WORDS]
+  int* n_items;                  // [2]: rows, 0 (no pool is rotated per work item)
+  int* counts;                   // [experts]
+  int* sorted_tokens;            // [rows] token of the row at each sorted position
+  float* sorted_weights;         // [rows]
+  int* sorted_rows;              // [rows] (token, slot) row at each sorted position
+  int* clear_words;              // tickets of a K range shared between workgroups (or NULL)
+  int clear_count;
+};
+
 // One workgroup of the top-k launch: four tokens, one per wave.
 struct TopkParams {
   const void* logits;            // [tokens, experts] fp32 or fp16 (the kernel's template type)
@@ -138,21 +163,101 @@ struct TopkParams {
   int* out_idx;
   SharedGate sg;
   int blocks;                    // workgroups of the top-k part: ceil(tokens / 4)
+  DirectPlan dp;
 };
 
 template <typename T>
 __device__ __forceinline__ void dmq_topk_wg(const TopkParams& tp, int block) {
   const int lane = threadIdx.x & 63;
   const int tok = block * 4 + (threadIdx.x >> 6);
-  if (tok >= tp.tokens) return;
-  float my_w;
-  int my_e;
-  dmq_topk_token<T>((const T*)tp.logits + (long)tok * tp.experts, tp.experts, tp.k, tp.renorm, lane,
-                    my_w, my_e);
   const int stride = tp.k + tp.sg.n_shared;
-  if (lane < tp.k) {
-    tp.out_w[(long)tok * stride + lane] = my_w;
-    tp.out_idx[(long)tok * stride + lane] = my_e;
+  if (!tp.dp.on) {
+    if (tok >= tp.tokens) return;
+    float my_w;
+    int my_e;
+    dmq_topk_token<T>((const T*)tp.logits + (long)tok * tp.experts, tp.experts, tp.k, tp.renorm, lane,
+                      my_w, my_e);
+    if (lane < tp.k) {
+      tp.out_w[(long)tok * stride + lane] = my_w;
+      tp.out_idx[(long)tok * stride + lane] = my_e;
+    }
+    dmq_shared_columns(tp.sg, tok, tp.experts, tp.k, lane, tp.out_w, tp.out_idx);
+    return;
   }
-  dmq_shared_columns(tp.sg, tok, tp.experts, tp.k, lane, tp.out_w, tp.out_idx);
+  // direct plan: a single workgroup, wave v takes tokens v, v + 4, ...; every wave reaches the barrier
+  __shared__ __attribute__((aligned(16))) int s_expert[DMQ_DIRECT_MAX_ROWS + 4];
+  __shared__ float s_weight[DMQ_DIRECT_MAX_ROWS];
+  const DirectPlan& dp = tp.dp;
+  const int rows = tp.tokens * stride;
+  const int wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < dp.clear_count; i += 256) dp.clear_words[i] = 0;
+  for (int t = wave; t < tp.tokens; t += 4) {
+    float my_w;
+    int my_e;
+    dmq_topk_token<T>((const T*)tp.logits + (long)t * tp.experts, tp.experts, tp.k, tp.renorm, lane,
+                      my_w, my_e);
+    if (tp.sg.n_shared > 0) {
+      const float g = dmq_shared_gate_value(tp.sg, t, lane);
+      if (lane >= tp.k && lane < stride) { my_w = g; my_e = tp.experts + (lane - tp.k); }
+    }
+    if (lane < stride) {
+      const int r = t * stride + lane;
+      tp.out_w[r] = my_w;
+      tp.out_idx[r] = my_e;
+      s_expert[r] = my_e;
+      s_weight[r] = my_w;
+    }
+  }
+  for (int i = rows + threadIdx.x; i < ((rows + 3) & ~3); i += 256) s_expert[i] = 0x7fffffff;   // pad to fours
+  __syncthreads();
+  // the scans read the list four experts at a time (one address for the whole wave: a broadcast)
+  const int rows4 = (rows + 3) >> 2;
+  for (int t = wave; t < tp.tokens; t += 4) {
+    const bool mine = lane < stride;
+    const int r = t * stride + lane;
+    const int my_e = mine ? s_expert[r] : -1;
+    // slices of the expert's pool (the first pool that holds a slice of it): requested before the scan
+    int pool = 0, ss = -1;
+    if (mine) {
+      bool found = false;
+#pragma unroll
+      for (int q = 0; q < DMQ_MAX_POOLS; ++q) {
+        if (q < dp.pools && !found && dp.slice_count_rows[q * dp.experts + my_e] > 0) {
+          found = true; pool = q; ss = dp.slice_start_rows[q * dp.experts + my_e];
+        }
+      }
+    }
+    int pos = 0, cnt = 0, before = 0;                 // before: rows of my expert ahead of mine
+    for (int q = 0; q < rows4; ++q) {
+      const int4_t e4 = *(const int4_t*)(s_expert + 4 * q);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int same = (e4[c] == my_e) ? 1 : 0;
+        pos += (e4[c] < my_e) ? 1 : 0;
+        cnt += same;
+        before += (same && 4 * q + c < r) ? 1 : 0;
+      }
+    }
+    pos += before;
+    if (mine) {
+      dp.sorted_tokens[pos] = t;
+      dp.sorted_weights[pos] = s_weight[r];
+      dp.sorted_rows[pos] = r;
+      // the record at the row's own sorted position: the first row of an expert carries the item,
+      // the others leave an empty record (no rows: its workgroups return at once)
+      const bool item = before == 0 && ss >= 0;
+      int4_t* it = (int4_t*)(dp.items + (long)DMQ_ITEM_WORDS * pos);
+      it[0] = (int4_t){pool, my_e, 0, pos};
+      it[1] = (int4_t){item ? cnt : 0, ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
+    }
+  }
+  for (int e = threadIdx.x; e < dp.experts; e += 256) {
+    int c = 0;
+    for (int q = 0; q < rows4; ++q) {
+      const int4_t e4 = *(const int4_t*)(s_expert + 4 * q);
+      c += (e4[0] == e) + (e4[1] == e) + (e4[2] == e) + (e4[3] == e);
+    }
+    dp.counts[e] = c;
+  }
+  if (threadIdx.x == 0) { dp.n_items[0] = rows; dp.n_items[1] = 0; }
 }

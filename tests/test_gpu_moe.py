@@ -300,6 +300,37 @@ def test_sub_expert_layer_from_logits_split_and_graph(sliced_layer, tokens):
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("tokens", [1, 2, 4])
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp4"])
+def test_few_tokens_from_logits_with_shared_expert(shared_layer, mode, tokens):
+    """Up to four tokens with logits: routing, shared columns and work items come from the top-k
+    workgroup.  Same bits as the forward from the same top-k (which sorts), the oracle's values,
+    and the per-expert counts of the routing."""
+    from dartmoq_hip import ops
+    from dartmoq_hip.moe import forward_staged
+    layer = shared_layer
+    g = torch.Generator().manual_seed(100 + tokens)
+    x = torch.randn(tokens, layer.hidden, generator=g).half().cuda()
+    # a flat router makes tokens share experts (rows of one expert from several tokens)
+    logits = (routing.zipf_logits(tokens, layer.num_experts, 5) * 0.05 +
+              routing.zipf_logits(1, layer.num_experts, 6)).cuda()
+    mod = make_module(layer, mode)
+    w, idx = ops.route_topk(logits, layer.top_k)
+    a = mod.forward(x, router_logits=logits).clone()
+    b = mod.forward(x, topk_idx=idx, topk_w=w).clone()
+    assert torch.equal(a, b)
+    ideal = moe.quantized_forward(layer, x.cpu(), idx.cpu().long(), w.cpu(), mode)
+    tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp4": 6e-2}[mode]
+    assert relerr(a.float().cpu(), ideal) < tight
+    _out, _stats, aux = forward_staged(mod, x, router_logits=logits)
+    counts = aux["counts"].cpu().long()
+    want = torch.bincount(idx.cpu().long().flatten(), minlength=layer.num_experts)
+    assert torch.equal(counts[:layer.num_experts], want)
+    assert torch.all(counts[layer.num_experts:] == tokens)          # the shared slices see every token
+    if tokens > 1:
+        assert int(want.max()) > 1                                   # the case has shared experts
+
+
 def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):
@@ -328,11 +359,11 @@ def test_from_reference_module_duck_typing():
     assert torch.equal(y1, y2)
 
 
-@pytest.mark.parametrize("tokens", [1, 64, 65, 128, 300])
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4, 5, 64, 65, 128, 300])
 def test_forward_from_logits_equals_forward_from_topk(small_layer, tokens):
-    """The routing step has three shapes (one fused launch with the top-k inside, fused launch
-    after a separate top-k, chunked sort): all must give the bits of the forward that is handed
-    the same top-k."""
+    """The routing step has four shapes (up to four tokens: ranking inside the top-k workgroup of
+    the rotation launch; one fused launch with the caller's top-k; fused launch after a separate
+    top-k; chunked sort): all must give the bits of the forward that is handed the same top-k."""
     from dartmoq_hip import ops
     g = torch.Generator().manual_seed(tokens)
     x = torch.randn(tokens, small_layer.hidden, generator=g).half().cuda()

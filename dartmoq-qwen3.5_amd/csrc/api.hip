@@ -22,14 +22,14 @@ static inline int scale_stride_for(int mode, int k) {
 
 static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE_FP4; }
 
-// K split across the four waves of a workgroup: a handful of routed rows leaves most CUs idle
-// unless every wave takes a quarter of K; otherwise the waves own different output features
 // K split of the 16-row tile kernels for short work lists.  Up to 128 routed rows leave most CUs
-// with at most one workgroup: two workgroups then share the K range of every gate_up block
-// (negative value; needs an even number of groups).  Splitting K over the four waves of a
-// workgroup instead only pays for a handful of rows.
+// with at most one workgroup: two workgroups then share the K range of every gate_up block, four
+// with at most 16 rows (negative value; the group count must divide).  Measured at H=2048 / 3072:
+// four-way wins up to 16 rows (1 token: 30.6 -> 28.7 us), two-way up to 128, none beyond.
+// Splitting K over the four waves of a workgroup instead only pays when the groups do not divide.
 static inline int pick_ks(int tt, long rows, int groups) {
   if (tt != 1) return 1;
+  if (rows <= 16 && groups % 4 == 0) return -4;
   if (rows <= 128 && groups % 2 == 0) return -2;
   return rows <= 16 ? 4 : 1;
 }

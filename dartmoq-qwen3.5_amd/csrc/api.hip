@@ -910,21 +910,23 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   // whole-batch rotation of the first mode: neither needs the other, both are short.
   bool whole_done[DMQ_MAX_POOLS] = {false, false, false, false};   // per mode
   bool topk_done = false;
-  // Up to four tokens with logits: no sort at all.  The top-k workgroup of that launch writes one
-  // work item per routed row (see DirectPlan); the routing launch below is skipped.
+  // Up to four tokens (logits or a caller-made top-k): no sort launch.  The top-k workgroup of the
+  // rotation launch ranks the routed rows itself and writes the work items (see DirectPlan); the
+  // routing launch below is skipped.
   const long R = (long)tokens * K;
-  bool direct = !sub && router->logits && tokens <= DMQ_DIRECT_MAX_TOKENS && R <= DMQ_DIRECT_MAX_ROWS &&
+  bool direct = !sub && tokens <= DMQ_DIRECT_MAX_TOKENS && R <= DMQ_DIRECT_MAX_ROWS &&
                 R <= w.max_items && K <= 64 &&
                 (wsplit_eff == 1 || R * (I / DMQ_GS) <= w.split_counters);
   bool direct_done = false;
-  if ((direct || !route_small) && router->logits) {
+  if (direct || (!route_small && router->logits)) {
     bool any_whole = false;
     for (int i = 0; i < P; ++i) any_whole |= (whole_batch[i] && layer->pool[i].mode == modes[0]);
     const int rk = K - n_shared, re = E - n_shared;
     if (any_whole && re <= 1024 && rk <= 64 && rk <= re && rk > 0 && n_shared <= 64) {
       const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
       TopkParams tp{router->logits, tokens, re, rk, router->renorm, w.topk_w, w.topk_idx, sg,
-                    (tokens + 3) / 4, DirectPlan{}};
+                    (tokens + 3) / 4, DirectPlan{}, (const int*)router->topk_idx,
+                    (const float*)router->topk_w};
       if (direct) {
         tp.blocks = 1;
         DirectPlan& dp = tp.dp;

@@ -164,6 +164,8 @@ struct TopkParams {
   SharedGate sg;
   int blocks;                    // workgroups of the top-k part: ceil(tokens / 4)
   DirectPlan dp;
+  const int* in_idx;             // direct plan without logits: the caller's top-k [tokens, k]
+  const float* in_w;
 };
 
 template <typename T>
@@ -192,10 +194,15 @@ __device__ __forceinline__ void dmq_topk_wg(const TopkParams& tp, int block) {
   const int wave = threadIdx.x >> 6;
   for (int i = threadIdx.x; i < dp.clear_count; i += 256) dp.clear_words[i] = 0;
   for (int t = wave; t < tp.tokens; t += 4) {
-    float my_w;
-    int my_e;
-    dmq_topk_token<T>((const T*)tp.logits + (long)t * tp.experts, tp.experts, tp.k, tp.renorm, lane,
-                      my_w, my_e);
+    float my_w = 0.f;
+    int my_e = 0;
+    if (tp.logits) {
+      dmq_topk_token<T>((const T*)tp.logits + (long)t * tp.experts, tp.experts, tp.k, tp.renorm, lane,
+                        my_w, my_e);
+    } else if (lane < tp.k) {
+      my_w = tp.in_w[(long)t * tp.k + lane];
+      my_e = tp.in_idx[(long)t * tp.k + lane];
+    }
     if (tp.sg.n_shared > 0) {
       const float g = dmq_shared_gate_value(tp.sg, t, lane);
       if (lane >= tp.k && lane < stride) { my_w = g; my_e = tp.experts + (lane - tp.k); }

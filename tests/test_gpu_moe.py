@@ -331,6 +331,27 @@ def test_few_tokens_from_logits_with_shared_expert(shared_layer, mode, tokens):
         assert int(want.max()) > 1                                   # the case has shared experts
 
 
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8"])
+def test_few_tokens_routing_matches_the_sorted_path(shared_layer, mode):
+    """Four tokens are routed inside the top-k workgroup, five by the one-workgroup sort: the rows
+    of the first four tokens must come out bit for bit the same either way (same tiling and K
+    sharing at both sizes), from logits and from a caller-made top-k."""
+    from dartmoq_hip import ops
+    layer = shared_layer
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(5, layer.hidden, generator=g).half().cuda()
+    logits = (routing.zipf_logits(5, layer.num_experts, 9) * 0.05 +
+              routing.zipf_logits(1, layer.num_experts, 10)).cuda()
+    mod = make_module(layer, mode)
+    mod.ks_override = -2
+    w, idx = ops.route_topk(logits, layer.top_k)
+    five = mod.forward(x, router_logits=logits).clone()
+    four = mod.forward(x[:4].contiguous(), router_logits=logits[:4].contiguous()).clone()
+    assert torch.equal(four, five[:4])
+    four_topk = mod.forward(x[:4].contiguous(), topk_idx=idx[:4].contiguous(), topk_w=w[:4].contiguous())
+    assert torch.equal(four_topk, four)
+
+
 def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):

@@ -225,7 +225,7 @@ __device__ __forceinline__ void dmq_topk_wg(const TopkParams& tp, int block) {
     const int my_e = mine ? s_expert[r] : -1;
     // slices of the expert's pool (the first pool that holds a slice of it): requested before the scan
     int pool = 0, ss = -1;
-    if (mine) {
+    if (mine && my_e >= 0 && my_e < dp.experts) {      // a caller-made top-k may name no expert
       bool found = false;
 #pragma unroll
       for (int q = 0; q < DMQ_MAX_POOLS; ++q) {

@@ -951,8 +951,25 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   {
     const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
     const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
+    // up to 256 routed rows with the top-k at hand: the one-row-per-thread ranking kernel
+    const int* rank_idx = topk_done ? w.topk_idx
+                                    : ((!router->logits && n_shared == 0) ? (const int*)router->topk_idx : nullptr);
+    const float* rank_w = topk_done ? w.topk_w
+                                    : ((!router->logits && n_shared == 0) ? (const float*)router->topk_w : nullptr);
     if (direct_done) {
       rc = DMQ_OK;
+    } else if (!sub && rank_idx && rank_w && R <= DMQ_ROUTE_RANK_ROWS && lead_pools == 0) {
+      RouteRankParams rr{};
+      rr.in_idx = rank_idx; rr.in_w = rank_w;
+      rr.rows = (int)R; rr.k = K; rr.experts = E; rr.pools = P; rr.tile_rows = w.tile_rows;
+      rr.max_items = w.max_items;
+      rr.slice_start_rows = (const int*)layer->slice_start;
+      rr.slice_count_rows = (const int*)layer->slice_count;
+      rr.counts = w.counts; rr.n_items = w.n_items; rr.items = w.items;
+      rr.sorted_tokens = w.sorted_tokens; rr.sorted_weights = w.sorted_weights;
+      rr.sorted_rows = w.sorted_rows;
+      if (wsplit_eff > 1) { rr.clear_words = w.split_counter; rr.clear_count = w.split_counters; }
+      rc = dmq_route_rank_launch(rr, st);
     } else if (route_small) {
       RouteSmallParams sp{};
       sp.logits = router->logits; sp.logits_fp16 = router->logits_fp16;

@@ -133,6 +133,29 @@ struct RouteSmallParams {
 };
 int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream);
 
+// Routing of at most DMQ_ROUTE_RANK_ROWS routed rows from a finished top-k, for the layer forward:
+// one workgroup, one row per thread, every row ranks itself against the whole list (stable sort by
+// expert without histograms or scans over experts).  Writes the permutation, the per-expert counts
+// and the work items (expert order, dense); no per-pool expert_info, no offsets: the layer's
+// launches read neither.  Needs every pool rotated by token (no per-work-item prefix).
+#define DMQ_ROUTE_RANK_ROWS 128
+struct RouteRankParams {
+  const int* in_idx;             // [rows] expert per routed row (token-major, k per token)
+  const float* in_w;             // [rows]
+  int rows, k, experts, pools, tile_rows, max_items;
+  const int* slice_start_rows;   // [pools, experts]
+  const int* slice_count_rows;
+  int* counts;                   // [experts]
+  int* n_items;                  // [2]
+  int* items;                    // [max_items, DMQ_ITEM_WORDS]
+  int* sorted_tokens;
+  float* sorted_weights;
+  int* sorted_rows;
+  int* clear_words;              // optional: clear_count int32 words set to zero by the launch
+  int clear_count;
+};
+int dmq_route_rank_launch(const RouteRankParams& p, hipStream_t stream);
+
 struct TopkParams;
 // tp != NULL: the launch also runs the router's top-k (workgroups in front; logits fp16 or fp32)
 int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream,

@@ -498,6 +498,90 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   }
 }
 
+// See RouteRankParams.  Rows with an expert id outside the layer rank behind all others and get no
+// entry anywhere (like the counting sort, which skips them).
+__global__ __launch_bounds__(256)
+void dmq_route_rank_kernel(RouteRankParams p) {
+  __shared__ __attribute__((aligned(16))) int s_expert[DMQ_ROUTE_RANK_ROWS + 4];
+  __shared__ __attribute__((aligned(16))) int s_tiles[DMQ_ROUTE_RANK_ROWS + 4];
+  const int r = threadIdx.x;
+  const bool mine = r < p.rows;
+  int e = mine ? p.in_idx[r] : 0x7fffffff;
+  const float w = mine ? p.in_w[r] : 0.f;
+  const bool valid = mine && e >= 0 && e < p.experts;
+  if (!valid) e = 0x7fffffff;
+  s_expert[r] = e;
+  s_tiles[r] = 0;
+  if (r < 4) { s_expert[DMQ_ROUTE_RANK_ROWS + r] = 0x7fffffff; s_tiles[DMQ_ROUTE_RANK_ROWS + r] = 0; }
+  for (int i = r; i < p.clear_count; i += 256) p.clear_words[i] = 0;
+  // slice of the expert in the first pool that holds one: in flight during the scan
+  int pool = 0, ss = -1;
+  if (valid) {
+    bool found = false;
+#pragma unroll
+    for (int q = 0; q < DMQ_MAX_POOLS; ++q) {
+      if (q < p.pools && !found && p.slice_count_rows[q * p.experts + e] > 0) {
+        found = true; pool = q; ss = p.slice_start_rows[q * p.experts + e];
+      }
+    }
+  }
+  __syncthreads();
+  // the list is read four experts at a time (one address for the whole wave: a broadcast)
+  const int rows4 = (p.rows + 3) >> 2;
+  int pos = 0, cnt = 0, before = 0;                   // before: rows of my expert ahead of mine
+  for (int q = 0; q < rows4; ++q) {
+    const int4_t e4 = *(const int4_t*)(s_expert + 4 * q);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int same = (e4[c] == e) ? 1 : 0;
+      pos += (e4[c] < e) ? 1 : 0;
+      cnt += same;
+      before += (same && 4 * q + c < r) ? 1 : 0;
+    }
+  }
+  if (valid) {
+    p.sorted_tokens[pos + before] = r / p.k;
+    p.sorted_weights[pos + before] = w;
+    p.sorted_rows[pos + before] = r;
+    if (before == 0 && ss >= 0) s_tiles[r] = (cnt + p.tile_rows - 1) / p.tile_rows;
+  }
+  __syncthreads();
+  // work items: expert order, the tiles of an expert one after the other; the row that opens a
+  // tile writes its record
+  if (valid && ss >= 0 && before % p.tile_rows == 0) {
+    int base = 0;
+    for (int q = 0; q < rows4; ++q) {
+      const int4_t e4 = *(const int4_t*)(s_expert + 4 * q);
+      const int4_t t4 = *(const int4_t*)(s_tiles + 4 * q);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) base += (e4[c] < e) ? t4[c] : 0;
+    }
+    const int idx = base + before / p.tile_rows;
+    if (idx < p.max_items) {
+      int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * idx);
+      it[0] = (int4_t){pool, e, before / p.tile_rows, pos};
+      it[1] = (int4_t){cnt, ss, ss / (2 * DMQ_GS), 0};
+    }
+  }
+  for (int x = r; x < p.experts; x += 256) {
+    int c = 0;
+    for (int q = 0; q < rows4; ++q) {
+      const int4_t e4 = *(const int4_t*)(s_expert + 4 * q);
+      c += (e4[0] == x) + (e4[1] == x) + (e4[2] == x) + (e4[3] == x);
+    }
+    p.counts[x] = c;
+  }
+  if (r == 0) {
+    int n = 0;
+    for (int q = 0; q < rows4; ++q) {
+      const int4_t t4 = *(const int4_t*)(s_tiles + 4 * q);
+      n += t4[0] + t4[1] + t4[2] + t4[3];
+    }
+    p.n_items[0] = min(n, p.max_items);
+    p.n_items[1] = 0;
+  }
+}
+
 // Work items for a caller-supplied expert_info (merged-GEMM entry points): one workgroup.
 __global__ __launch_bounds__(1024)
 void dmq_items_from_info_kernel(const int* expert_info, int experts, int tile_rows, int max_items,
@@ -606,6 +690,13 @@ int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(dmq_route_small_kernel<__half>, dim3(1), dim3(1024), 0, stream, p);
   else
     hipLaunchKernelGGL(dmq_route_small_kernel<float>, dim3(1), dim3(1024), 0, stream, p);
+  return dmq_check_launch();
+}
+
+int dmq_route_rank_launch(const RouteRankParams& p, hipStream_t stream) {
+  if (p.rows <= 0 || p.rows > DMQ_ROUTE_RANK_ROWS || p.k <= 0 || p.tile_rows <= 0) return DMQ_ERR_LIMIT;
+  if (p.pools <= 0 || p.pools > DMQ_MAX_POOLS || p.experts <= 0) return DMQ_ERR_LIMIT;
+  hipLaunchKernelGGL(dmq_route_rank_kernel, dim3(1), dim3(256), 0, stream, p);
   return dmq_check_launch();
 }
 

@@ -352,6 +352,30 @@ def test_few_tokens_routing_matches_the_sorted_path(shared_layer, mode):
     assert torch.equal(four_topk, four)
 
 
+@pytest.mark.parametrize("mode", ["wxa16", "wxfp8"])
+def test_ranking_kernel_matches_the_counting_sort(small_layer, mode):
+    """Up to 128 routed rows are routed by the one-row-per-thread ranking kernel, more by the
+    counting sort: 32 tokens (128 rows) alone and as the first 32 of 33 tokens must give the same
+    bits (experts with more than 16 rows: several row tiles per expert)."""
+    from dartmoq_hip import ops
+    layer = small_layer
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(33, layer.hidden, generator=g).half().cuda()
+    logits = routing.zipf_logits(33, layer.num_experts, 4).cuda()
+    mod = make_module(layer, mode)
+    mod.tt_override = 1
+    mod.ks_override = 1
+    big = mod.forward(x, router_logits=logits).clone()
+    small = mod.forward(x[:32].contiguous(), router_logits=logits[:32].contiguous()).clone()
+    assert torch.equal(small, big[:32])
+    w, idx = ops.route_topk(logits[:32].contiguous(), layer.top_k)
+    assert int(torch.bincount(idx.flatten().cpu().long()).max()) > 16
+    from_topk = mod.forward(x[:32].contiguous(), topk_idx=idx, topk_w=w)
+    assert torch.equal(from_topk, small)
+    ideal = moe.quantized_forward(layer, x[:32].cpu(), idx.cpu().long(), w.cpu(), mode)
+    assert relerr(small.float().cpu(), ideal) < {"wxa16": 3e-3, "wxfp8": 2e-2}[mode]
+
+
 def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):

@@ -285,6 +285,21 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     arow[t] = pw.act + (long)rphys[t] * p.act_row_bytes + q * (AW * 4) + in_group0 * AB;
   }
 
+  // scatter epilogue: routing weight and destination row of the lane's rows, requested now so that
+  // the epilogue does not end on a memory round trip (rows past the item take its last row's)
+  float row_w[TT];
+  int row_dst[TT];
+#pragma unroll
+  for (int t = 0; t < TT; ++t) { row_w[t] = 0.f; row_dst[t] = 0; }
+  if constexpr (EPI == DMQ_EPI_SCATTER) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      const int rr = min(rlog[t], r_end - 1);
+      row_w[t] = p.row_weight[rr];
+      row_dst[t] = p.row_slot[rr];
+    }
+  }
+
   float4_t total_acc[NT][TT];
 #pragma unroll
   for (int j = 0; j < NT; ++j)
@@ -468,9 +483,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
             h[r] = (_Float16)(dmq_silu(total_acc[j][t][r]) * total_acc[j + 1][t][r]);
           *(half4_t*)(p.out + (long)rlog[t] * p.out_stride + out_col0 + feat_k + (j >> 1) * 16 + 4 * q) = h;
         } else {
-          const float rw = p.row_weight[rlog[t]];
-          float4_t v = total_acc[j][t] * rw;
-          half4_t* dst = (half4_t*)(p.out_slots + (long)p.row_slot[rlog[t]] * p.out_stride + feat_k + j * 16 + 4 * q);
+          float4_t v = total_acc[j][t] * row_w[t];
+          half4_t* dst = (half4_t*)(p.out_slots + (long)row_dst[t] * p.out_stride + feat_k + j * 16 + 4 * q);
           if (p.accumulate) {                  // a further share of the expert: add to what is there
             const half4_t prev = *dst;
             v += (float4_t){(float)prev[0], (float)prev[1], (float)prev[2], (float)prev[3]};

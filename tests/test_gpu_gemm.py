@@ -57,7 +57,7 @@ def _mode_inputs(mode, x_rot, cb):
             luts.e2m1_value(nib), 2.0 ** e0, resid, 127 + e0)
 
 
-def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed):
+def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed, roomy=0):
     from dartmoq_hip import ops
     n_exp = len(counts)
     starts, rows_total = _expert_rows(counts)
@@ -93,7 +93,8 @@ def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed):
     out = ops.matmul_merged(
         mode, bit, STORE, act.cuda(), None if scale is None else scale.cuda(), w_dev,
         norms_used.cuda(), None if mode == FP4 else lut.cuda(), info_dev, groups=k // 128,
-        n_out=n_slice, slice_is_groups=slice_is_groups, rows_total=rows_total, w_scale_byte=wsb, tt=tt)
+        n_out=n_slice, slice_is_groups=slice_is_groups, rows_total=rows_total, w_scale_byte=wsb, tt=tt,
+        roomy=roomy)
     torch.cuda.synchronize()
     return out.cpu().float(), ref
 
@@ -107,6 +108,20 @@ def test_merged_rows_gate_up(mode, bit, tt):
                          seed=100 + 10 * mode + bit)
     # only the fp16 rounding of the output (and fp32 summation order) separates the two
     torch.testing.assert_close(out, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("mode", [A16, A8, FP8])
+@pytest.mark.parametrize("bit", [1, 2, 4])
+def test_two_per_cu_instance_gives_the_same_bits(mode, bit):
+    """16-row tiles have a second kernel instance (two waves per SIMD, registers instead of scratch
+    for the 4-bit weight ring): same arithmetic, so the same bits."""
+    counts = [3, 0, 17, 64, 1, 130]
+    lean, ref = _run_case(mode, bit, 1, counts, k=512, n_slice=128, slice_is_groups=False,
+                          seed=100 + 10 * mode + bit)
+    roomy, _ = _run_case(mode, bit, 1, counts, k=512, n_slice=128, slice_is_groups=False,
+                         seed=100 + 10 * mode + bit, roomy=1)
+    assert torch.equal(lean, roomy)
+    torch.testing.assert_close(roomy, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
 
 
 @pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])

@@ -376,6 +376,21 @@ def test_ranking_kernel_matches_the_counting_sort(small_layer, mode):
     assert relerr(small.float().cpu(), ideal) < {"wxa16": 3e-3, "wxfp8": 2e-2}[mode]
 
 
+@pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp4"])
+@pytest.mark.parametrize("tokens", [1, 5, 31])
+def test_pools_of_a_single_group(mode, tokens):
+    """Three experts, top-1, I = 128: every pool holds one or two experts, the down matrix of a
+    one-expert pool is a single group (the quantizer then returns its norms as a vector), the
+    shared expert is one 128-wide slice."""
+    layer = moe.build_layer(384, 128, 3, 1, [4, 2, 2], seed=11)
+    layer = moe.add_shared_expert(layer, 128, seed=12, bit=2)
+    assert layer.pools["4"].down["norms"].dim() == 1
+    x, idx, w, out = _run(layer, mode, tokens, seed=tokens)
+    ideal = moe.quantized_forward(layer, x, idx, w, mode)
+    tight = {"wxa16": 3e-3, "wxa8": 8e-3, "wxfp4": 7e-2}[mode]
+    assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
+
+
 def test_cpu_input_fails_loudly(small_layer):
     mod = make_module(small_layer, "wxa16")
     with pytest.raises(RuntimeError):

@@ -69,6 +69,7 @@ struct QuantParams {
 // multiple of 64 rows.
 #define DMQ_SORT_MAX_EXPERTS 2048
 #define DMQ_SORT_MAX_CHUNKS 64
+#define DMQ_FUSED_FILL_EXPERTS 512      // planning and scatter share a launch up to this many experts
 static inline void dmq_sort_chunks(long rows, int* chunk_rows, int* n_chunks) {
   long cr = (rows + DMQ_SORT_MAX_CHUNKS - 1) / DMQ_SORT_MAX_CHUNKS;
   cr = (cr + 63) / 64 * 64;

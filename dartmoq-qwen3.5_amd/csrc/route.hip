@@ -8,6 +8,7 @@
 //                             of every (chunk, expert), per-pool expert_info and the work-item
 //                             list (pool, expert, row tile) of the layer
 //   4. dmq_chunk_fill_kernel  one wave per chunk: write its rows to their sorted positions
+//      (up to DMQ_FUSED_FILL_EXPERTS experts steps 3 and 4 are one launch, dmq_plan_fill_kernel)
 //   5. dmq_combine_kernel     out[t] = sum over the k slot rows of token t (fixed order)
 #include "params.h"
 #include "topk.h"
@@ -52,45 +53,67 @@ void dmq_chunk_count_kernel(const int* topk_idx, int rows, int experts, int chun
   __builtin_amdgcn_wave_barrier();
   const int r0 = c * chunk_rows;
   const int r1 = min(rows, r0 + chunk_rows);
-  for (int r = r0 + lane; r < r1; r += 64) {
-    const int e = topk_idx[r];
-    if (e >= 0 && e < experts) atomicAdd(&cnt[e], 1);
+  for (int base = r0; base < r1; base += 64 * 8) {      // eight steps of 64 rows per round trip
+    int ev[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = base + 64 * i + lane;
+      ev[i] = (r < r1) ? topk_idx[r] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (ev[i] >= 0 && ev[i] < experts) atomicAdd(&cnt[ev[i]], 1);
   }
   __builtin_amdgcn_wave_barrier();
   for (int e = lane; e < experts; e += 64) hist[(long)c * experts + e] = cnt[e];
+}
+
+// Inclusive scan over the 64 lanes of a wave with data-parallel lane moves: shifts by 1, 2, 4 and
+// 8 inside the rows of 16 lanes, then lane 15 of rows 0 and 2 added to rows 1 and 3 and lane 31 to
+// the upper half (a lane with no source adds zero).
+__device__ __forceinline__ int wave_scan_incl(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);        // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);        // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);        // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);        // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);        // row_bcast:15 into rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);        // row_bcast:31 into rows 2, 3
+  return v;
 }
 
 // inclusive scan over the 1024 threads of the workgroup (16 waves)
 __device__ __forceinline__ int block_scan_incl(int v, int* wave_tot) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    int o = __shfl_up(v, d, 64);
-    if (lane >= d) v += o;
-  }
+  v = wave_scan_incl(v);
   if (lane == 63) wave_tot[wave] = v;
   __syncthreads();
-  int add = 0;
-  for (int w = 0; w < wave; ++w) add += wave_tot[w];
+  int add = 0;                                          // all 16 totals requested at once
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const int t = wave_tot[w];
+    add += (w < wave) ? t : 0;
+  }
   __syncthreads();
   return v + add;
 }
 
-// 64-bit variant of the scan: four 16-bit fields scanned at once
+// 64-bit variant of the scan: four 16-bit fields scanned at once (no field overflows, so the two
+// halves of the word are scanned on their own)
 __device__ __forceinline__ unsigned long long block_scan_incl_u64(unsigned long long v,
                                                                   unsigned long long* wave_tot) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const unsigned long long o = __shfl_up(v, d, 64);
-    if (lane >= d) v += o;
-  }
+  v = (unsigned long long)(unsigned)wave_scan_incl((int)(unsigned)v) |
+      ((unsigned long long)(unsigned)wave_scan_incl((int)(unsigned)(v >> 32)) << 32);
   if (lane == 63) wave_tot[wave] = v;
   __syncthreads();
   unsigned long long add = 0;
-  for (int w = 0; w < wave; ++w) add += wave_tot[w];
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const unsigned long long t = wave_tot[w];
+    add += (w < wave) ? t : 0ull;
+  }
   return v + add;
 }
 
@@ -122,7 +145,7 @@ __device__ __forceinline__ PlanSlices plan_load_slices(const PlanParams& p) {
 __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* s_cnt, const int* s_off,
                                                 int* wave_tot, unsigned long long* wave_tot64,
                                                 int* carry_p, const PlanSlices& pre_s,
-                                                int* item_first = nullptr) {
+                                                int* item_first = nullptr, int* item_ss = nullptr) {
   const int tid = threadIdx.x;
   const bool pre = p.experts <= 1024;
   if (pre && p.max_items < 65536) {
@@ -159,7 +182,10 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
       for (int o = 0; o < DMQ_MAX_POOLS; ++o) {
         if (o < p.pools) {
           const int pool = p.pool_order[o];
-          if (live) item_first[o * p.experts + e] = base + (int)((incl >> (16 * pool)) & 0xffffu) - pick4(ntile, pool);
+          if (live) {
+            item_first[o * p.experts + e] = base + (int)((incl >> (16 * pool)) & 0xffffu) - pick4(ntile, pool);
+            item_ss[o * p.experts + e] = pick4(pre_s.ss, pool);
+          }
           base += (int)((totals >> (16 * pool)) & 0xffffu);
           if (o + 1 == p.lead_pools) lead = base;
         }
@@ -177,7 +203,7 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
         const int o = idx / p.experts;
         const int ex = idx - o * p.experts;
         const int pool = p.pool_order[o];
-        const int ss = p.slice_start_rows[pool * p.experts + ex];
+        const int ss = item_ss[idx];
         int4_t* it = (int4_t*)(p.items + (long)DMQ_ITEM_WORDS * i);
         it[0] = (int4_t){pool, ex, i - item_first[idx], s_off[ex]};
         it[1] = (int4_t){s_cnt[ex], ss >= 0 ? ss : 0, ss >= 0 ? ss / (2 * DMQ_GS) : 0, 0};
@@ -255,8 +281,10 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
   }
 }
 
-__global__ __launch_bounds__(1024)
-void dmq_plan_kernel(PlanParams p) {
+// POSITIONS: also turn hist[c, e] into the position of the first row of chunk c routed to expert e
+// (for dmq_chunk_fill_kernel); without it the histogram is only read.
+template <bool POSITIONS>
+__device__ __forceinline__ void plan_body(const PlanParams& p) {
   // counts and offsets live in LDS between the phases; global memory is only written, so the
   // kernel pays one round trip for the histogram and one for the slice tables
   __shared__ int wave_tot[16];
@@ -266,6 +294,7 @@ void dmq_plan_kernel(PlanParams p) {
   __shared__ int s_off[DMQ_SORT_MAX_EXPERTS + 1];
   __shared__ unsigned long long wave_tot64[17];
   __shared__ int item_first[DMQ_MAX_POOLS * 1024];
+  __shared__ int item_ss[DMQ_MAX_POOLS * 1024];
   const int tid = threadIdx.x;
   if (tid == 0) carry = 0;
   const PlanSlices slices = plan_load_slices(p);       // in flight during the counting phases
@@ -323,7 +352,7 @@ void dmq_plan_kernel(PlanParams p) {
   if (tid == 0) { s_off[0] = 0; p.offsets[0] = 0; }
   __syncthreads();
   // hist[c, e] <- position of the first row of chunk c routed to expert e
-  for (int ebase = 0; ebase < p.experts; ebase += epad) {
+  for (int ebase = 0; POSITIONS && ebase < p.experts; ebase += epad) {
     const int e = ebase + el;
     if (!one_pass) {
       partial[tid] = chunk_sum(e);
@@ -343,8 +372,11 @@ void dmq_plan_kernel(PlanParams p) {
     }
     if (!one_pass) __syncthreads();
   }
-  plan_emit_items(p, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices, item_first);
+  plan_emit_items(p, s_cnt, s_off, wave_tot, wave_tot64, &carry, slices, item_first, item_ss);
 }
+
+__global__ __launch_bounds__(1024)
+void dmq_plan_kernel(PlanParams p) { plan_body<true>(p); }
 
 // Stable scatter of one chunk.  The rows of one token name distinct experts, so the lanes of a
 // token bump distinct counters; tokens are taken one after the other and LDS executes a wave's
@@ -380,6 +412,180 @@ void dmq_chunk_fill_kernel(const int* topk_idx, const float* topk_w, int rows, i
       sorted_tokens[at] = tok;
       sorted_weights[at] = w;
       sorted_rows[at] = r;
+    }
+  }
+}
+
+// Planning and scatter in one launch (layers of at most DMQ_FUSED_FILL_EXPERTS experts): the last
+// workgroup writes counts, offsets, expert_info and the work-item list from the chunk histogram,
+// the others scatter DMQ_FILL_CHUNKS chunks each (one per wave: the scattered stores of more waves
+// would queue up in one CU's memory pipeline) and derive the start positions of their chunks
+// from the same histogram themselves, all 16 waves helping: rows of expert e in earlier chunks
+// plus rows of all experts below e.  Nothing waits for the planning workgroup, and the histogram
+// is only read.
+#define DMQ_FILL_CHUNKS 4
+struct FillParams {
+  const int* topk_idx;
+  const float* topk_w;
+  int rows, k;
+  int* sorted_tokens;
+  float* sorted_weights;
+  int* sorted_rows;
+};
+
+__global__ __launch_bounds__(1024)
+void dmq_plan_fill_kernel(PlanParams p, FillParams f) {
+  const int fill_blocks = (p.n_chunks + DMQ_FILL_CHUNKS - 1) / DMQ_FILL_CHUNKS;
+  if ((int)blockIdx.x >= fill_blocks) {
+    plan_body<false>(p);
+    return;
+  }
+  constexpr int EMAX = DMQ_FUSED_FILL_EXPERTS;
+  constexpr int CPB = DMQ_FILL_CHUNKS;
+  __shared__ int own[CPB * EMAX];          // histogram rows of the block's chunks, then their positions
+  __shared__ int idle_all[CPB * 64];
+  __shared__ int part_all[1024], part_before[1024];
+  __shared__ int wave_tot[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int experts = p.experts;
+  const int c0 = blockIdx.x * CPB;
+  const int c = c0 + wave;
+  if (wave < CPB) {
+    for (int e = lane; e < experts; e += 64)
+      own[wave * EMAX + e] = (c < p.n_chunks) ? p.hist[(long)c * experts + e] : 0;
+  }
+  // column sums of the histogram: all chunks, and the chunks in front of this block
+  int epad = 64;
+  while (epad < experts) epad <<= 1;
+  const int parts = 1024 / epad;
+  const int part = tid / epad, el = tid % epad;
+  const int cpp = (p.n_chunks + parts - 1) / parts;
+  const int c_lo = part * cpp;
+  const int c_hi = min(p.n_chunks, c_lo + cpp);
+  int all = 0, before = 0;
+  for (int cc = c_lo; cc < c_hi; cc += 16) {
+    int h[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      h[i] = (el < experts && cc + i < c_hi) ? p.hist[(long)(cc + i) * experts + el] : 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      all += h[i];
+      before += (cc + i < c0) ? h[i] : 0;
+    }
+  }
+  // the first PRE steps of 64 rows of the wave's chunk are requested now, so that their memory
+  // latency passes during the scans
+  constexpr int PRE = 8;
+  const int r0 = c * p.chunk_rows;
+  const int r1 = (wave < CPB && c < p.n_chunks) ? min(f.rows, r0 + p.chunk_rows) : r0;
+  int pre_e[PRE];
+  float pre_w[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    const int r = r0 + 64 * i + lane;
+    pre_e[i] = (r < r1) ? f.topk_idx[r] : -1;
+    pre_w[i] = (r < r1) ? f.topk_w[r] : 0.f;
+  }
+  part_all[tid] = all;
+  part_before[tid] = before;
+  __syncthreads();
+  int tot = 0, bef = 0;
+  if (tid < experts) {
+    for (int q = 0; q < parts; ++q) {
+      tot += part_all[q * epad + tid];
+      bef += part_before[q * epad + tid];
+    }
+  }
+  const int incl = block_scan_incl(tot, wave_tot);
+  // thread e walks the block's chunks of expert e: own[j][e] <- position of the first row of
+  // chunk c0 + j routed to e (rows of the experts below e, rows of e in earlier chunks)
+  if (tid < experts) {
+    int at = incl - tot + bef;
+    int h[CPB];
+#pragma unroll
+    for (int j = 0; j < CPB; ++j) h[j] = own[j * EMAX + tid];
+#pragma unroll
+    for (int j = 0; j < CPB; ++j) {
+      own[j * EMAX + tid] = at;
+      at += h[j];
+    }
+  }
+  __syncthreads();
+  if (wave >= CPB || c >= p.n_chunks) return;
+  int* pos = own + wave * EMAX;
+  // Rows of one token name distinct experts, rows of different tokens may share one: the lanes of
+  // token j of the step bump the counters in the j-th of a fixed number of operations (LDS executes
+  // a wave's operations in order; the other lanes add zero to a word of their own, so the code has
+  // no branches and nothing waits for a result before all operations of a step are requested).
+  const int k = f.k;
+  constexpr int TOKS = 9;                                // tokens a step of 64 rows touches when k >= 8
+  int* idle = idle_all + wave * 64 + lane;
+  auto rank_fast = [&](int e, int tj) {
+    const bool hit = e >= 0 && e < experts;
+    int* mine = hit ? pos + e : idle;
+    int res[TOKS];
+#pragma unroll
+    for (int j = 0; j < TOKS; ++j) {
+      const bool on = hit && tj == j;
+      res[j] = atomicAdd(on ? mine : idle, on ? 1 : 0);
+    }
+    int at = -1;
+#pragma unroll
+    for (int j = 0; j < TOKS; ++j) at = (hit && tj == j) ? res[j] : at;
+    return at;
+  };
+  auto rank_any = [&](int base, int e, int tok) {
+    const bool hit = e >= 0 && e < experts;
+    const int tok_first = base / k;
+    const int tok_last = (min(base + 64, r1) - 1) / k;
+    int at = -1;
+    for (int t = tok_first; t <= tok_last; ++t)
+      if (hit && tok == t) at = atomicAdd(&pos[e], 1);
+    return at;
+  };
+  auto put = [&](int r, int tok, int at, float w) {
+    if (at >= 0) {
+      f.sorted_tokens[at] = tok;
+      f.sorted_weights[at] = w;
+      f.sorted_rows[at] = r;
+    }
+  };
+  // token of the lane's row, advanced by 64 rows per step without dividing again
+  const int q64 = 64 / k, m64 = 64 % k;
+  int tok = (r0 + lane) / k, rem = (r0 + lane) % k;
+  auto advance = [&]() {
+    tok += q64; rem += m64;
+    if (rem >= k) { rem -= k; ++tok; }
+  };
+  if (k >= 8) {
+    int at[PRE], tk[PRE];
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+      tk[i] = tok;
+      at[i] = (r0 + 64 * i < r1) ? rank_fast(pre_e[i], tok - __builtin_amdgcn_readfirstlane(tok)) : -1;
+      advance();
+    }
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) put(r0 + 64 * i + lane, tk[i], at[i], pre_w[i]);
+    for (int base = r0 + 64 * PRE; base < r1; base += 64) {
+      const int r = base + lane;
+      const bool in = r < r1;
+      const int at1 = rank_fast(in ? f.topk_idx[r] : -1, tok - __builtin_amdgcn_readfirstlane(tok));
+      put(r, tok, at1, in ? f.topk_w[r] : 0.f);
+      advance();
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+      if (r0 + 64 * i < r1) put(r0 + 64 * i + lane, tok, rank_any(r0 + 64 * i, pre_e[i], tok), pre_w[i]);
+      advance();
+    }
+    for (int base = r0 + 64 * PRE; base < r1; base += 64) {
+      const int r = base + lane;
+      const bool in = r < r1;
+      put(r, tok, rank_any(base, in ? f.topk_idx[r] : -1, tok), in ? f.topk_w[r] : 0.f);
+      advance();
     }
   }
 }
@@ -673,6 +879,13 @@ int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int token
   const int grid_c = (plan.n_chunks + 3) / 4;
   hipLaunchKernelGGL(dmq_chunk_count_kernel, dim3(grid_c), dim3(256), 0, stream, topk_idx, rows,
                      experts, plan.chunk_rows, plan.n_chunks, plan.hist);
+  if (experts <= DMQ_FUSED_FILL_EXPERTS) {
+    const FillParams f{topk_idx, topk_w, rows, k, sorted_tokens, sorted_weights, sorted_rows};
+    hipLaunchKernelGGL(dmq_plan_fill_kernel,
+                       dim3((plan.n_chunks + DMQ_FILL_CHUNKS - 1) / DMQ_FILL_CHUNKS + 1), dim3(1024), 0, stream,
+                       plan, f);
+    return dmq_check_launch();
+  }
   hipLaunchKernelGGL(dmq_plan_kernel, dim3(1), dim3(1024), 0, stream, plan);
   hipLaunchKernelGGL(dmq_chunk_fill_kernel, dim3(grid_c), dim3(256), 0, stream, topk_idx, topk_w,
                      rows, k, experts, plan.chunk_rows, plan.n_chunks, plan.hist, sorted_tokens,

@@ -87,11 +87,11 @@ def test_permute_matches_oracle(tokens, tile_rows):
 
 @pytest.mark.parametrize("tokens,experts,k", [(700, 100, 3), (1000, 37, 1), (333, 300, 5), (5000, 256, 8),
                                                    (113, 257, 9), (128, 512, 8), (60, 513, 8), (129, 512, 8),
-                                                   (2100, 600, 8)])
+                                                   (2100, 600, 8), (900, 1100, 6)])
 def test_permute_odd_shapes(tokens, experts, k):
     """Tokens whose k rows straddle the 64-row steps of the sort, expert counts off the wave size;
-    the last case has a chunk histogram too big for the planning kernel to build in LDS, so the
-    separate counting launch runs."""
+    the cases with more than 512 experts take the separate planning and scatter launches, the
+    others the launch that does both."""
     from dartmoq_hip import ops
     logits = routing.zipf_logits(tokens, experts, seed=7 * tokens + k)
     w, idx = routing.route_topk(logits, k)

@@ -101,19 +101,22 @@ __device__ __forceinline__ int block_scan_incl(int v, int* wave_tot) {
 // 64-bit variant of the scan: four 16-bit fields scanned at once (no field overflows, so the two
 // halves of the word are scanned on their own)
 __device__ __forceinline__ unsigned long long block_scan_incl_u64(unsigned long long v,
-                                                                  unsigned long long* wave_tot) {
+                                                                  unsigned long long* wave_tot,
+                                                                  unsigned long long* total) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   v = (unsigned long long)(unsigned)wave_scan_incl((int)(unsigned)v) |
       ((unsigned long long)(unsigned)wave_scan_incl((int)(unsigned)(v >> 32)) << 32);
   if (lane == 63) wave_tot[wave] = v;
   __syncthreads();
-  unsigned long long add = 0;
+  unsigned long long add = 0, all = 0;
 #pragma unroll
   for (int w = 0; w < 16; ++w) {
     const unsigned long long t = wave_tot[w];
     add += (w < wave) ? t : 0ull;
+    all += t;
   }
+  *total = all;
   return v + add;
 }
 
@@ -149,6 +152,8 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
   const int tid = threadIdx.x;
   const bool pre = p.experts <= 1024;
   if (pre && p.max_items < 65536) {
+    const bool tile_pow2 = (p.tile_rows & (p.tile_rows - 1)) == 0;
+    const int tile_shift = __builtin_ctz((unsigned)p.tile_rows);
     const int e = tid;
     const bool live = e < p.experts;
     const int ts = live ? s_off[e] : 0;
@@ -161,7 +166,7 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
         const int ss = pre_s.ss[pool], sc = pre_s.sc[pool];
         const int tc = (ss >= 0) ? s_cnt[e] : 0;
         tcs[pool] = tc;
-        ntile[pool] = (tc + p.tile_rows - 1) / p.tile_rows;
+        ntile[pool] = tile_pow2 ? (tc + p.tile_rows - 1) >> tile_shift : (tc + p.tile_rows - 1) / p.tile_rows;
         packed |= (unsigned long long)ntile[pool] << (16 * pool);
         int4_t* gi = (int4_t*)(p.gu_info + ((long)pool * p.experts + e) * 4);
         *gi = (int4_t){ts, tc, ss >= 0 ? ss : 0, sc};
@@ -169,10 +174,8 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
         *di = (int4_t){ts, tc, ss >= 0 ? ss / (2 * DMQ_GS) : 0, sc / (2 * DMQ_GS)};
       }
     }
-    const unsigned long long incl = block_scan_incl_u64(packed, wave_tot64);
-    if (tid == 1023) wave_tot64[16] = incl;            // per-pool totals
-    __syncthreads();
-    const unsigned long long totals = wave_tot64[16];
+    unsigned long long totals;                         // per-pool totals
+    const unsigned long long incl = block_scan_incl_u64(packed, wave_tot64, &totals);
     int base = 0, lead = 0;
     if (item_first) {
       // Long batches: an expert with many rows has many tiles, so the records are written one
@@ -604,6 +607,7 @@ void dmq_route_small_kernel(RouteSmallParams p) {
   __shared__ int s_hist[16 * DMQ_ROUTE_SMALL_EXPERTS];
   __shared__ int s_idx[DMQ_ROUTE_SMALL_ROWS];
   __shared__ float s_w[DMQ_ROUTE_SMALL_ROWS];
+  __shared__ int s_idle[1024];
   __shared__ unsigned long long wave_tot64[17];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -647,7 +651,36 @@ void dmq_route_small_kernel(RouteSmallParams p) {
       }
     }
   };
-  if (!p.logits || p.router_experts <= 256) tokens_of_wave(std::integral_constant<int, 4>{});
+  if (!p.logits) {
+    // a caller-made top-k: one routed row per thread (rows <= 1024), one round trip for all of them;
+    // the shared columns four tokens at a time per wave
+    if (tid < rows) {
+      const int tok = tid / kt, j = tid - tok * kt;
+      if (j < k) {
+        const float w = p.in_w[(long)tok * k + j];
+        const int e = p.in_idx[(long)tok * k + j];
+        s_idx[tid] = e;
+        s_w[tid] = w;
+        if (p.out_w) { p.out_w[tid] = w; p.out_idx[tid] = e; }
+      }
+    }
+    if (p.sg.n_shared > 0) {
+      for (int tok0 = wave; tok0 < p.tokens; tok0 += 64) {
+        float g[4];
+        dmq_shared_gate_values4(p.sg, tok0, 16, p.tokens, lane, g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = tok0 + 16 * i;
+          if (tok < p.tokens && lane >= k && lane < kt) {
+            const int e = p.router_experts + (lane - k);
+            s_idx[tok * kt + lane] = e;
+            s_w[tok * kt + lane] = g[i];
+            if (p.out_w) { p.out_w[(long)tok * kt + lane] = g[i]; p.out_idx[(long)tok * kt + lane] = e; }
+          }
+        }
+      }
+    }
+  } else if (p.router_experts <= 256) tokens_of_wave(std::integral_constant<int, 4>{});
   else if (p.router_experts <= 512) tokens_of_wave(std::integral_constant<int, 8>{});
   else tokens_of_wave(std::integral_constant<int, 16>{});
   __syncthreads();
@@ -693,8 +726,22 @@ void dmq_route_small_kernel(RouteSmallParams p) {
     const int tok_first = base / kt;
     const int tok_last = (min(base + 64, rows) - 1) / kt;
     int at = -1;
-    for (int t = tok_first; t <= tok_last; ++t) {
-      if (hit && tok == t) at = atomicAdd(&my_hist[e_r], 1);
+    if (kt >= 8) {
+      // at most nine tokens in the wave's 64 rows: one operation per token, issued back to back
+      // (lanes of other tokens add zero to a word of their own)
+      int* idle = s_idle + tid;
+      int res[9];
+#pragma unroll
+      for (int j = 0; j < 9; ++j) {
+        const bool on = hit && tok - tok_first == j;
+        res[j] = atomicAdd(on ? &my_hist[e_r] : idle, on ? 1 : 0);
+      }
+#pragma unroll
+      for (int j = 0; j < 9; ++j) at = (hit && tok - tok_first == j) ? res[j] : at;
+    } else {
+      for (int t = tok_first; t <= tok_last; ++t) {
+        if (hit && tok == t) at = atomicAdd(&my_hist[e_r], 1);
+      }
     }
     if (at >= 0) {
       p.sorted_tokens[at] = tok;

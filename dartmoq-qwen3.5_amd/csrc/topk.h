@@ -48,6 +48,34 @@ __device__ __forceinline__ float dmq_shared_gate_value(const SharedGate& sg, int
   return (float)(_Float16)(1.f / (1.f + expf(-z)));
 }
 
+// The same value for four tokens tok0, tok0 + step, ... at once (their rows are requested together);
+// every token sees the arithmetic of dmq_shared_gate_value in the same order.
+__device__ __forceinline__ void dmq_shared_gate_values4(const SharedGate& sg, int tok0, int step, int tokens,
+                                                        int lane, float (&g)[4]) {
+  float dot[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int h = lane * 8; h < sg.hidden; h += 512) {
+    const half8_t b = *(const half8_t*)(sg.gate_row + h);
+    half8_t a[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int tok = min(tok0 + i * step, tokens - 1);
+      a[i] = *(const half8_t*)(sg.x + (long)tok * sg.hidden + h);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) dot[i] += (float)a[i][c] * (float)b[c];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float d = dot[i];
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) d += __shfl_xor(d, m, 64);
+    const float z = (float)(_Float16)d;
+    g[i] = (float)(_Float16)(1.f / (1.f + expf(-z)));
+  }
+}
+
 __device__ __forceinline__ void dmq_shared_columns(const SharedGate& sg, int tok, int experts, int k,
                                                    int lane, float* out_w, int* out_idx) {
   if (sg.n_shared <= 0) return;

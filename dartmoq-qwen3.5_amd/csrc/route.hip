@@ -8,7 +8,8 @@
 //                             of every (chunk, expert), per-pool expert_info and the work-item
 //                             list (pool, expert, row tile) of the layer
 //   4. dmq_chunk_fill_kernel  one wave per chunk: write its rows to their sorted positions
-//      (up to DMQ_FUSED_FILL_EXPERTS experts steps 3 and 4 are one launch, dmq_plan_fill_kernel)
+//      (up to DMQ_FUSED_FILL_EXPERTS experts steps 3 and 4 are one launch, dmq_plan_fill_kernel,
+//      which up to DMQ_FILL_COUNT_ROWS routed rows also counts and so replaces step 2)
 //   5. dmq_combine_kernel     out[t] = sum over the k slot rows of token t (fixed order)
 #include "params.h"
 #include "topk.h"
@@ -286,8 +287,11 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
 
 // POSITIONS: also turn hist[c, e] into the position of the first row of chunk c routed to expert e
 // (for dmq_chunk_fill_kernel); without it the histogram is only read.
+// count_idx != NULL: the rows per expert are counted from the routed rows themselves (no chunk
+// histogram is read; at most 16 rows per thread: count_rows <= 16384).
 template <bool POSITIONS>
-__device__ __forceinline__ void plan_body(const PlanParams& p) {
+__device__ __forceinline__ void plan_body(const PlanParams& p, const int* count_idx = nullptr,
+                                          int count_rows = 0) {
   // counts and offsets live in LDS between the phases; global memory is only written, so the
   // kernel pays one round trip for the histogram and one for the slice tables
   __shared__ int wave_tot[16];
@@ -328,8 +332,32 @@ __device__ __forceinline__ void plan_body(const PlanParams& p) {
     }
     return sum;
   };
+  if (count_idx) {
+    // sixteen rows per thread and round trip, each into a counter array of its own: the rows of a
+    // popular expert then meet at sixteen addresses instead of one (experts <= DMQ_FUSED_FILL_EXPERTS)
+    __shared__ int cnt16[16 * DMQ_FUSED_FILL_EXPERTS];
+    for (int i = tid; i < 16 * DMQ_FUSED_FILL_EXPERTS; i += 1024) cnt16[i] = 0;
+    int ev[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = 1024 * i + tid;
+      ev[i] = (r < count_rows) ? count_idx[r] : -1;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (ev[i] >= 0 && ev[i] < p.experts) atomicAdd(&cnt16[i * DMQ_FUSED_FILL_EXPERTS + ev[i]], 1);
+    __syncthreads();
+    if (tid < p.experts) {
+      int total = 0;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) total += cnt16[i * DMQ_FUSED_FILL_EXPERTS + tid];
+      s_cnt[tid] = total;
+      p.counts[tid] = total;
+    }
+  }
   // rows per expert: column sums of the chunk histogram
-  for (int ebase = 0; ebase < p.experts; ebase += epad) {
+  for (int ebase = 0; !count_idx && ebase < p.experts; ebase += epad) {
     const int e = ebase + el;
     partial[tid] = chunk_sum(e);
     __syncthreads();
@@ -419,14 +447,19 @@ void dmq_chunk_fill_kernel(const int* topk_idx, const float* topk_w, int rows, i
   }
 }
 
-// Planning and scatter in one launch (layers of at most DMQ_FUSED_FILL_EXPERTS experts): the last
-// workgroup writes counts, offsets, expert_info and the work-item list from the chunk histogram,
-// the others scatter DMQ_FILL_CHUNKS chunks each (one per wave: the scattered stores of more waves
-// would queue up in one CU's memory pipeline) and derive the start positions of their chunks
-// from the same histogram themselves, all 16 waves helping: rows of expert e in earlier chunks
-// plus rows of all experts below e.  Nothing waits for the planning workgroup, and the histogram
-// is only read.
+// Planning and scatter in one launch (layers of at most DMQ_FUSED_FILL_EXPERTS experts).  The last
+// workgroup writes counts, offsets, expert_info and the work-item list; the others scatter
+// DMQ_FILL_CHUNKS chunks each (one per wave: the scattered stores of more waves would queue up in
+// one CU's memory pipeline) and derive the start positions of their chunks themselves, all 16
+// waves helping: rows of the experts below e, rows of e in earlier chunks.  Nothing waits for
+// another workgroup.
+//   COUNT (at most DMQ_FILL_COUNT_ROWS routed rows): straight from the top-k arrays, no histogram
+//     launch in front and nothing in global memory between the two: every workgroup counts all
+//     routed rows itself (16 per thread, one round trip), per expert and group of DMQ_FILL_CHUNKS
+//     chunks.  One CU's LDS takes ~1 us per 16384 atomic adds, so beyond that size
+//   !COUNT reads the chunk histogram of dmq_chunk_count_kernel, which 16 CUs build together.
 #define DMQ_FILL_CHUNKS 4
+#define DMQ_FILL_COUNT_ROWS (1024 * 16)
 struct FillParams {
   const int* topk_idx;
   const float* topk_w;
@@ -436,68 +469,116 @@ struct FillParams {
   int* sorted_rows;
 };
 
+template <bool COUNT>
 __global__ __launch_bounds__(1024)
 void dmq_plan_fill_kernel(PlanParams p, FillParams f) {
   const int fill_blocks = (p.n_chunks + DMQ_FILL_CHUNKS - 1) / DMQ_FILL_CHUNKS;
   if ((int)blockIdx.x >= fill_blocks) {
-    plan_body<false>(p);
+    if constexpr (COUNT) plan_body<false>(p, f.topk_idx, f.rows);
+    else plan_body<false>(p);
     return;
   }
   constexpr int EMAX = DMQ_FUSED_FILL_EXPERTS;
   constexpr int CPB = DMQ_FILL_CHUNKS;
-  __shared__ int own[CPB * EMAX];          // histogram rows of the block's chunks, then their positions
+  constexpr int GMAX = DMQ_SORT_MAX_CHUNKS / CPB;
+  __shared__ int own[CPB * EMAX];          // rows per (chunk of the block, expert), then their positions
   __shared__ int idle_all[CPB * 64];
-  __shared__ int part_all[1024], part_before[1024];
   __shared__ int wave_tot[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int experts = p.experts;
   const int c0 = blockIdx.x * CPB;
   const int c = c0 + wave;
-  if (wave < CPB) {
-    for (int e = lane; e < experts; e += 64)
-      own[wave * EMAX + e] = (c < p.n_chunks) ? p.hist[(long)c * experts + e] : 0;
-  }
-  // column sums of the histogram: all chunks, and the chunks in front of this block
-  int epad = 64;
-  while (epad < experts) epad <<= 1;
-  const int parts = 1024 / epad;
-  const int part = tid / epad, el = tid % epad;
-  const int cpp = (p.n_chunks + parts - 1) / parts;
-  const int c_lo = part * cpp;
-  const int c_hi = min(p.n_chunks, c_lo + cpp);
-  int all = 0, before = 0;
-  for (int cc = c_lo; cc < c_hi; cc += 16) {
-    int h[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      h[i] = (el < experts && cc + i < c_hi) ? p.hist[(long)(cc + i) * experts + el] : 0;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      all += h[i];
-      before += (cc + i < c0) ? h[i] : 0;
-    }
-  }
-  // the first PRE steps of 64 rows of the wave's chunk are requested now, so that their memory
-  // latency passes during the scans
+  // the first PRE steps of 64 rows of the wave's chunk are requested at once
   constexpr int PRE = 8;
   const int r0 = c * p.chunk_rows;
   const int r1 = (wave < CPB && c < p.n_chunks) ? min(f.rows, r0 + p.chunk_rows) : r0;
   int pre_e[PRE];
   float pre_w[PRE];
+  auto prefetch = [&]() {
 #pragma unroll
-  for (int i = 0; i < PRE; ++i) {
-    const int r = r0 + 64 * i + lane;
-    pre_e[i] = (r < r1) ? f.topk_idx[r] : -1;
-    pre_w[i] = (r < r1) ? f.topk_w[r] : 0.f;
-  }
-  part_all[tid] = all;
-  part_before[tid] = before;
-  __syncthreads();
+    for (int i = 0; i < PRE; ++i) {
+      const int r = r0 + 64 * i + lane;
+      pre_e[i] = (r < r1) ? f.topk_idx[r] : -1;
+      pre_w[i] = (r < r1) ? f.topk_w[r] : 0.f;
+    }
+  };
   int tot = 0, bef = 0;
-  if (tid < experts) {
-    for (int q = 0; q < parts; ++q) {
-      tot += part_all[q * epad + tid];
-      bef += part_before[q * epad + tid];
+  if constexpr (COUNT) {
+    __shared__ int cnt[GMAX * EMAX];       // rows per (group of CPB chunks, expert)
+    for (int i = tid; i < GMAX * EMAX; i += 1024) cnt[i] = 0;
+    for (int i = tid; i < CPB * EMAX; i += 1024) own[i] = 0;
+    prefetch();
+    // all rows, sixteen per thread; the group of row r = tid + 1024 i follows without dividing per row
+    const int grows = CPB * p.chunk_rows;
+    const int gq = 1024 / grows, gm = 1024 % grows;
+    int g = tid / grows, rem = tid % grows;
+    int ev[16], gv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = 1024 * i + tid;
+      ev[i] = (r < f.rows) ? f.topk_idx[r] : -1;
+      gv[i] = g;
+      g += gq; rem += gm;
+      if (rem >= grows) { rem -= grows; ++g; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (ev[i] >= 0 && ev[i] < experts) atomicAdd(&cnt[gv[i] * EMAX + ev[i]], 1);
+    if (wave < CPB) {
+      int* mine = own + wave * EMAX;
+#pragma unroll
+      for (int i = 0; i < PRE; ++i)
+        if (pre_e[i] >= 0 && pre_e[i] < experts) atomicAdd(&mine[pre_e[i]], 1);
+      for (int r = r0 + 64 * PRE + lane; r < r1; r += 64) {
+        const int e = f.topk_idx[r];
+        if (e >= 0 && e < experts) atomicAdd(&mine[e], 1);
+      }
+    }
+    __syncthreads();
+    if (tid < experts) {
+#pragma unroll
+      for (int gi = 0; gi < GMAX; ++gi) {
+        const int v = cnt[gi * EMAX + tid];
+        tot += v;
+        bef += (gi < (int)blockIdx.x) ? v : 0;
+      }
+    }
+  } else {
+    __shared__ int part_all[1024], part_before[1024];
+    if (wave < CPB) {
+      for (int e = lane; e < experts; e += 64)
+        own[wave * EMAX + e] = (c < p.n_chunks) ? p.hist[(long)c * experts + e] : 0;
+    }
+    // column sums of the histogram: all chunks, and the chunks in front of this block
+    int epad = 64;
+    while (epad < experts) epad <<= 1;
+    const int parts = 1024 / epad;
+    const int part = tid / epad, el = tid % epad;
+    const int cpp = (p.n_chunks + parts - 1) / parts;
+    const int c_lo = part * cpp;
+    const int c_hi = min(p.n_chunks, c_lo + cpp);
+    int all = 0, before = 0;
+    for (int cc = c_lo; cc < c_hi; cc += 16) {
+      int h[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        h[i] = (el < experts && cc + i < c_hi) ? p.hist[(long)(cc + i) * experts + el] : 0;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        all += h[i];
+        before += (cc + i < c0) ? h[i] : 0;
+      }
+    }
+    prefetch();
+    part_all[tid] = all;
+    part_before[tid] = before;
+    __syncthreads();
+    if (tid < experts) {
+      for (int q = 0; q < parts; ++q) {
+        tot += part_all[q * epad + tid];
+        bef += part_before[q * epad + tid];
+      }
     }
   }
   const int incl = block_scan_incl(tot, wave_tot);
@@ -923,14 +1004,17 @@ int dmq_route_permute_launch(const int* topk_idx, const float* topk_w, int token
   const int rows = tokens * k;
   const int experts = plan.experts;
   if (experts > DMQ_SORT_MAX_EXPERTS) return DMQ_ERR_LIMIT;
+  const FillParams f{topk_idx, topk_w, rows, k, sorted_tokens, sorted_weights, sorted_rows};
+  const dim3 grid_pf((plan.n_chunks + DMQ_FILL_CHUNKS - 1) / DMQ_FILL_CHUNKS + 1);
+  if (experts <= DMQ_FUSED_FILL_EXPERTS && rows <= DMQ_FILL_COUNT_ROWS) {
+    hipLaunchKernelGGL(dmq_plan_fill_kernel<true>, grid_pf, dim3(1024), 0, stream, plan, f);
+    return dmq_check_launch();
+  }
   const int grid_c = (plan.n_chunks + 3) / 4;
   hipLaunchKernelGGL(dmq_chunk_count_kernel, dim3(grid_c), dim3(256), 0, stream, topk_idx, rows,
                      experts, plan.chunk_rows, plan.n_chunks, plan.hist);
   if (experts <= DMQ_FUSED_FILL_EXPERTS) {
-    const FillParams f{topk_idx, topk_w, rows, k, sorted_tokens, sorted_weights, sorted_rows};
-    hipLaunchKernelGGL(dmq_plan_fill_kernel,
-                       dim3((plan.n_chunks + DMQ_FILL_CHUNKS - 1) / DMQ_FILL_CHUNKS + 1), dim3(1024), 0, stream,
-                       plan, f);
+    hipLaunchKernelGGL(dmq_plan_fill_kernel<false>, grid_pf, dim3(1024), 0, stream, plan, f);
     return dmq_check_launch();
   }
   hipLaunchKernelGGL(dmq_plan_kernel, dim3(1), dim3(1024), 0, stream, plan);

@@ -87,11 +87,14 @@ def test_permute_matches_oracle(tokens, tile_rows):
 
 @pytest.mark.parametrize("tokens,experts,k", [(700, 100, 3), (1000, 37, 1), (333, 300, 5), (5000, 256, 8),
                                                    (113, 257, 9), (128, 512, 8), (60, 513, 8), (129, 512, 8),
-                                                   (2100, 600, 8), (900, 1100, 6)])
+                                                   (2100, 600, 8), (900, 1100, 6), (2048, 200, 8), (2049, 200, 8),
+                                                   (16384, 16, 1), (5461, 30, 3)])
 def test_permute_odd_shapes(tokens, experts, k):
     """Tokens whose k rows straddle the 64-row steps of the sort, expert counts off the wave size;
     the cases with more than 512 experts take the separate planning and scatter launches, the
-    others the launch that does both."""
+    others the launch that does both: counting the rows itself up to 16384 routed rows (2048 x 8,
+    16384 x 1 and 5461 x 3 sit at that limit, 2049 x 8 just past it), reading the chunk histogram
+    beyond."""
     from dartmoq_hip import ops
     logits = routing.zipf_logits(tokens, experts, seed=7 * tokens + k)
     w, idx = routing.route_topk(logits, k)

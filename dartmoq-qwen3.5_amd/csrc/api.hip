@@ -798,7 +798,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   }
   const int wsplit_eff = sub ? 1 : wsplit;
   if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
-  if (nbl <= 0) nbl = pick_nbl((long)tokens * K, tt);
+  const bool nbl_auto = nbl <= 0;
+  if (nbl_auto) nbl = pick_nbl((long)tokens * K, tt);
   // a rotation wave covers 16 or 32 rows: 64-row work items are rotated by two waves each
   const int rot_tt = tt > 2 ? 2 : tt;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
@@ -898,11 +899,16 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
       if (live && hoisted && whole) rp.hoisted_pool[rp.n_hoisted++] = i;
       if (live && !hoisted && tiled) any_tiled = true;
     }
+    // 16 rows per wave wherever the launch does not fill the chip several times over: a wave's
+    // chain (matrix, rows, 32 MFMAs per tile, quantization) is serial, so more and shorter waves
+    // finish earlier (FP4, whose quantization is the longest: -6 us at 512 tokens, -8 at 4096);
+    // the per-work-item pass of big batches keeps the tile of the work items
+    const int rtt = (!any_tiled || tokens <= 2048) ? 1 : rot_tt;
     long n = 0;                                    // waves of the per-work-item part
-    if (any_tiled) n = (long)w.max_items * (w.tile_rows / (16 * rot_tt)) * rp.groups;
+    if (any_tiled) n = (long)w.max_items * (w.tile_rows / (16 * rtt)) * rp.groups;
     else rp.items = nullptr;
     if (rp.n_hoisted == 0 && !any_tiled && !tp) return DMQ_OK;
-    return dmq_rotate_dispatch(mode, rp, n, rot_tt, st, tp, tp_fp16);
+    return dmq_rotate_dispatch(mode, rp, n, rtt, st, tp, tp_fp16);
   };
   const bool route_small = (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
                            K <= 64 && (!router->logits || tokens <= DMQ_ROUTE_SMALL_TOKENS);
@@ -1108,7 +1114,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     const long avg_rows = (long)tokens * K / E;
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
     d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
-    d.ks = ks; d.nbl = nbl; d.n_pools = P;
+    d.ks = ks; d.n_pools = P;
+    d.nbl = (nbl_auto && down_tt != tt) ? pick_nbl((long)tokens * K, down_tt) : nbl;   // by its own tile count
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       d.pool[i] = dmq_gemm_pool{pd.dn_w, pd.dn_norms, pd.dn_lut, w.dn_info + (size_t)i * E * 4,

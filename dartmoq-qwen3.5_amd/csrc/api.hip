@@ -680,12 +680,20 @@ struct MoeWorkspace {
 
 static inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
-static int pick_tt(int tokens, int top_k, int experts) {
+// weights: 0 = mostly 1- and 2-bit pools, 1 = mostly 4-bit pools behind the look-up table,
+// 2 = mostly FP4 (e2m1 weights, no table)
+static int pick_tt(int tokens, int top_k, int experts, int weights) {
   const long avg = (long)tokens * top_k / (experts > 0 ? experts : 1);
-  // 64-row work items pay off once the experts are big: the gate_up GEMM then halves its look-ups
-  // per row (two workgroups per CU instead of three); measured equal at 96 rows per expert, -1 %
-  // at 128, -4 % at 256.  The down GEMM keeps 32-row tiles on those items (down_tt below).
-  return avg <= 8 ? 1 : (avg <= DMQ_TT4_MIN_AVG ? 2 : 4);
+  // 64-row work items halve the gate_up GEMM's look-ups per row (two workgroups per CU instead of
+  // three) and, where an expert's rows fit one 64-row tile but not one 32-row tile, its tiles.
+  // 2-bit layers (Zipf routing: most experts stay small): equal at 96 rows per expert, -1 % at 128,
+  // -4 % at 256.  4-bit layers pay twice the look-ups per weight (uniform routing, 256 experts:
+  // +3 % at 32 rows per expert, -10 % at 48, -2 % at 64); FP4 streams its weights and gains from
+  // 12 rows per expert on (-5 % at 24, -6 % at 32, -3 % at 64).  The down GEMM keeps 32-row tiles
+  // on those items (down_tt below).
+  const long min4 = weights == 2 ? 10 : (weights == 1 ? 40 : DMQ_TT4_MIN_AVG);
+  if (avg <= (weights == 1 ? 12 : 8)) return 1;   // 4-bit look-up layers: 16-row tiles 3 % ahead at 12 rows per expert
+  return avg <= min4 ? 2 : 4;
 }
 
 static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* base) {
@@ -775,7 +783,13 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   if (H % DMQ_GS || I % DMQ_GS || H / DMQ_GS < 1 || I / DMQ_GS < 1) return DMQ_ERR_ALIGN;
   if (P <= 0 || E <= 0 || K <= 0) return DMQ_ERR_SHAPE;
   if (P > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
-  if (tt <= 0) tt = pick_tt(tokens, K, E);
+  long w4 = 0, wf4 = 0, w_all = 0;         // gate_up rows held by 4-bit look-up pools / FP4 pools / all pools
+  for (int i = 0; i < P; ++i) {
+    w_all += layer->pool[i].n_gate_up;
+    if (layer->pool[i].mode == DMQ_MODE_FP4) wf4 += layer->pool[i].n_gate_up;
+    else if (layer->pool[i].bit == 4) w4 += layer->pool[i].n_gate_up;
+  }
+  if (tt <= 0) tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
   if (ks == 0) ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
   // ks < 0: -ks workgroups share the K range of a gate_up block; the other launches do not split
@@ -840,11 +854,6 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   bool roomy = false;
   if (tt == 1) {
     roomy = (long)tokens * K * (I / DMQ_GS) <= 4096;
-    long w4 = 0, w_all = 0;                            // gate_up rows held by 4-bit pools / by all pools
-    for (int i = 0; i < P; ++i) {
-      w_all += layer->pool[i].n_gate_up;
-      if (layer->pool[i].bit == 4 && layer->pool[i].mode != DMQ_MODE_FP4) w4 += layer->pool[i].n_gate_up;
-    }
     if (2 * w4 > w_all) roomy = true;
   }
 

@@ -302,7 +302,7 @@ def main():
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--cpu-tokens", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--modes", type=str, default="2:wxa8:2048/64,4:wxfp8:2048/64,4:wxfp4:2048/64",
+    ap.add_argument("--modes", type=str, default="2:wxa8:2048/64,4:wxfp8:2048/64,4:wxfp4:2048/64,3:wxa8:64/8/1",
                     help='extra entries of the "modes" array, "config:mode:tokens[/tokens...]" comma '
                          'separated ("" for none)')
     ap.add_argument("--traffic-probe", action="store_true",

@@ -53,7 +53,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 15; }
+int dmq_abi_version(void) { return 16; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -388,6 +388,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.home_filter = a->width_filter != 0 ? a->home_filter : -1;
   p.accumulate = (a->epi == DMQ_EPI_SCATTER && a->accumulate) ? 1 : 0;
   p.wsplit = wsplit;
+  p.spread = a->spread != 0;
   p.subs = subs;
   p.split_rows = a->split_rows;
   p.split_partial = (float*)a->split_partial;
@@ -407,7 +408,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
     // several n-blocks per workgroup need every block complete and the waves on distinct features
     int nbl = a->nbl > 0 ? a->nbl : 1;
-    if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block) nbl = 1;
+    if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block || a->spread) nbl = 1;
     if (nbl > p.n_blocks) nbl = p.n_blocks;
     p.nbl = nbl;
     // several blocks per workgroup: the tail of every XCD's share is cut into single blocks
@@ -421,7 +422,9 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
       per_xcd = (per_xcd + nbl - 1) / nbl * nbl;
       work = (per_xcd / nbl + p.tail_slots) * DMQ_XCDS;
     } else {
-      work = (long)a->max_items * subs * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
+      const long units = a->spread ? ((long)a->max_items * subs + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS
+                                   : (long)a->max_items * subs;
+      work = units * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
       work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
     }
     if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
@@ -848,6 +851,22 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if (!seen) modes[n_modes++] = m;
   }
 
+  // A layer with pools of several precision modes launches each GEMM once per mode over the whole
+  // work list.  The mode with the most weights keeps the contiguous XCD shares; the items of a
+  // smaller mode sit together somewhere in the list (a shared expert's slices: the last items), so
+  // its launches deal the items out one per XCD (dmq_gemm_args.spread) instead of leaving them to
+  // the one XCD whose share they fall into (configs[3] wxa8, 256 tokens: the fp16 launch of the
+  // 4-bit shared expert 67 -> 28 us).
+  int main_mode = modes[0];
+  {
+    long best = -1;
+    for (int mi = 0; mi < n_modes; ++mi) {
+      long rows_m = 0;
+      for (int i = 0; i < P; ++i) if (layer->pool[i].mode == modes[mi]) rows_m += layer->pool[i].n_gate_up;
+      if (rows_m > best) { best = rows_m; main_mode = modes[mi]; }
+    }
+  }
+
   // 16-row tiles: which kernel instance (see dmq_gemm_args.roomy).  The two-per-CU instance wins
   // while the gate_up launch has few workgroups (routed rows x feature blocks; measured: H=2048
   // I=512 up to 128 tokens, H=3072 I=1024 up to 32) and whenever most rows go to 4-bit weights.
@@ -1045,6 +1064,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     // the gate_up blocks are four times as long as the down blocks (K = H against K = I) and end in
     // the rotation epilogue: more than two per workgroup costs more in balance than it saves
     g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P; g.roomy = roomy;
+    g.spread = (n_modes > 1 && mode != main_mode) ? 1 : 0;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = whole_batch[i];
@@ -1123,6 +1143,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     const long avg_rows = (long)tokens * K / E;
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
     d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
+    d.spread = (n_modes > 1 && mode != main_mode) ? 1 : 0;
     d.ks = ks; d.n_pools = P;
     d.nbl = (nbl_auto && down_tt != tt) ? pick_nbl((long)tokens * K, down_tt) : nbl;   // by its own tile count
     for (int i = 0; i < P; ++i) {

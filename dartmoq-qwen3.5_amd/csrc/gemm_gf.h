@@ -97,6 +97,7 @@ struct GemmParams {
   int home_filter;
   int accumulate;
   int wsplit;                  // 1, 2, 4, 8 or 16
+  int spread;                  // work item i on XCD i % 8 instead of a contiguous share per XCD (nbl == 1)
   int split_rows;              // rows of one plane
   float* split_partial;        // fp32 [wsplit, split_rows, 2 * n_out (SiLU) or n_out (store)]
   int* split_counter;          // int32 [max_items * n_blocks], zero before the launch and after it
@@ -1089,12 +1090,21 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   } else {
     const int nbg = (p.n_blocks + p.nbl - 1) / p.nbl * wsplit;   // workgroups per item
     const int total = p.n_items[0] * p.subs * nbg;
-    const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
     const int slot = blockIdx.x / DMQ_XCDS;
-    const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
-    if (slot >= per_xcd || unit >= total) return;
-    item = unit / nbg;
-    const int sub = unit - item * nbg;
+    int sub;
+    if (p.spread) {
+      // items dealt out one at a time: a run of items of this launch's pools anywhere in the
+      // list still reaches every XCD
+      item = (slot / nbg) * DMQ_XCDS + blockIdx.x % DMQ_XCDS;
+      sub = slot % nbg;
+      if (item >= p.n_items[0] * p.subs) return;
+    } else {
+      const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
+      const int unit = (blockIdx.x % DMQ_XCDS) * per_xcd + slot;
+      if (slot >= per_xcd || unit >= total) return;
+      item = unit / nbg;
+      sub = unit - item * nbg;
+    }
     split = sub % wsplit;                                  // workgroups sharing a block are neighbours
     nb = (sub / wsplit) * p.nbl;
     nbc = min(p.nbl, p.n_blocks - nb);

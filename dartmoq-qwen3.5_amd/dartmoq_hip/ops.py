@@ -304,7 +304,7 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None,
-                 item_tile_rows=0, split_ws=None, nt=0, roomy=0):
+                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
     out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 (plain-store
@@ -353,6 +353,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.item_tile_rows = int(item_tile_rows)
     a.nt = int(nt)
     a.roomy = int(roomy)
+    a.spread = int(spread)
     if k_split > 1:
         if rows_total is None:
             raise ValueError("k_split needs rows_total")
@@ -375,7 +376,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
                   tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0, split_ws=None, nt=0,
-                  roomy=0):
+                  roomy=0, spread=0):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -396,7 +397,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
                         dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total,
-                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy)
+                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy, spread=spread)
 
 
 def linear_gemm_i8(x_i8: torch.Tensor, x_scale: torch.Tensor, indices_gf: torch.Tensor,

@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 15). */
+/* Library / build identification: returns the ABI version (currently 16). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -292,6 +292,11 @@ typedef struct {
    * registers (the three-per-CU instance keeps part of it in scratch memory).  Pays for launches
    * of at most two workgroups per CU and for layers with 4-bit pools; same results either way. */
   int roomy;
+  /* != 0: work item i goes to XCD i % 8 (with all its feature blocks) instead of every XCD taking a
+   * contiguous eighth of the list.  For launches that serve a small part of the list sitting in
+   * one place (the mode of a shared expert: its items are the last ones), which the contiguous
+   * split would leave to one XCD; nbl is then 1.  Same results either way. */
+  int spread;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

@@ -53,7 +53,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 16; }
+int dmq_abi_version(void) { return 17; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -294,12 +294,19 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (!a) return DMQ_ERR_NULL;
   if (a->n_pools <= 0 || a->n_pools > DMQ_MAX_POOLS) return DMQ_ERR_LIMIT;
   bool any_wide = false, any_narrow = false;
+  const int mode2 = a->mode2_on ? a->mode2 : -1;
   for (int i = 0; i < a->n_pools; ++i) {
     const int b = a->pool[i].bit;
     if (!dmq_valid_bit_wide(b)) return DMQ_ERR_BIT;
-    if (a->pool[i].mode != a->mode) continue;
+    if (a->pool[i].mode != a->mode && a->pool[i].mode != mode2) continue;
     if (b == 8 && a->mode == DMQ_MODE_FP4) return DMQ_ERR_BIT;
     (b == 8 ? any_wide : any_narrow) = true;
+  }
+  if (mode2 >= 0) {
+    const int ks2 = a->ks > 0 ? a->ks : 1;
+    if (mode2 != DMQ_MODE_A16 || a->mode == DMQ_MODE_A16 || !valid_mode(a->mode)) return DMQ_ERR_MODE;
+    if (a->tt != 1 || ks2 != 1 || any_wide || a->epi == DMQ_EPI_STORE || a->dbg_acc || a->nt == 1)
+      return DMQ_ERR_MODE;
   }
   if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
   if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SILU_ROT) return DMQ_ERR_MODE;
@@ -312,6 +319,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (q.mode == a->mode && a->mode != DMQ_MODE_FP4 && !q.lut &&
         !(a->mode == DMQ_MODE_A8 && q.bit == 8))          // 8-bit int8: NULL = identity table
       return DMQ_ERR_NULL;
+    if (mode2 >= 0 && q.mode == mode2 && !q.lut) return DMQ_ERR_NULL;
     if (q.mode == a->mode && a->mode != DMQ_MODE_A16 && !q.act_scale) return DMQ_ERR_NULL;
     if (q.n_total <= 0 || q.n_total % 16) return DMQ_ERR_ALIGN;
   }
@@ -333,7 +341,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
     if (!a->post_out || (a->mode != DMQ_MODE_A16 && !a->post_scale)) return DMQ_ERR_NULL;
     for (int i = 0; i < a->n_pools; ++i)
-      if (a->pool[i].mode == a->mode && !a->post_rot[i]) return DMQ_ERR_NULL;
+      if ((a->pool[i].mode == a->mode || a->pool[i].mode == mode2) && !a->post_rot[i]) return DMQ_ERR_NULL;
   }
   if (a->act_row_bytes < (long)a->groups * act_bytes_per_group(a->mode)) return DMQ_ERR_SHAPE;
   const int wsplit = a->k_split > 1 ? a->k_split : 1;
@@ -398,6 +406,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   L.nt = one_tile ? 1 : 4;
   L.dbg = a->dbg_acc != nullptr;
   L.roomy = (a->roomy != 0 && a->tt == 1 && ks == 1 && !L.dbg) ? 1 : 0;
+  L.mode2 = mode2;
   L.stream = (hipStream_t)stream;
   // the 1/2/4-bit pools and the 8-bit pools of the mode are separate launches over the same work
   // list (each skips the items of the other kind); 8-bit pools never split K over the waves
@@ -867,6 +876,15 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     }
   }
 
+  // Two modes, the smaller one fp16 (a shared expert that keeps fp16 activations), 16-row tiles, no
+  // 8-bit pools: both modes ride one launch per GEMM (dmq_gemm_args.mode2).
+  bool dual = false;
+  if (n_modes >= 2 && tt == 1 && ks == 1 && !sub && main_mode != DMQ_MODE_A16) {
+    for (int mi = 0; mi < n_modes; ++mi) dual |= modes[mi] == DMQ_MODE_A16;
+    for (int i = 0; i < P; ++i)
+      if (layer->pool[i].mode == main_mode || layer->pool[i].mode == DMQ_MODE_A16) dual &= layer->pool[i].bit != 8;
+  }
+
   // 16-row tiles: which kernel instance (see dmq_gemm_args.roomy).  The two-per-CU instance wins
   // while the gate_up launch has few workgroups (routed rows x feature blocks; measured: H=2048
   // I=512 up to 128 tokens, H=3072 I=1024 up to 32) and whenever most rows go to 4-bit weights.
@@ -1059,8 +1077,10 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   // 3. gate_up GEMM with fused SiLU * up -> act[R, I]
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
+    if (dual && mode == DMQ_MODE_A16) continue;        // rides the main mode's launch
     dmq_gemm_args g{};
     g.mode = mode; g.epi = fuse_rot[mi] ? DMQ_EPI_SILU_ROT : DMQ_EPI_SILU;
+    if (dual && mode == main_mode) { g.mode2_on = 1; g.mode2 = DMQ_MODE_A16; }
     // the gate_up blocks are four times as long as the down blocks (K = H against K = I) and end in
     // the rotation epilogue: more than two per workgroup costs more in balance than it saves
     g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P; g.roomy = roomy;
@@ -1137,7 +1157,9 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   // 5. down GEMM with fused routing weight, rows scattered to their (token, slot) rows
   for (int mi = 0; mi < n_modes; ++mi) {
     const int mode = modes[mi];
+    if (dual && mode == DMQ_MODE_A16) continue;
     dmq_gemm_args d{};
+    if (dual && mode == main_mode) { d.mode2_on = 1; d.mode2 = DMQ_MODE_A16; }
     // 64-row work items: the down GEMM (K = I, four steps per block) runs them as two 32-row tiles
     // until the experts are big enough for its 64-row kernel to pay
     const long avg_rows = (long)tokens * K / E;

@@ -12,6 +12,7 @@ struct GemmLaunch {
   int wide;        // 1: the pools of 8-bit indices (ks must be 1 unless nt == 1), 0: the 1/2/4-bit pools
   int nt;          // n-tiles per wave: 4, or 1 (plain store, tt == 1, ks == 4 only)
   int roomy;       // tt == 1, ks == 1: the two-waves-per-SIMD instance (see ROOMY)
+  int mode2;       // -1, or DMQ_MODE_A16 next to a quantized mode (tt == 1, ks == 1, no 8-bit pools: see MODE2)
   int grid;
   hipStream_t stream;
 };
@@ -26,12 +27,21 @@ template <int MODE, int TT, int KS, int EPI, bool DBG>
 static int dmq_gemm_launch_one(const GemmLaunch& L) {
   if constexpr (MODE != DMQ_MODE_FP4 && KS == 1 && !DBG) {
     if (L.wide) {
+      if (L.mode2 >= 0) return DMQ_ERR_MODE;
       hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, true>), dim3(L.grid), dim3(256), 0,
                          L.stream, L.p);
       return dmq_check_launch();
     }
   }
   if (L.wide) return DMQ_ERR_MODE;
+  if constexpr (MODE != DMQ_MODE_A16 && TT == 1 && KS == 1 && !DBG && EPI != DMQ_EPI_STORE) {
+    if (L.mode2 == DMQ_MODE_A16) {     // the fp16 body of 4-bit pools wants the registers of the roomy instance
+      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, true, DMQ_MODE_A16>),
+                         dim3(L.grid), dim3(256), 0, L.stream, L.p);
+      return dmq_check_launch();
+    }
+  }
+  if (L.mode2 >= 0) return DMQ_ERR_MODE;
   if constexpr (MODE != DMQ_MODE_FP4 && TT == 1 && KS == 1 && !DBG) {
     if (L.roomy) {
       hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, true>), dim3(L.grid),

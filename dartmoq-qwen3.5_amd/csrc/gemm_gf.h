@@ -1052,12 +1052,29 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 // of the 4-bit weights keeps part of its weight ring in scratch memory inside the K loop; a
 // launch that fills at most two workgroups per CU anyway, or one with 4-bit pools, runs the
 // instance that has the registers.
-template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT = 4, bool ROOMY = false>
+//
+// MODE2 >= 0: the launch also serves the pools of a second precision mode (a work item runs the
+// body of its pool's mode).  For a layer whose shared expert keeps fp16 activations next to
+// quantized routed pools: one launch per GEMM instead of one per mode, and the handful of
+// workgroups of the smaller mode run beside the others instead of after them.  The launch
+// parameters are those of MODE; the fp16 body ignores the ones that differ (activation scales).
+template <int M, int NT, int TT, int KS> constexpr int dmq_smem2_bytes() {
+  if constexpr (M < 0) return 16; else return GemmGeom<M, NT, TT, KS>::SMEM2;
+}
+template <int M, int TT, int EPI> constexpr int dmq_post_bytes() {
+  if constexpr (M < 0) return 16; else return PostGeom<M, TT, EPI>::BYTES;
+}
+template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT = 4, bool ROOMY = false,
+          int MODE2 = -1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2 && !ROOMY) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(16))) uint8_t tbl[(MODE == DMQ_MODE_FP4) ? 16 : DMQ_LUT_BYTES];
-  __shared__ __attribute__((aligned(16))) uint8_t smem2[GemmGeom<MODE, NT, TT, KS>::SMEM2];
-  __shared__ __attribute__((aligned(16))) uint8_t smem_post[PostGeom<MODE, TT, EPI>::BYTES];
+  constexpr int S2A = dmq_smem2_bytes<MODE, NT, TT, KS>(), S2B = dmq_smem2_bytes<MODE2, NT, TT, KS>();
+  constexpr int PSA = dmq_post_bytes<MODE, TT, EPI>(), PSB = dmq_post_bytes<MODE2, TT, EPI>();
+  __shared__ __attribute__((aligned(16))) uint8_t
+      tbl[(MODE == DMQ_MODE_FP4 && (MODE2 < 0 || MODE2 == DMQ_MODE_FP4)) ? 16 : DMQ_LUT_BYTES];
+  __shared__ __attribute__((aligned(16))) uint8_t smem2[S2A > S2B ? S2A : S2B];
+  __shared__ __attribute__((aligned(16))) uint8_t smem_post[PSA > PSB ? PSA : PSB];
+  static_assert(MODE2 < 0 || (!WIDE && !DBG && NT == 4), "two modes: 1/2/4-bit pools, four n-tiles per wave");
   static_assert(EPI != DMQ_EPI_SILU_ROT || KS == 1, "the fused rotation needs the whole block in one workgroup");
   // Workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD gets a contiguous range of
   // the work list, so the workgroups that share an activation tile (the feature blocks of an
@@ -1126,7 +1143,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   // down slice at group start / 128 (holds for items of either origin)
   const int post_slice = r1[1] / (2 * DMQ_GS);
   const PoolW& pw = p.pool[pool];
-  if (pw.mode != MODE) return;
+  if (pw.mode != MODE && (MODE2 < 0 || pw.mode != MODE2)) return;
   if (WIDE != (pw.bit == 8)) return;
   int col0 = 0;
   if (p.width_filter != 0) {                             // sub-expert layers: one width (and rank) per launch
@@ -1135,18 +1152,28 @@ void dmq_gemm_gf_kernel(GemmParams p) {
     if (p.home_filter >= 0 && (pw.home ? pw.home[e] : 0) != p.home_filter) return;
     col0 = pw.col_start ? pw.col_start[e] : 0;
   }
-  if constexpr (MODE == DMQ_MODE_FP4) {
-    dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
-  } else if constexpr (WIDE) {
-    if (MODE == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
-      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG, MODE == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
-    else
-      dmq_gemm_body<MODE, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
-  } else {
-    switch (pw.bit) {
-      case 1: dmq_gemm_body<MODE, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-      case 2: dmq_gemm_body<MODE, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-      default: dmq_gemm_body<MODE, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+  auto run = [&](auto mode_tag) __attribute__((always_inline)) {
+    constexpr int M = decltype(mode_tag)::value;
+    if constexpr (M == DMQ_MODE_FP4) {
+      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+    } else if constexpr (WIDE) {
+      if (M == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
+        dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+      else
+        dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+    } else {
+      switch (pw.bit) {
+        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+      }
+    }
+  };
+  if constexpr (MODE2 >= 0) {
+    if (pw.mode == MODE2) {                             // uniform over the workgroup
+      run(std::integral_constant<int, MODE2>{});
+      return;
     }
   }
+  run(std::integral_constant<int, MODE>{});
 }

@@ -304,7 +304,7 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None,
-                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0):
+                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
     out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 (plain-store
@@ -354,6 +354,8 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.nt = int(nt)
     a.roomy = int(roomy)
     a.spread = int(spread)
+    a.mode2_on = 0 if mode2 is None else 1
+    a.mode2 = 0 if mode2 is None else int(mode2)
     if k_split > 1:
         if rows_total is None:
             raise ValueError("k_split needs rows_total")

@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 16). */
+/* Library / build identification: returns the ABI version (currently 17). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -297,6 +297,13 @@ typedef struct {
    * one place (the mode of a shared expert: its items are the last ones), which the contiguous
    * split would leave to one XCD; nbl is then 1.  Same results either way. */
   int spread;
+  /* mode2_on != 0: the launch also serves the pools whose mode is mode2 (a work item runs the body of
+   * its pool's mode).  Only mode2 == DMQ_MODE_A16 next to a quantized `mode`, tt == 1, ks == 1, no
+   * 8-bit pool in either mode, epilogues other than the plain store, no dbg_acc: the shared
+   * expert that keeps fp16 activations rides the routed pools' launch.  Scalar fields
+   * (act_scale_stride, post_scale ...) are those of `mode`.  Same results as one launch per mode. */
+  int mode2_on;
+  int mode2;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

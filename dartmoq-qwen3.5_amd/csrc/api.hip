@@ -924,8 +924,14 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   // Rotation (+ quantization) of the gate_up input of one precision mode.  whole: the pools that
   // rotate every token once (no dependence on the routing step); tiled: the pools rotated per
   // work item; tp: the router's top-k rides the same launch.
+  bool whole_done[DMQ_MAX_POOLS] = {false, false, false, false};   // per mode
+  int a16_mi = -1;
+  for (int mi = 0; mi < n_modes; ++mi) if (modes[mi] == DMQ_MODE_A16) a16_mi = mi;
   auto rotate_gate_up_input = [&](int mode, bool whole, bool tiled, const TopkParams* tp,
                                   int tp_fp16) -> int {
+    // the whole-batch pools of the fp16 mode ride the main mode's launch (see `dual`): same
+    // rotation, their rows are stored as fp16 instead of going through the quantizer
+    const bool with_f16 = dual && mode == main_mode && whole && !whole_done[a16_mi];
     RotParams rp{};
     rp.x = (const __half*)x; rp.x_stride = H; rp.row_index = w.sorted_tokens;
     rp.rows = tokens; rp.groups = H / DMQ_GS;
@@ -935,8 +941,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     for (int i = 0; i < DMQ_MAX_POOLS; ++i) {
       const int pi = i < P ? i : 0;
       const dmq_pool_desc& pd = layer->pool[pi];
-      const bool live = i < P && pd.mode == mode;
       const bool hoisted = whole_batch[pi];
+      const bool live = i < P && (pd.mode == mode || (with_f16 && pd.mode == DMQ_MODE_A16 && hoisted));
       const long row_bytes = (long)H * 2;
       rp.pool[i] = RotPool{(const __half*)pd.gu_rot, hoisted ? w.xq[pi] : w.xq_rows, row_bytes,
                            hoisted ? (void*)w.xq_scale[pi] : (void*)w.xq_rows_scale,
@@ -954,13 +960,15 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if (any_tiled) n = (long)w.max_items * (w.tile_rows / (16 * rtt)) * rp.groups;
     else rp.items = nullptr;
     if (rp.n_hoisted == 0 && !any_tiled && !tp) return DMQ_OK;
-    return dmq_rotate_dispatch(mode, rp, n, rtt, st, tp, tp_fp16);
+    rp.also_f16 = with_f16 ? 1 : 0;
+    const int rc_rot = dmq_rotate_dispatch(mode, rp, n, rtt, st, tp, tp_fp16);
+    if (!rc_rot && with_f16) whole_done[a16_mi] = true;   // fp16 pools rotated per work item keep their own pass
+    return rc_rot;
   };
   const bool route_small = (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
                            K <= 64 && (!router->logits || tokens <= DMQ_ROUTE_SMALL_TOKENS);
   // When the top-k is a launch of its own (logits, more than 16 tokens) it shares the launch of the
   // whole-batch rotation of the first mode: neither needs the other, both are short.
-  bool whole_done[DMQ_MAX_POOLS] = {false, false, false, false};   // per mode
   bool topk_done = false;
   // Up to four tokens (logits or a caller-made top-k): no sort launch.  The top-k workgroup of the
   // rotation launch ranks the routed rows itself and writes the work items (see DirectPlan); the

@@ -49,6 +49,7 @@ struct RotParams {
   int tile_rows;           // rows per work item (multiple of 16*TT)
   int scale_fp32;
   int items_prefix;        // 1: only the first n_items[1] items belong to tiled pools
+  int also_f16;            // 1: whole-batch pools of mode DMQ_MODE_A16 are served too (rows stored as fp16)
   LinearPrep prep;
 };
 

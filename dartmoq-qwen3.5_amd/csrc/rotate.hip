@@ -117,7 +117,8 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
   if (cg < 0) cg = g;
   const RotPool& rp = p.pool[pool];
   const bool tiled_wg = !hoisted && p.tiled_staged;
-  if (!tiled_wg && rp.mode != MODE) return;
+  const bool f16_guest = MODE != DMQ_MODE_A16 && hoisted && p.also_f16 && rp.mode == DMQ_MODE_A16;
+  if (!tiled_wg && rp.mode != MODE && !f16_guest) return;
 
   int rlog[TT];
   bool valid[TT];
@@ -193,7 +194,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
 #pragma unroll
   for (int t = 0; t < TT; ++t) {
     uint8_t* orow = rp.out + (long)rlog[t] * rp.out_row_bytes;
-    if (MODE == DMQ_MODE_A16) {
+    if (MODE == DMQ_MODE_A16 || f16_guest) {
       if (!valid[t]) continue;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {

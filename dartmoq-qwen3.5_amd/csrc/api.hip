@@ -919,6 +919,16 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     for (int i = 0; i < P; ++i) if (!whole_batch[i]) pool_order[n++] = i;
     lead_pools = n;
     for (int i = 0; i < P; ++i) if (whole_batch[i]) pool_order[n++] = i;
+    // Among the whole-batch pools the ones with the longest work items go first (the order of the
+    // list is the order in which workgroups get their slots): 4-bit weights cost twice the look-ups
+    // of 2-bit ones, fp16 activations more than quantized ones.  A 4-bit fp16 shared expert at the
+    // end of the list would start when the first routed items finish and end long after them.
+    auto item_cost = [&](int i) { return layer->pool[i].bit * (layer->pool[i].mode == DMQ_MODE_A16 ? 2 : 1); };
+    for (int a = lead_pools; a < n; ++a)
+      for (int b = a + 1; b < n; ++b)
+        if (item_cost(pool_order[b]) > item_cost(pool_order[a])) {
+          const int t = pool_order[a]; pool_order[a] = pool_order[b]; pool_order[b] = t;
+        }
   }
 
   // Rotation (+ quantization) of the gate_up input of one precision mode.  whole: the pools that

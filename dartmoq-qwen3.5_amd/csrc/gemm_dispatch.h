@@ -35,9 +35,13 @@ static int dmq_gemm_launch_one(const GemmLaunch& L) {
   }
   if (L.wide) return DMQ_ERR_MODE;
   if constexpr (MODE != DMQ_MODE_A16 && TT == 1 && KS == 1 && !DBG && EPI != DMQ_EPI_STORE) {
-    if (L.mode2 == DMQ_MODE_A16) {     // the fp16 body of 4-bit pools wants the registers of the roomy instance
-      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, true, DMQ_MODE_A16>),
-                         dim3(L.grid), dim3(256), 0, L.stream, L.p);
+    if (L.mode2 == DMQ_MODE_A16) {     // both instances, picked like those of a single mode
+      if (L.roomy || MODE == DMQ_MODE_FP4)
+        hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, true, DMQ_MODE_A16>),
+                           dim3(L.grid), dim3(256), 0, L.stream, L.p);
+      else
+        hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, false, DMQ_MODE_A16>),
+                           dim3(L.grid), dim3(256), 0, L.stream, L.p);
       return dmq_check_launch();
     }
   }

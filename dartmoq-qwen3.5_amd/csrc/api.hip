@@ -416,8 +416,12 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     const int feat_per_block = (4 / lks) * feat_per_wave;
     p.n_blocks = (a->n_out + feat_per_block - 1) / feat_per_block;
     // several n-blocks per workgroup need every block complete and the waves on distinct features
+    // 8-bit pools next to 1/2/4-bit pools are the few wide Linears of a layer (a shared expert):
+    // their items sit together in the list, so their launch deals the items out (see spread)
+    const bool spread_l = a->spread != 0 || (wide && any_narrow);
+    p.spread = spread_l;
     int nbl = a->nbl > 0 ? a->nbl : 1;
-    if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block || a->spread) nbl = 1;
+    if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block || spread_l) nbl = 1;
     if (nbl > p.n_blocks) nbl = p.n_blocks;
     p.nbl = nbl;
     // several blocks per workgroup: the tail of every XCD's share is cut into single blocks
@@ -431,8 +435,8 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
       per_xcd = (per_xcd + nbl - 1) / nbl * nbl;
       work = (per_xcd / nbl + p.tail_slots) * DMQ_XCDS;
     } else {
-      const long units = a->spread ? ((long)a->max_items * subs + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS
-                                   : (long)a->max_items * subs;
+      const long units = spread_l ? ((long)a->max_items * subs + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS
+                                  : (long)a->max_items * subs;
       work = units * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
       work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
     }

@@ -57,7 +57,7 @@ def _mode_inputs(mode, x_rot, cb):
             luts.e2m1_value(nib), 2.0 ** e0, resid, 127 + e0)
 
 
-def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed, roomy=0):
+def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed, roomy=0, spread=0):
     from dartmoq_hip import ops
     n_exp = len(counts)
     starts, rows_total = _expert_rows(counts)
@@ -94,7 +94,7 @@ def _run_case(mode, bit, tt, counts, k, n_slice, slice_is_groups, seed, roomy=0)
         mode, bit, STORE, act.cuda(), None if scale is None else scale.cuda(), w_dev,
         norms_used.cuda(), None if mode == FP4 else lut.cuda(), info_dev, groups=k // 128,
         n_out=n_slice, slice_is_groups=slice_is_groups, rows_total=rows_total, w_scale_byte=wsb, tt=tt,
-        roomy=roomy)
+        roomy=roomy, spread=spread)
     torch.cuda.synchronize()
     return out.cpu().float(), ref
 
@@ -122,6 +122,69 @@ def test_two_per_cu_instance_gives_the_same_bits(mode, bit):
                          seed=100 + 10 * mode + bit, roomy=1)
     assert torch.equal(lean, roomy)
     torch.testing.assert_close(roomy, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("mode", [A16, A8, FP4])
+@pytest.mark.parametrize("tt", [1, 2, 4])
+def test_items_dealt_out_one_per_xcd_give_the_same_bits(mode, tt):
+    """spread: work item i goes to XCD i % 8 instead of every XCD taking a contiguous eighth of the
+    list; a different schedule of the same work."""
+    counts = [3, 0, 17, 64, 1, 130, 300, 5, 33]
+    a, ref = _run_case(mode, 2, tt, counts, k=256, n_slice=192, slice_is_groups=False, seed=200 + mode + tt)
+    b, _ = _run_case(mode, 2, tt, counts, k=256, n_slice=192, slice_is_groups=False, seed=200 + mode + tt,
+                     spread=1)
+    assert torch.equal(a, b)
+    torch.testing.assert_close(b, ref, rtol=2e-3, atol=2e-3 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("main", [A8, FP8, FP4])
+@pytest.mark.parametrize("roomy", [0, 1])
+def test_two_modes_in_one_launch_give_the_bits_of_two_launches(main, roomy):
+    """mode2: the fp16 pool (4-bit weights) rides the launch of a quantized pool (2-bit weights);
+    every work item runs the body of its pool's mode, so the result is that of one launch per mode."""
+    from dartmoq_hip import ops
+    k, inter = 384, 128
+    counts0, counts1 = [5, 40, 0, 17], [21, 2]
+    r0, r1 = sum(counts0), sum(counts1)
+    rows = r0 + r1
+    g = torch.Generator().manual_seed(77 + main)
+    x_rot = torch.randn(rows, k, generator=g) * 0.7
+    pools = []
+    infos = []
+    for pi, (mode, bit, counts, first_row) in enumerate([(main, 2, counts0, 0), (A16, 4, counts1, r0)]):
+        idx_gf, norms_gf, cb = _pool(bit, 2 * inter * len(counts), k, 300 + pi)
+        act, scale, _, _, lut, _, _, nfac, wsb = _mode_inputs(mode, x_rot, cb)
+        norms_used = (norms_gf.float() * nfac).half() if mode == FP4 else norms_gf
+        w_dev = idx_gf.cuda()
+        if mode == FP4:
+            w_dev = ops.fold_indices_to_e2m1(w_dev, lut, bit)
+        # one row pitch for both pools (that of the fp16 rows), as in the layer's activation buffers
+        buf = torch.zeros(rows, 2 * k, dtype=torch.uint8)
+        raw = act.contiguous().view(torch.uint8).reshape(rows, -1)
+        buf[:, :raw.shape[1]] = raw
+        starts = [first_row + sum(counts[:e]) for e in range(len(counts))]
+        info = torch.tensor([(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(len(counts))],
+                            dtype=torch.int32).cuda()
+        infos.append(info)
+        pools.append(dict(w=w_dev, norms=norms_used.cuda(), lut=None if mode == FP4 else lut.cuda(),
+                          expert_info=info, act=buf.cuda(), act_scale=None if scale is None else scale.cuda(),
+                          row_index=None, bit=bit, mode=mode, w_scale_byte=wsb))
+    lists = [ops.build_tiles(infos[pi], rows, 16, pool=pi) for pi in range(2)]
+    n = [int(l[0][0]) for l in lists]
+    items = torch.cat([lists[0][1][:n[0]], lists[1][1][:n[1]]]).contiguous()
+    n_items = torch.tensor([n[0] + n[1], 0, 0, 0], dtype=torch.int32).cuda()
+    scale_stride = pools[0]["act_scale"].stride(0)
+    common = dict(groups=k // 128, n_out=inter, half_width=inter, slice_is_groups=False, tt=1,
+                  out_stride=inter, act_row_bytes=2 * k, act_scale_stride=scale_stride, roomy=roomy)
+    both = torch.full((rows, inter), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_pools(main, SILU, pools, items, n_items, items.shape[0], out=both, mode2=A16, **common)
+    apart = torch.full((rows, inter), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_pools(main, SILU, pools, items, n_items, items.shape[0], out=apart, **common)
+    assert torch.isnan(apart[r0:].float()).all() and not torch.isnan(apart[:r0].float()).any()
+    ops.matmul_pools(A16, SILU, pools, items, n_items, items.shape[0], out=apart, spread=1, **common)
+    torch.cuda.synchronize()
+    assert not torch.isnan(both.float()).any()
+    assert torch.equal(both, apart)
 
 
 @pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])

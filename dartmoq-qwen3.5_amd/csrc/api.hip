@@ -305,7 +305,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (mode2 >= 0) {
     const int ks2 = a->ks > 0 ? a->ks : 1;
     if (mode2 != DMQ_MODE_A16 || a->mode == DMQ_MODE_A16 || !valid_mode(a->mode)) return DMQ_ERR_MODE;
-    if (a->tt != 1 || ks2 != 1 || any_wide || a->epi == DMQ_EPI_STORE || a->dbg_acc || a->nt == 1)
+    if (a->tt > 2 || ks2 != 1 || any_wide || a->epi == DMQ_EPI_STORE || a->dbg_acc || a->nt == 1)
       return DMQ_ERR_MODE;
   }
   if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
@@ -880,10 +880,13 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     }
   }
 
-  // Two modes, the smaller one fp16 (a shared expert that keeps fp16 activations), 16-row tiles, no
-  // 8-bit pools: both modes ride one launch per GEMM (dmq_gemm_args.mode2).
+  // Several modes, a smaller one fp16 (a shared expert that keeps fp16 activations), no 8-bit pools:
+  // the fp16 mode rides the main mode's launch of each GEMM (dmq_gemm_args.mode2).  With 16-row
+  // tiles always; with 32-row tiles up to 1024 tokens, the items dealt out one per XCD (the shared
+  // expert's items are neighbours in the list): configs[3] wxa8 512 tokens 227 -> 198 us, 1024
+  // tokens 340 -> 323, 2048 tokens 545 -> 551; the 64-row kernel with both bodies spills.
   bool dual = false;
-  if (n_modes >= 2 && tt == 1 && ks == 1 && !sub && main_mode != DMQ_MODE_A16) {
+  if (n_modes >= 2 && (tt == 1 || (tt == 2 && tokens <= 1024)) && ks == 1 && !sub && main_mode != DMQ_MODE_A16) {
     for (int mi = 0; mi < n_modes; ++mi) dual |= modes[mi] == DMQ_MODE_A16;
     for (int i = 0; i < P; ++i)
       if (layer->pool[i].mode == main_mode || layer->pool[i].mode == DMQ_MODE_A16) dual &= layer->pool[i].bit != 8;
@@ -1106,7 +1109,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     // the gate_up blocks are four times as long as the down blocks (K = H against K = I) and end in
     // the rotation epilogue: more than two per workgroup costs more in balance than it saves
     g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P; g.roomy = roomy;
-    g.spread = (n_modes > 1 && mode != main_mode) ? 1 : 0;
+    g.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = whole_batch[i];
@@ -1187,7 +1190,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     const long avg_rows = (long)tokens * K / E;
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
     d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
-    d.spread = (n_modes > 1 && mode != main_mode) ? 1 : 0;
+    d.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
     d.ks = ks; d.n_pools = P;
     d.nbl = (nbl_auto && down_tt != tt) ? pick_nbl((long)tokens * K, down_tt) : nbl;   // by its own tile count
     for (int i = 0; i < P; ++i) {

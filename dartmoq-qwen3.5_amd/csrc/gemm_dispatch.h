@@ -34,9 +34,9 @@ static int dmq_gemm_launch_one(const GemmLaunch& L) {
     }
   }
   if (L.wide) return DMQ_ERR_MODE;
-  if constexpr (MODE != DMQ_MODE_A16 && TT == 1 && KS == 1 && !DBG && EPI != DMQ_EPI_STORE) {
+  if constexpr (MODE != DMQ_MODE_A16 && TT <= 2 && KS == 1 && !DBG && EPI != DMQ_EPI_STORE) {
     if (L.mode2 == DMQ_MODE_A16) {     // both instances, picked like those of a single mode
-      if (L.roomy || MODE == DMQ_MODE_FP4)
+      if (TT == 1 && (L.roomy || MODE == DMQ_MODE_FP4))
         hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, false, 4, true, DMQ_MODE_A16>),
                            dim3(L.grid), dim3(256), 0, L.stream, L.p);
       else

@@ -298,7 +298,7 @@ typedef struct {
    * split would leave to one XCD; nbl is then 1.  Same results either way. */
   int spread;
   /* mode2_on != 0: the launch also serves the pools whose mode is mode2 (a work item runs the body of
-   * its pool's mode).  Only mode2 == DMQ_MODE_A16 next to a quantized `mode`, tt == 1, ks == 1, no
+   * its pool's mode).  Only mode2 == DMQ_MODE_A16 next to a quantized `mode`, tt <= 2, ks == 1, no
    * 8-bit pool in either mode, epilogues other than the plain store, no dbg_acc: the shared
    * expert that keeps fp16 activations rides the routed pools' launch.  Scalar fields
    * (act_scale_stride, post_scale ...) are those of `mode`.  Same results as one launch per mode. */

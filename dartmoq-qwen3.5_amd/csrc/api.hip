@@ -53,7 +53,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 17; }
+int dmq_abi_version(void) { return 18; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -336,8 +336,12 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   const int feat_per_wave = silu ? 32 : (one_tile ? 16 : 64);
   if (a->n_out % feat_per_wave) return DMQ_ERR_ALIGN;
   if (silu && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
+  // 16-row tiles, no K sharing: the 8-bit pools and the others ride one launch (and the fused down
+  // rotation is then open to 8-bit pools as well)
+  const bool both_widths = any_wide && !a->widths_apart && a->tt == 1 && ks == 1 && a->k_split <= 1 && !a->dbg_acc &&
+                           mode2 < 0 && a->nt != 1 && a->epi != DMQ_EPI_STORE && a->mode != DMQ_MODE_FP4;
   if (a->epi == DMQ_EPI_SILU_ROT) {
-    if (ks != 1 || any_wide) return DMQ_ERR_MODE;
+    if (ks != 1 || (any_wide && !both_widths)) return DMQ_ERR_MODE;
     if (a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
     if (!a->post_out || (a->mode != DMQ_MODE_A16 && !a->post_scale)) return DMQ_ERR_NULL;
     for (int i = 0; i < a->n_pools; ++i)
@@ -411,6 +415,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   // the 1/2/4-bit pools and the 8-bit pools of the mode are separate launches over the same work
   // list (each skips the items of the other kind); 8-bit pools never split K over the waves
   for (int wide = 0; wide < 2; ++wide) {
+    if (both_widths && wide == 0) continue;           // one launch, issued as the "wide" pass
     if (!(wide ? any_wide : any_narrow)) continue;
     const int lks = (wide && !one_tile) ? 1 : ks;
     const int feat_per_block = (4 / lks) * feat_per_wave;
@@ -418,7 +423,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     // several n-blocks per workgroup need every block complete and the waves on distinct features
     // 8-bit pools next to 1/2/4-bit pools are the few wide Linears of a layer (a shared expert):
     // their items sit together in the list, so their launch deals the items out (see spread)
-    const bool spread_l = a->spread != 0 || (wide && any_narrow);
+    const bool spread_l = a->spread != 0 || (wide && any_narrow && !both_widths);
     p.spread = spread_l;
     int nbl = a->nbl > 0 ? a->nbl : 1;
     if (lks > 1 || wsplit > 1 || a->n_out % feat_per_block || spread_l) nbl = 1;
@@ -428,7 +433,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     p.tail_slots = (nbl > 1 && wsplit == 1 && p.n_blocks % nbl == 0) ? DMQ_TAIL_SLOTS : 0;
     L.p = p;
     L.ks = lks;
-    L.wide = wide;
+    L.wide = both_widths ? 2 : wide;
     long work;
     if (p.tail_slots > 0) {
       long per_xcd = ((long)a->max_items * subs * p.n_blocks + DMQ_XCDS - 1) / DMQ_XCDS;
@@ -903,11 +908,16 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
 
   // The gate_up GEMM rotates (and quantizes) its SiLU*up rows for the down projection itself when
   // a workgroup owns whole blocks of 128 features: no K split, no 8-bit pools in the mode.
+  // 8-bit pools next to narrower ones: up to about a hundred work items one 16-row launch serves
+  // both index widths and fuses as well (dmq_gemm_args.widths_apart; configs[3] with the reference's
+  // default 8-bit shared expert, wxa8: 64 tokens 133 -> 107 us, 128 tokens 153 -> 146, 256 tokens
+  // 196 -> 240, so beyond 1280 routed rows the widths keep their own launches).
+  const bool widths_apart = tt != 1 || (long)tokens * K > 1280;
   bool fuse_rot[DMQ_MAX_POOLS];
   for (int mi = 0; mi < n_modes; ++mi) {
     fuse_rot[mi] = (ks == 1);
     for (int i = 0; i < P; ++i)
-      if (layer->pool[i].mode == modes[mi] && layer->pool[i].bit == 8) fuse_rot[mi] = false;
+      if (layer->pool[i].mode == modes[mi] && layer->pool[i].bit == 8 && widths_apart) fuse_rot[mi] = false;
   }
 
   // Which pools rotate every token once instead of their routed rows: the caller's choice (pools
@@ -1110,6 +1120,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     // the rotation epilogue: more than two per workgroup costs more in balance than it saves
     g.tt = tt; g.ks = ks; g.nbl = nbl > 2 ? 2 : nbl; g.n_pools = P; g.roomy = roomy;
     g.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
+    g.widths_apart = widths_apart;
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
       const bool hoisted = whole_batch[i];
@@ -1191,6 +1202,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
     d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
     d.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
+    d.widths_apart = widths_apart;
     d.ks = ks; d.n_pools = P;
     d.nbl = (nbl_auto && down_tt != tt) ? pick_nbl((long)tokens * K, down_tt) : nbl;   // by its own tile count
     for (int i = 0; i < P; ++i) {

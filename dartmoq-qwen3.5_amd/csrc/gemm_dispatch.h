@@ -9,7 +9,8 @@ struct GemmLaunch {
   int tt;          // activation tiles of 16 rows per wave: 1, 2 or 4
   int ks;          // waves splitting K: 1, 2 or 4
   int dbg;
-  int wide;        // 1: the pools of 8-bit indices (ks must be 1 unless nt == 1), 0: the 1/2/4-bit pools
+  int wide;        // 1: the pools of 8-bit indices (ks must be 1 unless nt == 1), 0: the 1/2/4-bit pools,
+                   // 2: both in one launch (tt == 1, ks == 1, epilogues other than the plain store)
   int nt;          // n-tiles per wave: 4, or 1 (plain store, tt == 1, ks == 4 only)
   int roomy;       // tt == 1, ks == 1: the two-waves-per-SIMD instance (see ROOMY)
   int mode2;       // -1, or DMQ_MODE_A16 next to a quantized mode (tt == 1, ks == 1, no 8-bit pools: see MODE2)
@@ -25,6 +26,15 @@ static inline bool dmq_gemm_config_ok(int tt, int ks) {
 
 template <int MODE, int TT, int KS, int EPI, bool DBG>
 static int dmq_gemm_launch_one(const GemmLaunch& L) {
+  if constexpr (MODE != DMQ_MODE_FP4 && TT == 1 && KS == 1 && !DBG && EPI != DMQ_EPI_STORE) {
+    if (L.wide == 2) {
+      if (L.mode2 >= 0) return DMQ_ERR_MODE;
+      hipLaunchKernelGGL((dmq_gemm_gf_kernel<MODE, TT, EPI, KS, DBG, 2>), dim3(L.grid), dim3(256), 0,
+                         L.stream, L.p);
+      return dmq_check_launch();
+    }
+  }
+  if (L.wide == 2) return DMQ_ERR_MODE;
   if constexpr (MODE != DMQ_MODE_FP4 && KS == 1 && !DBG) {
     if (L.wide) {
       if (L.mode2 >= 0) return DMQ_ERR_MODE;

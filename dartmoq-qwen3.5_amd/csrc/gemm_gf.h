@@ -1045,6 +1045,9 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 // WIDE kernels serve the pools of 8-bit indices (one byte per weight: twice the packed words per
 // lane of a 4-bit pool); they are separate instances so that their registers do not count against
 // the kernels of the 1/2/4-bit pools.  A launch skips the work items of the other kind.
+// WIDE == 2 serves both kinds in one launch (16-row tiles: the register budget is the wide one
+// anyway, and a layer whose shared expert is 8-bit next to 2-bit routed pools then launches each
+// GEMM once: the few workgroups of the shared expert run beside the routed ones).
 // NT: n-tiles of 16 features per wave.  Four everywhere except the instances for a Linear with a
 // handful of rows (NT = 1, K split over the four waves: a workgroup covers 16 features, so a
 // 4096-feature matrix gives 256 workgroups instead of 64).
@@ -1064,7 +1067,7 @@ template <int M, int NT, int TT, int KS> constexpr int dmq_smem2_bytes() {
 template <int M, int TT, int EPI> constexpr int dmq_post_bytes() {
   if constexpr (M < 0) return 16; else return PostGeom<M, TT, EPI>::BYTES;
 }
-template <int MODE, int TT, int EPI, int KS, bool DBG, bool WIDE = false, int NT = 4, bool ROOMY = false,
+template <int MODE, int TT, int EPI, int KS, bool DBG, int WIDE = 0, int NT = 4, bool ROOMY = false,
           int MODE2 = -1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && KS == 1 && TT <= 2 && !ROOMY) ? 3 : 2)))
 void dmq_gemm_gf_kernel(GemmParams p) {
@@ -1144,7 +1147,7 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   const int post_slice = r1[1] / (2 * DMQ_GS);
   const PoolW& pw = p.pool[pool];
   if (pw.mode != MODE && (MODE2 < 0 || pw.mode != MODE2)) return;
-  if (WIDE != (pw.bit == 8)) return;
+  if (WIDE != 2 && (WIDE == 1) != (pw.bit == 8)) return;
   int col0 = 0;
   if (p.width_filter != 0) {                             // sub-expert layers: one width (and rank) per launch
     const int e = r0[1];
@@ -1156,12 +1159,18 @@ void dmq_gemm_gf_kernel(GemmParams p) {
     constexpr int M = decltype(mode_tag)::value;
     if constexpr (M == DMQ_MODE_FP4) {
       dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
-    } else if constexpr (WIDE) {
-      if (M == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
-        dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
-      else
-        dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
-    } else {
+      return;
+    }
+    if constexpr (M != DMQ_MODE_FP4 && WIDE != 0) {
+      if (WIDE == 1 || pw.bit == 8) {                    // uniform over the workgroup
+        if (M == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+        else
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+        return;
+      }
+    }
+    if constexpr (M != DMQ_MODE_FP4 && WIDE != 1) {
       switch (pw.bit) {
         case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
         case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;

@@ -304,7 +304,7 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None,
-                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None):
+                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None, widths_apart=0):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
     out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 (plain-store
@@ -356,6 +356,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.spread = int(spread)
     a.mode2_on = 0 if mode2 is None else 1
     a.mode2 = 0 if mode2 is None else int(mode2)
+    a.widths_apart = int(widths_apart)
     if k_split > 1:
         if rows_total is None:
             raise ValueError("k_split needs rows_total")
@@ -378,7 +379,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
                   tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0, split_ws=None, nt=0,
-                  roomy=0, spread=0):
+                  roomy=0, spread=0, widths_apart=0):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -399,7 +400,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
                         dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total,
-                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy, spread=spread)
+                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy, spread=spread, widths_apart=widths_apart)
 
 
 def linear_gemm_i8(x_i8: torch.Tensor, x_scale: torch.Tensor, indices_gf: torch.Tensor,

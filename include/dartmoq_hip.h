@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 17). */
+/* Library / build identification: returns the ABI version (currently 18). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -304,10 +304,16 @@ typedef struct {
    * (act_scale_stride, post_scale ...) are those of `mode`.  Same results as one launch per mode. */
   int mode2_on;
   int mode2;
+  /* A launch with 8-bit pools next to narrower ones, tt == 1, no K sharing, not WxFP4, not the plain
+   * store: one kernel instance serves both index widths in ONE launch (two workgroups per CU; it
+   * also lets DMQ_EPI_SILU_ROT cover 8-bit pools).  widths_apart != 0 keeps the two launches (the
+   * narrower pools then run three workgroups per CU, which wins once the list holds more than
+   * about a hundred work items; DMQ_EPI_SILU_ROT with 8-bit pools is then refused).  Same results. */
+  int widths_apart;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more
- * for its 8-bit pools (never split over K).  Stands in for
+ * for its 8-bit pools (never split over K; see widths_apart for the single launch at tt == 1).  Stands in for
  *   triton_fused_matmul_merged_rows_gf / _merged_in_features_gf   (triton_kernels.py:1482-1615)
  *   wxa8_matmul_merged_rows_gf / _merged_in_features_gf           (triton_kernels_a8.py:959-1068)
  *   wxfp8_matmul_merged_rows_gf / _merged_in_features_gf          (triton_kernels_fp8.py:641-750)

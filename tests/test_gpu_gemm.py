@@ -187,6 +187,51 @@ def test_two_modes_in_one_launch_give_the_bits_of_two_launches(main, roomy):
     assert torch.equal(both, apart)
 
 
+@pytest.mark.parametrize("mode", [A16, A8])
+@pytest.mark.parametrize("roomy", [0, 1])
+def test_both_index_widths_in_one_launch_give_the_bits_of_two_launches(mode, roomy):
+    """16-row tiles: a 2-bit pool and an 8-bit pool of one mode ride one launch (the default) or one
+    launch per index width (widths_apart); the same work either way.  The 8-bit table is a 256-entry
+    fp16 grid in WxA16 and the identity idx - 128 in WxA8."""
+    from dartmoq_hip import ops
+    k, inter = 384, 128
+    counts0, counts1 = [5, 40, 0, 17], [21, 2]
+    r0, r1 = sum(counts0), sum(counts1)
+    rows = r0 + r1
+    g = torch.Generator().manual_seed(91 + mode)
+    x_rot = torch.randn(rows, k, generator=g) * 0.7
+    cb2 = codebook.get_codebook(2)[0].half()
+    act, scale, _, _, lut2, _, _, _, wsb = _mode_inputs(mode, x_rot, cb2)
+    lut8 = None if mode == A8 else (torch.arange(256).float() - 128).mul(3.0 / 128).half()
+    pools, infos = [], []
+    for pi, (bit, counts, first_row, lut) in enumerate([(2, counts0, 0, lut2), (8, counts1, r0, lut8)]):
+        idx_gf, norms_gf, _ = _pool(2, 2 * inter * len(counts), k, 400 + pi)
+        if bit == 8:                                   # one index byte per weight
+            idx_gf = torch.randint(0, 256, (k // 128, 2 * inter * len(counts), 128), dtype=torch.uint8,
+                                   generator=g)
+        starts = [first_row + sum(counts[:e]) for e in range(len(counts))]
+        info = torch.tensor([(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(len(counts))],
+                            dtype=torch.int32).cuda()
+        infos.append(info)
+        pools.append(dict(w=idx_gf.cuda(), norms=norms_gf.cuda(), lut=None if lut is None else lut.cuda(),
+                          expert_info=info, act=act.cuda(), act_scale=None if scale is None else scale.cuda(),
+                          row_index=None, bit=bit, mode=mode, w_scale_byte=wsb))
+    lists = [ops.build_tiles(infos[pi], rows, 16, pool=pi) for pi in range(2)]
+    n = [int(l[0][0]) for l in lists]
+    items = torch.cat([lists[0][1][:n[0]], lists[1][1][:n[1]]]).contiguous()
+    n_items = torch.tensor([n[0] + n[1], 0, 0, 0], dtype=torch.int32).cuda()
+    common = dict(groups=k // 128, n_out=inter, half_width=inter, slice_is_groups=False, tt=1,
+                  out_stride=inter, act_row_bytes=act.element_size() * k,
+                  act_scale_stride=0 if scale is None else scale.stride(0), roomy=roomy)
+    one = torch.full((rows, inter), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_pools(mode, SILU, pools, items, n_items, items.shape[0], out=one, **common)
+    two = torch.full((rows, inter), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_pools(mode, SILU, pools, items, n_items, items.shape[0], out=two, widths_apart=1, **common)
+    torch.cuda.synchronize()
+    assert not torch.isnan(one.float()).any()
+    assert torch.equal(one, two)
+
+
 @pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])
 @pytest.mark.parametrize("bit", [1, 2, 4])
 def test_merged_in_features_down(mode, bit):

@@ -123,10 +123,11 @@ def test_layer_with_shared_expert(shared_layer, mode, tokens, tt):
 
 
 @pytest.mark.parametrize("mode", ["wxa16", "wxa8", "wxfp8", "wxfp4"])
-@pytest.mark.parametrize("tokens", [1, 90])
+@pytest.mark.parametrize("tokens", [1, 90, 700])
 def test_layer_with_8bit_shared_expert(small_layer, mode, tokens):
-    """The shared expert of a real checkpoint is quantized with the 8-bit uniform codebook: its
-    slices are work items of separate launches for 8-bit pools (int8 path under wxfp4)."""
+    """The shared expert of a real checkpoint is quantized with the 8-bit uniform codebook (int8
+    path under wxfp4): its slices are work items of the 16-row launch that serves both index widths
+    (1 and 90 tokens) or of separate launches for 8-bit pools (700 tokens)."""
     import dataclasses
     layer = moe.add_shared_expert(dataclasses.replace(small_layer, shared=None), small_layer.inter,
                                   seed=31, bit=8, uniform_codebook=True)

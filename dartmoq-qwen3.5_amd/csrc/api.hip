@@ -341,7 +341,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   const bool both_widths = any_wide && !a->widths_apart && a->tt == 1 && ks == 1 && a->k_split <= 1 && !a->dbg_acc &&
                            mode2 < 0 && a->nt != 1 && a->epi != DMQ_EPI_STORE && a->mode != DMQ_MODE_FP4;
   if (a->epi == DMQ_EPI_SILU_ROT) {
-    if (ks != 1 || (any_wide && !both_widths)) return DMQ_ERR_MODE;
+    if (ks != 1) return DMQ_ERR_MODE;
     if (a->n_out % DMQ_GS) return DMQ_ERR_ALIGN;
     if (!a->post_out || (a->mode != DMQ_MODE_A16 && !a->post_scale)) return DMQ_ERR_NULL;
     for (int i = 0; i < a->n_pools; ++i)
@@ -907,18 +907,14 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   }
 
   // The gate_up GEMM rotates (and quantizes) its SiLU*up rows for the down projection itself when
-  // a workgroup owns whole blocks of 128 features: no K split, no 8-bit pools in the mode.
+  // a workgroup owns whole blocks of 128 features: no K split over the waves.
   // 8-bit pools next to narrower ones: up to about a hundred work items one 16-row launch serves
   // both index widths and fuses as well (dmq_gemm_args.widths_apart; configs[3] with the reference's
   // default 8-bit shared expert, wxa8: 64 tokens 133 -> 107 us, 128 tokens 153 -> 146, 256 tokens
   // 196 -> 240, so beyond 1280 routed rows the widths keep their own launches).
   const bool widths_apart = tt != 1 || (long)tokens * K > 1280;
   bool fuse_rot[DMQ_MAX_POOLS];
-  for (int mi = 0; mi < n_modes; ++mi) {
-    fuse_rot[mi] = (ks == 1);
-    for (int i = 0; i < P; ++i)
-      if (layer->pool[i].mode == modes[mi] && layer->pool[i].bit == 8 && widths_apart) fuse_rot[mi] = false;
-  }
+  for (int mi = 0; mi < n_modes; ++mi) fuse_rot[mi] = (ks == 1);
 
   // Which pools rotate every token once instead of their routed rows: the caller's choice (pools
   // expected to see more routed rows than tokens) and, for small batches, all of them: rotating a

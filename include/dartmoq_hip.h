@@ -305,10 +305,10 @@ typedef struct {
   int mode2_on;
   int mode2;
   /* A launch with 8-bit pools next to narrower ones, tt == 1, no K sharing, not WxFP4, not the plain
-   * store: one kernel instance serves both index widths in ONE launch (two workgroups per CU; it
-   * also lets DMQ_EPI_SILU_ROT cover 8-bit pools).  widths_apart != 0 keeps the two launches (the
-   * narrower pools then run three workgroups per CU, which wins once the list holds more than
-   * about a hundred work items; DMQ_EPI_SILU_ROT with 8-bit pools is then refused).  Same results. */
+   * store: one kernel instance serves both index widths in ONE launch (two
+   * workgroups per CU).  widths_apart != 0 keeps the two launches (the narrower pools then run
+   * three workgroups per CU, which wins once the list holds more than about a hundred work
+   * items).  Same results. */
   int widths_apart;
 } dmq_gemm_args;
 

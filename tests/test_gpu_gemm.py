@@ -391,22 +391,26 @@ def test_gemm_argument_errors():
                           groups=4, n_out=128, slice_is_groups=False, rows_total=16, tt=1)
 
 
-@pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])
+@pytest.mark.parametrize("mode,bit", [(A16, 2), (A8, 2), (FP8, 2), (FP4, 2), (A16, 8), (A8, 8)])
 @pytest.mark.parametrize("tt,nbl", [(1, 1), (2, 2), (4, 1)])
-def test_fused_down_rotation_equals_separate_kernels(mode, tt, nbl):
+def test_fused_down_rotation_equals_separate_kernels(mode, bit, tt, nbl):
     """DMQ_EPI_SILU_ROT: the gate_up GEMM hands over the rotated (+ quantized) input of the down
     projection.  It must be bit for bit what the SiLU epilogue followed by the per-expert rotation
-    kernel produces (same fp16 SiLU*up rows, same MFMA order, same quantizer)."""
+    kernel produces (same fp16 SiLU*up rows, same MFMA order, same quantizer).  8-bit pools: a
+    256-entry fp16 grid in WxA16, the identity idx - 128 (no table) in WxA8."""
     from dartmoq_hip import ops
     from dartmoq_hip._lib import EPI_SILU_ROT
-    bit, k, inter = 2, 256, 256
+    k, inter = 256, 256
     counts = [9, 70, 0, 33]
     n_exp = len(counts)
     starts, rows_total = _expert_rows(counts)
     g = torch.Generator().manual_seed(17 + mode)
-    idx_gf, norms_gf, cb = _pool(bit, 2 * inter * n_exp, k, 91)
+    idx_gf, norms_gf, cb = _pool(2, 2 * inter * n_exp, k, 91)
     x_rot = torch.randn(rows_total, k, generator=g) * 0.7
     act, scale, _oc, _os, lut, _ol, _wbs, nfac, wsb = _mode_inputs(mode, x_rot, cb)
+    if bit == 8:                                       # one index byte per weight
+        idx_gf = torch.randint(0, 256, (k // 128, 2 * inter * n_exp, 128), dtype=torch.uint8, generator=g)
+        lut = None if mode == A8 else (torch.arange(256).float() - 128).mul(3.0 / 128).half()
     norms_used = (norms_gf.float() * nfac).half() if mode == FP4 else norms_gf
     w_dev = idx_gf.cuda()
     if mode == FP4:
@@ -423,7 +427,7 @@ def test_fused_down_rotation_equals_separate_kernels(mode, tt, nbl):
                   rows_total=rows_total, w_scale_byte=wsb, tt=tt, nbl=nbl, tiling=tiling)
     args = (mode, bit)
     tens = (act.cuda(), None if scale is None else scale.cuda(), w_dev, norms_used.cuda(),
-            None if mode == FP4 else lut.cuda(), info_dev)
+            None if (mode == FP4 or lut is None) else lut.cuda(), info_dev)
     silu = ops.matmul_merged(*args, SILU, *tens, **common)
     # the rotation kernel takes the down slice of an expert from its own work items
     dn_items, ditems, dmax = ops.build_tiles(dinfo_dev, rows_total, 16 * tt)

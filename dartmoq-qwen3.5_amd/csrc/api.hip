@@ -338,7 +338,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (silu && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
   // 16-row tiles, no K sharing: the 8-bit pools and the others ride one launch (and the fused down
   // rotation is then open to 8-bit pools as well)
-  const bool both_widths = any_wide && !a->widths_apart && a->tt == 1 && ks == 1 && a->k_split <= 1 && !a->dbg_acc &&
+  const bool both_widths = any_wide && !a->widths_apart && a->tt == 1 && ks == 1 && !a->dbg_acc &&
                            mode2 < 0 && a->nt != 1 && a->epi != DMQ_EPI_STORE && a->mode != DMQ_MODE_FP4;
   if (a->epi == DMQ_EPI_SILU_ROT) {
     if (ks != 1) return DMQ_ERR_MODE;
@@ -356,12 +356,11 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (subs > 1 && wsplit > 1) return DMQ_ERR_MODE;
   }
   if (wsplit > 1) {
-    // SiLU epilogues: 2 or 4 workgroups, 1/2/4-bit pools; plain store (a Linear with a handful
-    // of rows): up to 16, any bit width
+    // SiLU epilogues: 2 or 4 workgroups; plain store (a Linear with a handful of rows): up to 16
     const bool store = a->epi == DMQ_EPI_STORE;
     if (!silu && !store) return DMQ_ERR_MODE;
     if (wsplit != 2 && wsplit != 4 && !(store && (wsplit == 8 || wsplit == 16))) return DMQ_ERR_MODE;
-    if (ks != 1 || a->tt != 1 || (any_wide && !store)) return DMQ_ERR_MODE;
+    if (ks != 1 || a->tt != 1) return DMQ_ERR_MODE;
     if (a->groups % wsplit || (silu && a->n_out % DMQ_GS)) return DMQ_ERR_ALIGN;
     if (!a->split_partial || !a->split_counter) return DMQ_ERR_NULL;
     if (a->split_rows <= 0) return DMQ_ERR_SHAPE;
@@ -812,7 +811,15 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   }
   if (tt <= 0) tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
   if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
-  if (ks == 0) ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
+  if (ks == 0) {
+    ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
+    // an 8-bit pool on the fp16 path (a shared expert with a 256-entry table) makes few, long work
+    // items: two workgroups per block pay up to 256 routed rows (configs[3] with such a shared
+    // expert, wxa16, 16 tokens: 88 -> 75 us; the int8 identity path gains nothing there)
+    if (ks == 1 && tt == 1 && (long)tokens * K <= 256 && (H / DMQ_GS) % 2 == 0)
+      for (int i = 0; i < P; ++i)
+        if (layer->pool[i].bit == 8 && layer->pool[i].mode == DMQ_MODE_A16) ks = -2;
+  }
   // ks < 0: -ks workgroups share the K range of a gate_up block; the other launches do not split
   const int wsplit = ks < 0 ? -ks : 1;
   if (ks < 0) {
@@ -1140,9 +1147,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     g.out = w.act; g.out_stride = I;
     g.post_out = actq_of(mode); g.post_row_bytes = (long)I * 2;
     g.post_scale = actq_scale_of(mode); g.post_scale_stride = scale_stride_for(mode, I);
-    bool mode_wide = false;
-    for (int i = 0; i < P; ++i) mode_wide |= (layer->pool[i].mode == mode && layer->pool[i].bit == 8);
-    if (wsplit_eff > 1 && !mode_wide) {
+    if (wsplit_eff > 1) {
       g.k_split = wsplit_eff; g.split_rows = w.split_rows;
       g.split_partial = w.split_partial; g.split_counter = w.split_counter;
     }

@@ -194,7 +194,7 @@ def test_both_index_widths_in_one_launch_give_the_bits_of_two_launches(mode, roo
     launch per index width (widths_apart); the same work either way.  The 8-bit table is a 256-entry
     fp16 grid in WxA16 and the identity idx - 128 in WxA8."""
     from dartmoq_hip import ops
-    k, inter = 384, 128
+    k, inter = 512, 128
     counts0, counts1 = [5, 40, 0, 17], [21, 2]
     r0, r1 = sum(counts0), sum(counts1)
     rows = r0 + r1
@@ -230,6 +230,16 @@ def test_both_index_widths_in_one_launch_give_the_bits_of_two_launches(mode, roo
     torch.cuda.synchronize()
     assert not torch.isnan(one.float()).any()
     assert torch.equal(one, two)
+    # K shared by 2 or 4 workgroups per block (partial sums added in fp32 by the last to arrive):
+    # the same sums in another order
+    for apart in (0, 1):
+        for share in (2, 4):
+            got = torch.full((rows, inter), float("nan"), dtype=torch.float16, device="cuda")
+            ops.matmul_pools(mode, SILU, pools, items, n_items, items.shape[0], out=got, widths_apart=apart,
+                             k_split=share, rows_total=rows, **common)
+            torch.cuda.synchronize()
+            torch.testing.assert_close(got.float(), one.float(), rtol=2e-3,
+                                       atol=2e-3 * one.float().abs().max().item())
 
 
 @pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])

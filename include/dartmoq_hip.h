@@ -256,9 +256,9 @@ typedef struct {
   int post_scale_stride;
   /* k_split = 2 or 4 (0 / 1 = off): the groups of one (work item, feature block) are shared by
    * that many workgroups, for short work lists that leave most of the chip idle.  tt == 1,
-   * ks <= 1, groups % k_split == 0; nbl is ignored.  With a SILU epilogue: 1/2/4-bit pools,
+   * ks <= 1, groups % k_split == 0, any bit width; nbl is ignored.  With a SILU epilogue:
    * n_out a multiple of 128, split_partial fp32 [k_split, split_rows, 2 * n_out].  With
-   * DMQ_EPI_STORE (a Linear with a handful of rows): k_split may also be 8 or 16, any bit width,
+   * DMQ_EPI_STORE (a Linear with a handful of rows): k_split may also be 8 or 16,
    * split_partial fp32 [k_split, split_rows, n_out].  split_rows >= every routed row index + 1.
    * Each workgroup parks its fp32 sums in its plane of split_partial and the last to arrive adds
    * the planes in a fixed order and runs the epilogue, so the result does not depend on the order
@@ -304,7 +304,7 @@ typedef struct {
    * (act_scale_stride, post_scale ...) are those of `mode`.  Same results as one launch per mode. */
   int mode2_on;
   int mode2;
-  /* A launch with 8-bit pools next to narrower ones, tt == 1, no K sharing, not WxFP4, not the plain
+  /* A launch with 8-bit pools next to narrower ones, tt == 1, ks <= 1, not WxFP4, not the plain
    * store: one kernel instance serves both index widths in ONE launch (two
    * workgroups per CU).  widths_apart != 0 keeps the two launches (the narrower pools then run
    * three workgroups per CU, which wins once the list holds more than about a hundred work

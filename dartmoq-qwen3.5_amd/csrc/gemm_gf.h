@@ -133,11 +133,11 @@ template <int N> __device__ __forceinline__ void dmq_load_words(const uint8_t* p
 // Expand the packed bytes of MFMA step S into the lane's operand words.
 // IDENT (int8 operands, 8-bit indices): the table is the identity w = idx - 128 of a uniform
 // codebook, so the operand bytes are the index bytes with the top bit flipped and no table is read.
-template <int MODE, int BIT, int S, bool IDENT = false>
+template <int MODE, int BIT, int S, bool IDENT = false, int ROW = DMQ_LUT_ROW>
 __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t lane_base,
                                                  const uint32_t* pk, uint32_t* w) {
   using T = ModeTraits<MODE>;
-  using G = LutGeom<BIT, T::ES>;
+  using G = LutGeom<BIT, T::ES, ROW>;
   constexpr int BYTES = (4 * BIT) / T::STEPS;           // packed bytes per step
   if constexpr (IDENT) {
     static_assert(MODE == DMQ_MODE_A8 && BIT == 8, "identity table: int8 operands, 8-bit indices");
@@ -149,14 +149,14 @@ __device__ __forceinline__ void dmq_dequant_step(const uint8_t* tbl, uint32_t la
     constexpr int b = decltype(bc)::value;
     constexpr int bi = S * BYTES + b;
     if constexpr (G::EB >= 4) {
-      dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], w + b * (G::EB / 4));
+      dmq_lut_read_word<BIT, T::ES, (bi & 3), ROW>(tbl, lane_base, pk[bi >> 2], w + b * (G::EB / 4));
     } else if constexpr (G::EB == 2) {                  // two two-byte entries per operand word
       uint32_t v;
-      dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], &v);
+      dmq_lut_read_word<BIT, T::ES, (bi & 3), ROW>(tbl, lane_base, pk[bi >> 2], &v);
       if (b & 1) w[b >> 1] |= v << 16; else w[b >> 1] = v;
     } else {                                            // four one-byte entries per operand word
       uint32_t v;
-      dmq_lut_read_word<BIT, T::ES, (bi & 3)>(tbl, lane_base, pk[bi >> 2], &v);
+      dmq_lut_read_word<BIT, T::ES, (bi & 3), ROW>(tbl, lane_base, pk[bi >> 2], &v);
       if (b & 3) w[b >> 2] |= v << (8 * (b & 3)); else w[b >> 2] = v;
     }
   };
@@ -218,7 +218,8 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
                                                        : (RED_BYTES > 16 ? RED_BYTES : 16);
 };
 
-template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG, bool IDENT = false>
+template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG, bool IDENT = false,
+          int ROW = DMQ_LUT_ROW>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
                                               uint8_t* smem2, uint8_t* smem_post, int token_start,
                                               int token_count, int slice_start, int post_slice,
@@ -249,7 +250,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   const int q = lane >> 4;
   const int kpart = wave % KS;
   const int rowpart = wave / KS;
-  const uint32_t lane_base = (MODE == DMQ_MODE_FP4) ? 0u : dmq_lut_lane_base<BIT, T::ES>(lane);
+  const uint32_t lane_base = (MODE == DMQ_MODE_FP4) ? 0u : dmq_lut_lane_base<BIT, T::ES, ROW>(lane);
 
   const int feat0 = (nb * ROWPARTS + rowpart) * (FEAT_TILES * 16);   // first output feature of the wave
   const bool wave_active = feat0 < p.n_out;                          // wave-uniform
@@ -348,11 +349,11 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   constexpr int WQ = (MODE == DMQ_MODE_FP4) ? 1 : T::STEPS * OPW;
   auto dequant_tile = [&](const uint32_t (&pkj)[WW], uint32_t (&w)[WQ]) {
     if constexpr (MODE != DMQ_MODE_FP4) {
-      dmq_dequant_step<MODE, BIT, 0, IDENT>(tbl, lane_base, pkj, w);
-      if constexpr (T::STEPS > 1) dmq_dequant_step<MODE, BIT, 1, IDENT>(tbl, lane_base, pkj, w + OPW);
+      dmq_dequant_step<MODE, BIT, 0, IDENT, ROW>(tbl, lane_base, pkj, w);
+      if constexpr (T::STEPS > 1) dmq_dequant_step<MODE, BIT, 1, IDENT, ROW>(tbl, lane_base, pkj, w + OPW);
       if constexpr (T::STEPS > 2) {
-        dmq_dequant_step<MODE, BIT, 2, IDENT>(tbl, lane_base, pkj, w + 2 * OPW);
-        dmq_dequant_step<MODE, BIT, 3, IDENT>(tbl, lane_base, pkj, w + 3 * OPW);
+        dmq_dequant_step<MODE, BIT, 2, IDENT, ROW>(tbl, lane_base, pkj, w + 2 * OPW);
+        dmq_dequant_step<MODE, BIT, 3, IDENT, ROW>(tbl, lane_base, pkj, w + 3 * OPW);
       }
     }
   };
@@ -377,7 +378,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         const half8_t n8 = {n, n, n, n, n, n, n, n};
         auto step = [&](auto sc) {
           constexpr int s = decltype(sc)::value;
-          if (j + 1 < NT) dmq_dequant_step<MODE, BIT, s, IDENT>(tbl, lane_base, pk[j + 1 < NT ? j + 1 : j], wn + s * OPW);
+          if (j + 1 < NT) dmq_dequant_step<MODE, BIT, s, IDENT, ROW>(tbl, lane_base, pk[j + 1 < NT ? j + 1 : j], wn + s * OPW);
           const half8_t a = __builtin_bit_cast(half8_t, (uint4_t){wq[4 * s], wq[4 * s + 1],
                                                                     wq[4 * s + 2], wq[4 * s + 3]}) * n8;
 #pragma unroll
@@ -516,7 +517,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     };
     // the first chunk is in flight while the look-up table is built
     if (g_lo < g_hi) load_chunk(g_lo);
-    if (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_build<BIT, T::ES>(tbl, pw.lut);
+    if (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_build<BIT, T::ES, ROW>(tbl, pw.lut);
     __syncthreads();
     for (int g0 = g_lo; g0 < g_hi; g0 += PF) {
       if (g0 != g_lo) load_chunk(g0);
@@ -827,7 +828,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
         auto look = [&](auto mc) {
           constexpr int m = decltype(mc)::value;
           if constexpr (m < 4 * NT)
-            dmq_dequant_step<MODE, BIT, m / NT, IDENT>(tbl, lane_base, pk[m % NT], wq[m % 3]);
+            dmq_dequant_step<MODE, BIT, m / NT, IDENT, ROW>(tbl, lane_base, pk[m % NT], wq[m % 3]);
         };
         read_b(std::integral_constant<int, 0>{}, braw[0]);
         look(std::integral_constant<int, 0>{});
@@ -962,7 +963,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
       load_packed(lk, g_first + lg, pkb[u]);
       next_load();
     }
-    if constexpr (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_store_wave<BIT, T::ES>(tbl, wave, lutw);
+    if constexpr (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_store_wave<BIT, T::ES, ROW>(tbl, wave, lutw);
     stage_store(0, srb[0]);
     __syncthreads();
     int cg = 0;                                        // group of the step being computed
@@ -1073,8 +1074,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((!WIDE && K
 void dmq_gemm_gf_kernel(GemmParams p) {
   constexpr int S2A = dmq_smem2_bytes<MODE, NT, TT, KS>(), S2B = dmq_smem2_bytes<MODE2, NT, TT, KS>();
   constexpr int PSA = dmq_post_bytes<MODE, TT, EPI>(), PSB = dmq_post_bytes<MODE2, TT, EPI>();
+  // table rows of 256 bytes where two workgroups per CU leave the room (see LutGeom) and the K
+  // range is long enough to pay for writing 64 KiB of table: the gate_up launches (K = hidden
+  // size), not the down projection (four groups per block at I = 512: measured slower there)
+  constexpr int ROW = (ROOMY && (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT)) ? 256 : DMQ_LUT_ROW;
   __shared__ __attribute__((aligned(16))) uint8_t
-      tbl[(MODE == DMQ_MODE_FP4 && (MODE2 < 0 || MODE2 == DMQ_MODE_FP4)) ? 16 : DMQ_LUT_BYTES];
+      tbl[(MODE == DMQ_MODE_FP4 && (MODE2 < 0 || MODE2 == DMQ_MODE_FP4)) ? 16 : 256 * ROW];
   __shared__ __attribute__((aligned(16))) uint8_t smem2[S2A > S2B ? S2A : S2B];
   __shared__ __attribute__((aligned(16))) uint8_t smem_post[PSA > PSB ? PSA : PSB];
   static_assert(MODE2 < 0 || (!WIDE && !DBG && NT == 4), "two modes: 1/2/4-bit pools, four n-tiles per wave");
@@ -1158,23 +1163,23 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   auto run = [&](auto mode_tag) __attribute__((always_inline)) {
     constexpr int M = decltype(mode_tag)::value;
     if constexpr (M == DMQ_MODE_FP4) {
-      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
       return;
     }
     if constexpr (M != DMQ_MODE_FP4 && WIDE != 0) {
       if (WIDE == 1 || pw.bit == 8) {                    // uniform over the workgroup
         if (M == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
-          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
         else
-          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
         return;
       }
     }
     if constexpr (M != DMQ_MODE_FP4 && WIDE != 1) {
       switch (pw.bit) {
-        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
       }
     }
   };

@@ -6,25 +6,28 @@
 // each for the int8 / e4m3 look-ups), so dequantizing costs one LDS read per
 // packed byte.  Every entry is replicated across a row of DMQ_LUT_ROW bytes; lane L
 // reads the copy at (L % copies) so that the lanes of a wave hit distinct LDS banks
-// whatever byte values they look up.  128-byte rows (a 32 KiB table) measured faster than
-// 256-byte rows on MI355X: three workgroups fit a CU instead of two, which outweighs the
-// cheaper address arithmetic ((byte << 8) | lane offset is one byte permute) of wide rows.
+// whatever byte values they look up.  128-byte rows (a 32 KiB table) let three workgroups share a
+// CU; the kernel instances that keep two per CU anyway take 256-byte rows (64 KiB), where the
+// address of a look-up, (byte << 8) | lane offset, is one byte permute (see LutGeom).
 #pragma once
 #include "common.h"
 
 #define DMQ_LUT_ROW 128
 #define DMQ_LUT_BYTES (256 * DMQ_LUT_ROW)
 
-template <int BIT, int ES>   // ES = bytes per dequantized element (2: fp16, 1: int8 / e4m3)
+// ROW = bytes of a table row (all copies of one entry): 128, or 256 for the kernel instances that
+// keep two workgroups per CU anyway (a 64 KiB table; the address of a look-up is then one byte
+// permute instead of a bit-field extract and a shift-or)
+template <int BIT, int ES, int ROW = DMQ_LUT_ROW>   // ES = bytes per dequantized element (2: fp16, 1: int8 / e4m3)
 struct LutGeom {
   static constexpr int ELEMS = 8 / BIT;                 // elements per packed byte
   static constexpr int EB = ELEMS * ES;                 // payload bytes per entry
   static constexpr int STRIDE = EB < 4 ? 4 : EB;        // bytes between copies
-  static constexpr int COPIES = DMQ_LUT_ROW / STRIDE;
+  static constexpr int COPIES = ROW / STRIDE;
   // 2-bit codebooks (4 values: 8 bytes of fp16, 4 bytes of int8 / e4m3) fit the source operands
   // of one byte permute, so every lane composes table entries itself instead of receiving them
   // from the lane that fetched them
-  static constexpr bool PERM_BUILD = (BIT == 2) && (DMQ_LUT_ROW == 128);
+  static constexpr bool PERM_BUILD = (BIT == 2);
 };
 
 // Entry `e` of the table: the codebook values of the 8/BIT indices packed in byte value e.
@@ -60,22 +63,23 @@ __device__ __forceinline__ void dmq_lut_fetch(const void* codebook, int e, uint3
 // Write the 64 entries a wave fetched (lane i holds entry 64*wave + i) with all their copies.
 // Each store covers 256 contiguous bytes, one dword per lane, so it touches every LDS bank once;
 // the entry words are broadcast from the lane that fetched them.
-template <int BIT, int ES>
+template <int BIT, int ES, int ROW = DMQ_LUT_ROW>
 __device__ __forceinline__ void dmq_lut_store_wave(uint8_t* tbl, int wave, const uint32_t (&w)[4]) {
-  using G = LutGeom<BIT, ES>;
+  using G = LutGeom<BIT, ES, ROW>;
   constexpr int DW = G::STRIDE / 4;                     // dwords per copy
-  constexpr int RPW = 256 / DMQ_LUT_ROW;                // table rows per 256-byte store
+  constexpr int RPW = 256 / ROW;                        // table rows per 256-byte store
   const int lane = threadIdx.x & 63;
   if constexpr (G::PERM_BUILD) {
-    // Store t of wave v covers the eight entries 64 v + 8 t .. + 7: lane l writes 16 bytes (two or
-    // four copies) of entry e = 64 v + 8 t + l / 8.  The four indices of e are (l/8) & 3,
-    // ((l/8) >> 2) | (t & 1) << 1, t >> 1 and v: only the first two depend on the lane.
-    const uint32_t sub = (uint32_t)lane >> 3;
-    uint8_t* dst = tbl + ((long)wave * 64 + sub) * DMQ_LUT_ROW + (lane & 7) * 16;
+    // A store covers 64 * 16 / ROW whole rows: lane l writes 16 bytes (two or four copies) of entry
+    // e = 64 v + EPS t + l / LPR.  The four indices of e are its 2-bit digits; the top one is the wave.
+    constexpr int LPR = ROW / 16;                       // lanes per row
+    constexpr int EPS = 64 / LPR;                       // entries per store
+    const uint32_t sub = (uint32_t)lane / LPR;
+    uint8_t* dst = tbl + ((long)wave * 64 + sub) * ROW + (lane % LPR) * 16;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const uint32_t i0 = sub & 3u, i1 = (sub >> 2) | ((uint32_t)(t & 1) << 1);
-      const uint32_t i2 = (uint32_t)(t >> 1), i3 = (uint32_t)wave;
+    for (int t = 0; t < 64 / EPS; ++t) {
+      const uint32_t el = (uint32_t)t * EPS + sub;      // entry of this wave
+      const uint32_t i0 = el & 3u, i1 = (el >> 2) & 3u, i2 = (el >> 4) & 3u, i3 = (uint32_t)wave;
       uint4_t v;
       if (ES == 2) {
         const uint32_t s0 = 0x01000100u + i0 * 0x0202u + i1 * 0x02020000u;
@@ -88,12 +92,12 @@ __device__ __forceinline__ void dmq_lut_store_wave(uint8_t* tbl, int wave, const
         const uint32_t e0 = __builtin_amdgcn_perm(0u, w[0], sel);
         v = (uint4_t){e0, e0, e0, e0};
       }
-      *(uint4_t*)(dst + t * 8 * DMQ_LUT_ROW) = v;
+      *(uint4_t*)(dst + t * EPS * ROW) = v;
     }
     return;
   }
   const int d = lane % DW;
-  uint32_t* dst = (uint32_t*)(tbl + (long)wave * 64 * DMQ_LUT_ROW) + lane;
+  uint32_t* dst = (uint32_t*)(tbl + (long)wave * 64 * ROW) + lane;
 #pragma unroll
   for (int t = 0; t < 64 / RPW; ++t) {
     uint32_t v = 0u;
@@ -107,37 +111,37 @@ __device__ __forceinline__ void dmq_lut_store_wave(uint8_t* tbl, int wave, const
         const uint32_t e3 = __builtin_amdgcn_readlane(w[3], i);
         e = (d == 2) ? e2 : ((d == 3) ? e3 : e);
       }
-      v = (RPW == 1 || (lane * 4) / DMQ_LUT_ROW == r) ? e : v;
+      v = (RPW == 1 || (lane * 4) / ROW == r) ? e : v;
     }
     dst[t * 64] = v;
   }
 }
 
 // Build the table with a workgroup of 256 threads; caller syncs afterwards.
-template <int BIT, int ES>
+template <int BIT, int ES, int ROW = DMQ_LUT_ROW>
 __device__ __forceinline__ void dmq_lut_build(uint8_t* tbl, const void* codebook) {
   uint32_t w[4];
   dmq_lut_fetch<BIT, ES>(codebook, threadIdx.x, w);
-  dmq_lut_store_wave<BIT, ES>(tbl, threadIdx.x >> 6, w);
+  dmq_lut_store_wave<BIT, ES, ROW>(tbl, threadIdx.x >> 6, w);
 }
 
-template <int BIT, int ES>
+template <int BIT, int ES, int ROW = DMQ_LUT_ROW>
 __device__ __forceinline__ uint32_t dmq_lut_lane_base(int lane) {
-  using G = LutGeom<BIT, ES>;
+  using G = LutGeom<BIT, ES, ROW>;
   return (uint32_t)(lane % G::COPIES) * G::STRIDE;
 }
 
 // Look up byte K (0..3) of a packed word.  out receives EB bytes (rounded up to whole words).
-template <int BIT, int ES, int K>
+template <int BIT, int ES, int K, int ROW = DMQ_LUT_ROW>
 __device__ __forceinline__ void dmq_lut_read_word(const uint8_t* tbl, uint32_t lane_base,
                                                   uint32_t word, uint32_t* out) {
-  using G = LutGeom<BIT, ES>;
+  using G = LutGeom<BIT, ES, ROW>;
   uint32_t off;
-  if (DMQ_LUT_ROW == 256) {
+  if (ROW == 256) {
     // result bytes: [0] lane offset, [1] byte K of the word, [2] = [3] = 0
     off = __builtin_amdgcn_perm(word, lane_base, 0x0c0c0400u + ((uint32_t)K << 8));
   } else {
-    off = (((word >> (8 * K)) & 0xffu) * DMQ_LUT_ROW) + lane_base;
+    off = (((word >> (8 * K)) & 0xffu) * ROW) + lane_base;
   }
   const uint8_t* p = tbl + off;
   if (G::EB == 1) {

@@ -219,7 +219,7 @@ template <int MODE, int NT, int TT, int KS> struct GemmGeom {
 };
 
 template <int MODE, int BIT, int NT, int TT, int EPI, int KS, bool DBG, bool IDENT = false,
-          int ROW = DMQ_LUT_ROW>
+          int ROW = DMQ_LUT_ROW, bool AHEAD = false>
 __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& pw, uint8_t* tbl,
                                               uint8_t* smem2, uint8_t* smem_post, int token_start,
                                               int token_count, int slice_start, int post_slice,
@@ -362,10 +362,15 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
   // running sums.  This drops the per-group accumulators (32 registers at TT = 2, which is
   // what lets a third workgroup fit a CU) at the price of one fp16 rounding per weight.
   constexpr bool FOLD = (MODE == DMQ_MODE_A16) && STAGE && (TT >= DMQ_FOLD_MIN_TT);
+  // PREF (16-row tiles of the two-per-CU instances): the operands of n-tile 0 were looked up
+  // while the previous group finished (wpre), so a group does not start on an LDS round trip
+  // that nothing hides when the wave has its SIMD to itself.
+  constexpr bool PREF = AHEAD && GG::STAGE && TT == 1 && MODE != DMQ_MODE_FP4 && NT > 1;
+  uint32_t wpre[WQ];
   auto compute = [&](int g, const uint32_t (&pk)[NT][WW], const uint2_t (&nr)[NT],
                      const uint32_t (&xa)[TT][AW], const float (&xs)[TT], const int (&xsb)[TT]) {
     uint32_t wqb[2][WQ];
-    dequant_tile(pk[0], wqb[0]);
+    if constexpr (!PREF) dequant_tile(pk[0], wqb[0]);
     if constexpr (FOLD) {
       // Explicit software pipeline, one fence per MFMA step: scale this step's operand, issue a
       // quarter of the next tile's look-ups, then the TT matrix instructions of the step.  The
@@ -399,7 +404,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       if (j + 1 < NT) dequant_tile(pk[j + 1], wqb[(j + 1) & 1]);
-      const uint32_t (&wq)[WQ] = wqb[j & 1];
+      const uint32_t (&wq)[WQ] = (PREF && j == 0) ? wpre : wqb[j & 1];
       acc_t acc[TT];
 #pragma unroll
       for (int t = 0; t < TT; ++t) acc[t] = (acc_t){0, 0, 0, 0};
@@ -966,6 +971,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     if constexpr (MODE != DMQ_MODE_FP4 && !IDENT) dmq_lut_store_wave<BIT, T::ES, ROW>(tbl, wave, lutw);
     stage_store(0, srb[0]);
     __syncthreads();
+    if constexpr (PREF) dequant_tile(pkb[0][0], wpre);
     int cg = 0;                                        // group of the step being computed
     for (int sb = 0; sb < steps; sb += D) {
 #pragma unroll
@@ -982,6 +988,8 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
             int xsb[TT];
             stage_read(u & 1, xa, nr, xs, xsb);
             compute(cg, pkb[u], nr, xa, xs, xsb);
+            // n-tile 0 of the next step (a step past the last one looks a stale entry up: unused)
+            if constexpr (PREF) dequant_tile(pkb[(u + 1) % D][0], wpre);
           }
         }
         load_packed(lk, g_first + lg, pkb[u]);
@@ -1163,23 +1171,23 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   auto run = [&](auto mode_tag) __attribute__((always_inline)) {
     constexpr int M = decltype(mode_tag)::value;
     if constexpr (M == DMQ_MODE_FP4) {
-      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
       return;
     }
     if constexpr (M != DMQ_MODE_FP4 && WIDE != 0) {
       if (WIDE == 1 || pw.bit == 8) {                    // uniform over the workgroup
         if (M == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
-          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
         else
-          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
         return;
       }
     }
     if constexpr (M != DMQ_MODE_FP4 && WIDE != 1) {
       switch (pw.bit) {
-        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
       }
     }
   };

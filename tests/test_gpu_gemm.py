@@ -453,6 +453,16 @@ def test_fused_down_rotation_equals_separate_kernels(mode, bit, tt, nbl):
     assert torch.equal(codes.view(torch.uint8), want.view(torch.uint8))
     if sc is not None:
         assert torch.equal(sc.view(torch.uint8), want_scale.view(torch.uint8))
+    if tt == 1 and bit != 8 and mode != FP4:
+        # the two-per-CU instance (256-byte table rows, look-ups of the next group issued ahead)
+        codes2, sc2, _ = ops._alloc_codes(mode, rows_total, inter, "cuda", False)
+        codes2.view(torch.uint8).fill_(0x5a)
+        ops.matmul_merged(*args, EPI_SILU_ROT, *tens, out=silu, out_stride=inter, roomy=1,
+                          post=dict(rot=[rot], extra=[extra], out=codes2, scale=sc2), **common)
+        torch.cuda.synchronize()
+        assert torch.equal(codes2.view(torch.uint8), want.view(torch.uint8))
+        if sc2 is not None:
+            assert torch.equal(sc2.view(torch.uint8), want_scale.view(torch.uint8))
 
 
 @pytest.mark.parametrize("mode", [A16, A8, FP4])

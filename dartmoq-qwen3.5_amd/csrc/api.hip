@@ -1041,7 +1041,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   {
     const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
     const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
-    // up to 256 routed rows with the top-k at hand: the one-row-per-thread ranking kernel
+    // up to DMQ_ROUTE_RANK_ROWS (128) routed rows with the top-k at hand: the one-row-per-thread ranking kernel
     const int* rank_idx = topk_done ? w.topk_idx
                                     : ((!router->logits && n_shared == 0) ? (const int*)router->topk_idx : nullptr);
     const float* rank_w = topk_done ? w.topk_w

@@ -834,7 +834,8 @@ void dmq_route_small_kernel(RouteSmallParams p) {
 
 // See RouteRankParams.  Rows with an expert id outside the layer rank behind all others and get no
 // entry anywhere (like the counting sort, which skips them).
-__global__ __launch_bounds__(256)
+#define DMQ_ROUTE_RANK_THREADS 256
+__global__ __launch_bounds__(DMQ_ROUTE_RANK_THREADS)
 void dmq_route_rank_kernel(RouteRankParams p) {
   __shared__ __attribute__((aligned(16))) int s_expert[DMQ_ROUTE_RANK_ROWS + 4];
   __shared__ __attribute__((aligned(16))) int s_tiles[DMQ_ROUTE_RANK_ROWS + 4];
@@ -844,10 +845,13 @@ void dmq_route_rank_kernel(RouteRankParams p) {
   const float w = mine ? p.in_w[r] : 0.f;
   const bool valid = mine && e >= 0 && e < p.experts;
   if (!valid) e = 0x7fffffff;
-  s_expert[r] = e;
-  s_tiles[r] = 0;
+  // the workgroup has more threads than the list has entries (the extra ones only help with the
+  // clearing and the per-expert counts): they own no list entry
+  static_assert(DMQ_ROUTE_RANK_ROWS <= DMQ_ROUTE_RANK_THREADS && DMQ_ROUTE_RANK_ROWS % 4 == 0,
+                "one list entry per thread, read four at a time");
+  if (r < DMQ_ROUTE_RANK_ROWS) { s_expert[r] = e; s_tiles[r] = 0; }
   if (r < 4) { s_expert[DMQ_ROUTE_RANK_ROWS + r] = 0x7fffffff; s_tiles[DMQ_ROUTE_RANK_ROWS + r] = 0; }
-  for (int i = r; i < p.clear_count; i += 256) p.clear_words[i] = 0;
+  for (int i = r; i < p.clear_count; i += DMQ_ROUTE_RANK_THREADS) p.clear_words[i] = 0;
   // slice of the expert in the first pool that holds one: in flight during the scan
   int pool = 0, ss = -1;
   if (valid) {
@@ -897,7 +901,7 @@ void dmq_route_rank_kernel(RouteRankParams p) {
       it[1] = (int4_t){cnt, ss, ss / (2 * DMQ_GS), 0};
     }
   }
-  for (int x = r; x < p.experts; x += 256) {
+  for (int x = r; x < p.experts; x += DMQ_ROUTE_RANK_THREADS) {
     int c = 0;
     for (int q = 0; q < rows4; ++q) {
       const int4_t e4 = *(const int4_t*)(s_expert + 4 * q);
@@ -1040,7 +1044,7 @@ int dmq_route_small_launch(const RouteSmallParams& p, hipStream_t stream) {
 int dmq_route_rank_launch(const RouteRankParams& p, hipStream_t stream) {
   if (p.rows <= 0 || p.rows > DMQ_ROUTE_RANK_ROWS || p.k <= 0 || p.tile_rows <= 0) return DMQ_ERR_LIMIT;
   if (p.pools <= 0 || p.pools > DMQ_MAX_POOLS || p.experts <= 0) return DMQ_ERR_LIMIT;
-  hipLaunchKernelGGL(dmq_route_rank_kernel, dim3(1), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL(dmq_route_rank_kernel, dim3(1), dim3(DMQ_ROUTE_RANK_THREADS), 0, stream, p);
   return dmq_check_launch();
 }
 

@@ -43,6 +43,8 @@ static inline int pick_ks(int tt, long rows, int groups) {
 #define DMQ_TT4_MIN_AVG 112
 #define DMQ_HOIST_ALL_TOKENS 1024
 #define DMQ_TAIL_SLOTS 96
+// routed rows from which an fp16 layer is cut into work items of 128 rows (the persistent GEMM)
+#define DMQ_ROWS_MIN_ROUTED 8192
 
 // Feature blocks one workgroup walks back to back.  With few row tiles every block gets its own
 // workgroup (parallelism); with many, a workgroup amortizes its start-up over several blocks.
@@ -53,7 +55,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 18; }
+int dmq_abi_version(void) { return 19; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -139,7 +141,8 @@ static int route_permute_ordered(const void* topk_idx, const void* topk_w, int t
                       int max_items, void* counts, void* offsets, void* sorted_tokens,
                       void* sorted_weights, void* sorted_rows, void* gu_info, void* dn_info,
                       void* n_items, void* items, void* scratch, size_t scratch_bytes,
-                      const int* pool_order, int lead_pools, void* stream) {
+                      const int* pool_order, int lead_pools, void* stream, int* zero_words = nullptr,
+                      int zero_count = 0) {
   if (!topk_idx || !topk_w || !slice_start || !slice_count || !counts || !offsets ||
       !sorted_tokens || !sorted_weights || !sorted_rows || !gu_info || !dn_info || !n_items ||
       !items || !scratch)
@@ -157,6 +160,7 @@ static int route_permute_ordered(const void* topk_idx, const void* topk_w, int t
   plan.n_items = (int*)n_items; plan.items = (int*)items;
   for (int i = 0; i < DMQ_MAX_POOLS; ++i) plan.pool_order[i] = pool_order ? pool_order[i] : i;
   plan.lead_pools = pool_order ? lead_pools : -1;
+  plan.zero_words = zero_words; plan.zero_count = zero_words ? zero_count : 0;
   if ((long)tokens * k <= DMQ_ROUTE_SMALL_ROWS && experts <= DMQ_ROUTE_SMALL_EXPERTS && k <= 64) {
     RouteSmallParams sp{};                   // one launch instead of three
     sp.in_idx = (const int*)topk_idx; sp.in_w = (const float*)topk_w;
@@ -311,7 +315,19 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (!valid_mode(a->mode)) return DMQ_ERR_MODE;
   if (a->epi < DMQ_EPI_STORE || a->epi > DMQ_EPI_SILU_ROT) return DMQ_ERR_MODE;
   const int ks = a->ks > 0 ? a->ks : 1;
-  if (!dmq_gemm_config_ok(a->tt, ks)) return DMQ_ERR_MODE;
+  const bool rows_kernel = a->tt == DMQ_ROWS_TT;          // work items of 128 rows (fp16 pools)
+  if (!rows_kernel && !dmq_gemm_config_ok(a->tt, ks)) return DMQ_ERR_MODE;
+  if (rows_kernel) {
+    if (a->mode != DMQ_MODE_A16 || mode2 >= 0 || ks != 1 || a->k_split > 1 || a->dbg_acc || any_wide ||
+        (a->nt != 0 && a->nt != 4) || (a->item_tile_rows != 0 && a->item_tile_rows != DMQ_ROWS_TILE) ||
+        a->width_filter != 0 || a->accumulate)
+      return DMQ_ERR_MODE;
+    if (a->groups % 4) return DMQ_ERR_ALIGN;
+    if (!a->rows_queue) return DMQ_ERR_NULL;
+    if (a->max_items > DMQ_ROWS_MAX_ITEMS) return DMQ_ERR_LIMIT;
+    // lane offsets into the activation rows are 32 bits wide
+    if ((long)a->max_items * DMQ_ROWS_TILE * a->act_row_bytes > 0xffffffffL) return DMQ_ERR_LIMIT;
+  }
   if (!a->items || !a->n_items || (!a->out && a->epi != DMQ_EPI_SILU_ROT)) return DMQ_ERR_NULL;
   for (int i = 0; i < a->n_pools; ++i) {
     const dmq_gemm_pool& q = a->pool[i];
@@ -334,7 +350,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
                  a->dbg_acc || a->k_split > 1))
     return DMQ_ERR_MODE;
   const int feat_per_wave = silu ? 32 : (one_tile ? 16 : 64);
-  if (a->n_out % feat_per_wave) return DMQ_ERR_ALIGN;
+  if (a->n_out % (rows_kernel ? 4 * feat_per_wave : feat_per_wave)) return DMQ_ERR_ALIGN;
   if (silu && (a->half_width != a->n_out)) return DMQ_ERR_SHAPE;
   // 16-row tiles, no K sharing: the 8-bit pools and the others ride one launch (and the fused down
   // rotation is then open to 8-bit pools as well)
@@ -350,7 +366,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   if (a->act_row_bytes < (long)a->groups * act_bytes_per_group(a->mode)) return DMQ_ERR_SHAPE;
   const int wsplit = a->k_split > 1 ? a->k_split : 1;
   int subs = 1;
-  if (a->item_tile_rows > 0) {
+  if (a->item_tile_rows > 0 && !rows_kernel) {
     if (a->item_tile_rows % (16 * a->tt)) return DMQ_ERR_ALIGN;
     subs = a->item_tile_rows / (16 * a->tt);
     if (subs > 1 && wsplit > 1) return DMQ_ERR_MODE;
@@ -411,6 +427,18 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   L.roomy = (a->roomy != 0 && a->tt == 1 && ks == 1 && !L.dbg) ? 1 : 0;
   L.mode2 = mode2;
   L.stream = (hipStream_t)stream;
+  if (rows_kernel) {
+    // a unit is a run of feature blocks of one work item: the smallest run that gives 16 group steps
+    // (8 at least, or the unit after it cannot be looked up while it runs)
+    p.n_blocks = a->n_out / (4 * feat_per_wave);
+    int run = 0;
+    for (int want = 16; want >= DMQ_ROWS_MIN_STEPS && !run; want -= 8)
+      for (int d = 1; d <= p.n_blocks && !run; ++d)
+        if (p.n_blocks % d == 0 && d * a->groups >= want) run = d;
+    if (!run) run = p.n_blocks;                          // short units: drawn one after the other
+    p.nbl = run; p.tail_slots = 0; p.spread = 0;
+    return dmq_gemm_rows_launch(p, a->epi, (int*)a->rows_queue, run, (hipStream_t)stream);
+  }
   // the 1/2/4-bit pools and the 8-bit pools of the mode are separate launches over the same work
   // list (each skips the items of the other kind); 8-bit pools never split K over the waves
   for (int wide = 0; wide < 2; ++wide) {
@@ -691,6 +719,7 @@ struct MoeWorkspace {
   uint8_t *xq_rows, *xq_rows_scale, *act, *actq, *actq_scale;
   float* split_partial;              // gate_up K range shared between workgroups: fp32 sums
   int* split_counter;
+  int* rows_queue;                   // queue words of the persistent gate_up and down launches
   int split_rows, split_counters;
   void* sort_scratch;
   size_t sort_scratch_bytes;
@@ -720,7 +749,7 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   MoeWorkspace w;
   const size_t R = (size_t)tokens * L->top_k;
   const size_t E = L->experts, P = L->pools, H = L->hidden, I = L->inter;
-  w.tile_rows = 16 * tt;
+  w.tile_rows = tt == DMQ_ROWS_TT ? DMQ_ROWS_TILE : 16 * tt;
   // an expert of a sub-expert layer has work items in every pool that holds a share of it
   const size_t homes = L->n_widths > 0 && L->max_homes > 1 ? (size_t)L->max_homes : 1;
   w.max_items = (int)((R / w.tile_rows + E) * homes);
@@ -736,6 +765,7 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.gu_info = (int*)take(P * E * 16);
   w.dn_info = (int*)take(P * E * 16);
   w.n_items = (int*)take(16);
+  w.rows_queue = (int*)take(2 * DMQ_ROWS_QUEUE_WORDS * 4);
   w.sort_scratch_bytes = dmq_route_scratch_bytes(tokens, L->top_k, L->experts);
   w.sort_scratch = take(w.sort_scratch_bytes);
   w.items = (int*)take((size_t)w.max_items * DMQ_ITEM_WORDS * sizeof(int));
@@ -809,8 +839,21 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     if (layer->pool[i].mode == DMQ_MODE_FP4) wf4 += layer->pool[i].n_gate_up;
     else if (layer->pool[i].bit == 4) w4 += layer->pool[i].n_gate_up;
   }
-  if (tt <= 0) tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
-  if (tt != 1 && tt != 2 && tt != 4) return DMQ_ERR_MODE;
+  // Big batches of fp16 layers (1/2/4-bit pools, group counts multiples of four, single-home
+  // experts): work items of 128 rows for the persistent GEMM launches (tt = 8).  A caller's tt = 8
+  // on another layer falls back to 64-row items.
+  bool rows_ok = (H / DMQ_GS) % 4 == 0 && (I / DMQ_GS) % 4 == 0 && H % 256 == 0 &&
+                 layer->n_widths == 0 &&
+                 (long)tokens * K / DMQ_ROWS_TILE + E <= DMQ_ROWS_MAX_ITEMS &&
+                 ((long)tokens * K + (long)E * DMQ_ROWS_TILE) * 2 * (H > I ? H : I) <= 0xffffffffL;
+  for (int i = 0; i < P; ++i)
+    rows_ok = rows_ok && layer->pool[i].mode == DMQ_MODE_A16 && layer->pool[i].bit != 8;
+  if (tt <= 0) {
+    tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
+    if (rows_ok && (long)tokens * K >= DMQ_ROWS_MIN_ROUTED) tt = DMQ_ROWS_TT;
+  }
+  if (tt == DMQ_ROWS_TT && !rows_ok) tt = 4;
+  if (tt != 1 && tt != 2 && tt != 4 && tt != DMQ_ROWS_TT) return DMQ_ERR_MODE;
   if (ks == 0) {
     ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
     // an 8-bit pool on the fp16 path (a shared expert with a 256-entry table) makes few, long work
@@ -839,9 +882,9 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     ks = 1;
   }
   const int wsplit_eff = sub ? 1 : wsplit;
-  if (!dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
+  if (tt == DMQ_ROWS_TT ? ks != 1 : !dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   const bool nbl_auto = nbl <= 0;
-  if (nbl_auto) nbl = pick_nbl((long)tokens * K, tt);
+  if (nbl_auto) nbl = pick_nbl((long)tokens * K, tt > 4 ? 4 : tt);
   // a rotation wave covers 16 or 32 rows: 64-row work items are rotated by two waves each
   const int rot_tt = tt > 2 ? 2 : tt;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);
@@ -1096,7 +1139,8 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
                                  w.tile_rows, w.max_items, w.counts, w.offsets, w.sorted_tokens,
                                  w.sorted_weights, w.sorted_rows, w.gu_info, w.dn_info, w.n_items,
                                  w.items, w.sort_scratch, w.sort_scratch_bytes, pool_order,
-                                 lead_pools, stream);
+                                 lead_pools, stream, tt == DMQ_ROWS_TT ? w.rows_queue : nullptr,
+                                 2 * DMQ_ROWS_QUEUE_WORDS);
       if (!rc && wsplit_eff > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
     }
   }
@@ -1147,6 +1191,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     g.out = w.act; g.out_stride = I;
     g.post_out = actq_of(mode); g.post_row_bytes = (long)I * 2;
     g.post_scale = actq_scale_of(mode); g.post_scale_stride = scale_stride_for(mode, I);
+    g.rows_queue = w.rows_queue;
     if (wsplit_eff > 1) {
       g.k_split = wsplit_eff; g.split_rows = w.split_rows;
       g.split_partial = w.split_partial; g.split_counter = w.split_counter;
@@ -1201,7 +1246,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     // until the experts are big enough for its 64-row kernel to pay
     const long avg_rows = (long)tokens * K / E;
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
-    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = 16 * tt; d.roomy = roomy;
+    d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = w.tile_rows; d.roomy = roomy;
     d.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
     d.widths_apart = widths_apart;
     d.ks = ks; d.n_pools = P;
@@ -1218,6 +1263,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     d.items = w.items; d.n_items = w.n_items; d.max_items = w.max_items;
     d.out = w.slots; d.out_stride = H;
     d.row_weight = w.sorted_weights; d.row_slot = w.sorted_rows;
+    d.rows_queue = w.rows_queue + DMQ_ROWS_QUEUE_WORDS;
     if (!sub) {
       rc = dmq_matmul_merged_gf(&d, stream);
       if (rc) return rc;

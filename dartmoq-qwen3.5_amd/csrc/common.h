@@ -6,6 +6,13 @@
 
 #define DMQ_GS 128            // quantization group: 128 consecutive input features
 #define DMQ_WAVE 64
+// The persistent GEMM for big batches of fp16 layers (gemm_rows.h), selected by tt == DMQ_ROWS_TT:
+#define DMQ_ROWS_TT 8
+#define DMQ_ROWS_TILE 128                 // rows of a work item
+#define DMQ_ROWS_MAX_ITEMS 2048           // work items a launch can order (it sorts them in LDS)
+#define DMQ_ROWS_MIN_STEPS 8              // group steps per unit its descriptor pipeline needs
+// queue words in device memory: [0, 8) next position of every XCD's queue, [8] workgroups that left
+#define DMQ_ROWS_QUEUE_WORDS 16
 
 // status codes, precision modes and epilogue kinds come from the public C header
 #include "dartmoq_hip.h"

@@ -120,3 +120,6 @@ int dmq_gemm_launch_a16(const GemmLaunch& L);
 int dmq_gemm_launch_a8(const GemmLaunch& L);
 int dmq_gemm_launch_fp8(const GemmLaunch& L);
 int dmq_gemm_launch_fp4(const GemmLaunch& L);
+// persistent launch over work items of 128 rows, fp16 pools of 1/2/4-bit indices (gemm_rows.h);
+// nbl: feature blocks per unit; queue: DMQ_ROWS_QUEUE_WORDS zeroed device words
+int dmq_gemm_rows_launch(const GemmParams& p, int epi, int* queue, int nbl, hipStream_t stream);

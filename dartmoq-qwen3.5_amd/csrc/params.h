@@ -109,6 +109,10 @@ struct PlanParams {
   // their items are a prefix of the list); lead_pools < 0 leaves n_items[1] alone.
   int pool_order[DMQ_MAX_POOLS];
   int lead_pools;
+  // up to 1024 int32 words the planning step sets to zero (the queue words of the persistent GEMM
+  // launches that follow); zero_count == 0: none
+  int* zero_words;
+  int zero_count;
 };
 
 // One-workgroup routing for small batches: top-k (or a copy of the caller's top-k), the shared

@@ -151,6 +151,7 @@ __device__ __forceinline__ void plan_emit_items(const PlanParams& p, const int* 
                                                 int* carry_p, const PlanSlices& pre_s,
                                                 int* item_first = nullptr, int* item_ss = nullptr) {
   const int tid = threadIdx.x;
+  if (tid < p.zero_count) p.zero_words[tid] = 0;           // words later launches want cleared
   const bool pre = p.experts <= 1024;
   if (pre && p.max_items < 65536) {
     const bool tile_pow2 = (p.tile_rows & (p.tile_rows - 1)) == 0;

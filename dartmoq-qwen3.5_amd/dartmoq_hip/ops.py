@@ -16,6 +16,7 @@ from ._lib import (EPI_SILU_ROT,  # noqa: F401
                    check, load)
 
 GROUP_SIZE = 128
+ROWS_TT = 8          # tt value of the persistent launch over 128-row work items (fp16 layers)
 ITEM_WORDS = 8          # int32 words of a work-item record (DMQ_ITEM_WORDS)
 
 
@@ -357,6 +358,9 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.mode2_on = 0 if mode2 is None else 1
     a.mode2 = 0 if mode2 is None else int(mode2)
     a.widths_apart = int(widths_apart)
+    if tt == ROWS_TT:       # the persistent launch over 128-row work items: its queue words start at zero
+        rows_queue = torch.zeros(16, dtype=torch.int32, device=dev)
+        a.rows_queue = rows_queue.data_ptr()
     if k_split > 1:
         if rows_total is None:
             raise ValueError("k_split needs rows_total")

@@ -221,7 +221,7 @@ typedef struct {
 typedef struct {
   int mode;                 /* DMQ_MODE_* */
   int epi;                  /* DMQ_EPI_* */
-  int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4 */
+  int tt;                   /* activation tiles of 16 rows per wave: 1, 2 or 4; 8: see rows_queue */
   int ks;                   /* waves of a workgroup splitting K: 0 = 1; 4 or 1 for tt == 1, else 1 */
   int nbl;                  /* blocks of output features one workgroup walks back to back (its
                                loads stay in flight across blocks): 0 = 1; used when ks == 1 */
@@ -310,6 +310,15 @@ typedef struct {
    * three workgroups per CU, which wins once the list holds more than about a hundred work
    * items).  Same results. */
   int widths_apart;
+  /* tt == 8: the launch for big batches of fp16 layers (DMQ_MODE_A16, 1/2/4-bit pools only): work
+   * items of 128 rows (items built with tile_rows == 128; item_tile_rows 0 or 128), one persistent
+   * workgroup per CU that dequantizes a weight tile once per stretch of up to 128 rows and draws its
+   * units from per-XCD queues, longest first.  groups % 4 == 0; n_out a multiple of 128 (SiLU
+   * epilogues) or 256; max_items <= 2048; not with ks > 1, k_split, nt == 1, dbg_acc, mode2,
+   * width_filter or accumulate; other pools' items are skipped.  rows_queue: 16 int32 words of
+   * device memory, zero before the launch; the launch leaves them zero.  Same results, bit for bit,
+   * as tt == 2 and tt == 4. */
+  void* rows_queue;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

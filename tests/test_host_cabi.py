@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/dartmoq_hip.h but not exported"
     assert set(declared) == set(_lib.PROTOTYPES), "ctypes prototypes and header disagree"
-    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 18
+    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 19
     assert lib.dmq_status_string(0) == b"ok"
     assert b"bit width" in lib.dmq_status_string(1)
 
@@ -255,3 +255,33 @@ def test_k_sharing_argument_validation():
     a.nt, a.ks = 0, 0
     a.epi, a.k_split, a.groups, a.act_row_bytes = _lib.EPI_SILU, 4, 6, 2048
     assert lib.dmq_matmul_merged_gf(ctypes.byref(a), None) == 2           # 6 groups, 4 workgroups
+
+
+def test_ctypes_structs_match_the_header_layout(tmp_path):
+    """Size and the offset of the last field of every argument struct, as gcc lays the header out,
+    against the ctypes mirror: a field missing on one side shifts everything behind it (and ctypes
+    accepts an assignment to a field it does not know without a word)."""
+    import ctypes
+    import shutil
+    import subprocess
+    from dartmoq_hip import _lib
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    pairs = [("dmq_gemm_pool", _lib.GemmPool), ("dmq_gemm_args", _lib.GemmArgs),
+             ("dmq_pool_desc", _lib.PoolDesc), ("dmq_linear_desc", _lib.LinearDesc),
+             ("dmq_layer_desc", _lib.LayerDesc), ("dmq_router_args", _lib.RouterArgs)]
+    lines = ['#include "dartmoq_hip.h"', "#include <stdio.h>", "#include <stddef.h>", "int main(void) {"]
+    for cname, cls in pairs:
+        last = cls._fields_[-1][0]
+        lines.append(f'  printf("%zu %zu\\n", sizeof({cname}), offsetof({cname}, {last}));')
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.dirname(HEADER), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    for (cname, cls), line in zip(pairs, out):
+        size, off = (int(v) for v in line.split())
+        last = cls._fields_[-1][0]
+        assert ctypes.sizeof(cls) == size, f"{cname}: ctypes {ctypes.sizeof(cls)} bytes, header {size}"
+        assert getattr(cls, last).offset == off, f"{cname}.{last}: ctypes offset differs from the header"

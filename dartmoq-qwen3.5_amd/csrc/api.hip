@@ -43,8 +43,10 @@ static inline int pick_ks(int tt, long rows, int groups) {
 #define DMQ_TT4_MIN_AVG 112
 #define DMQ_HOIST_ALL_TOKENS 1024
 #define DMQ_TAIL_SLOTS 96
-// routed rows from which an fp16 layer is cut into work items of 128 rows (the persistent GEMM)
-#define DMQ_ROWS_MIN_ROUTED 8192
+// routed rows from which an fp16 layer is cut into work items of 128 rows (the persistent GEMM).
+// Not chosen automatically at present: at 16384 routed rows (H = 2048, I = 512, Zipf routing) the
+// launch pair measures slower than the 32-row launches; tt = 8 asks for it explicitly.
+#define DMQ_ROWS_MIN_ROUTED (1L << 40)
 
 // Feature blocks one workgroup walks back to back.  With few row tiles every block gets its own
 // workgroup (parallelism); with many, a workgroup amortizes its start-up over several blocks.

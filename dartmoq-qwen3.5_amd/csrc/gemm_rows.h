@@ -19,9 +19,11 @@
 //     so the short units of the ragged ends fill the gaps the long ones leave.
 //   * A wave with the SIMD to itself hides no latency by occupancy, so everything is software
 //     pipelined: packed weights and norms travel three groups ahead in a register ring, the
-//     activation tile of a group is staged in one of three LDS buffers two groups ahead, and inside
-//     a group the look-ups, scaled operands and activation operands of the next micro-step
-//     (MFMA step s, n-tile j) are produced between the MFMAs of the current one.
+//     activation tile of a group goes from memory straight into one of three LDS buffers two
+//     groups ahead (global_load_lds_dwordx4: no registers, no LDS store instructions, and nothing
+//     waits for it until the barrier in front of the group that reads it), and inside a group the
+//     scaled operands and look-ups of the following MFMA steps and the activation operands of the
+//     following micro-steps (MFMA step s, row tile t) are produced between the MFMAs.
 //   * The pipeline does not drain between units: while a unit runs, the workgroup draws the next
 //     one from the queue (one atomic), reads its record and row indices, and directs the loads of
 //     its last three groups at the next unit's first three.  Only a change of tile class or pool
@@ -133,8 +135,13 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
   constexpr int FPB = SILU ? 128 : 256;                  // output features per block
   constexpr int CPT = TT;                                // 16-byte chunks a thread stages per group
 
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // The kernel holds nine instances of this body in one loop.  The thread index goes through an
+  // empty asm so that the lane constants below are computed here, per call: hoisted out of that
+  // loop, the constants of all nine instances would be live at once and spill.
+  int tidv = threadIdx.x;
+  asm volatile("" : "+v"(tidv));
+  const int lane = tidv & 63;
+  const int wave = tidv >> 6;
   const int l16 = lane & 15;
   const int q = lane >> 4;
   const uint32_t lane_base = dmq_lut_lane_base<BIT, 2>(lane);
@@ -159,12 +166,11 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
   // contiguous bytes of the row's group); a thread stages chunk lane % 16 of rows
   // wave*4*TT + 4c + lane / 16.  Rows past the expert's last row stage a copy of that last row:
   // every load is unconditional and nothing computed from such a row is ever stored.
-  uint32_t a_dst[CPT];
-#pragma unroll
-  for (int c = 0; c < CPT; ++c) {
-    const int srow = wave * (4 * TT) + c * 4 + q;
-    a_dst[c] = (uint32_t)(srow * AB + ((l16 ^ (srow & 15)) * 16));
-  }
+  // The load writes LDS lane by lane (lane L of load c: byte 16 L of the four rows), so the
+  // swizzle is applied on the memory side: position lane % 16 of row r holds chunk
+  // (lane % 16) ^ (r % 16) of that row, and that is the chunk the lane requests.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const uint32_t stage_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)stage;
   // operand reads: row 16 t + l16, chunk (4 q + s) ^ l16
   uint32_t b_off[4];
 #pragma unroll
@@ -174,8 +180,8 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
   const uint8_t* Lw;
   const uint8_t* Ln;
   uint32_t a_lane[CPT];
-  int lk = 0, lg = 0;                                    // weights: step + 3
-  int ak = 0, ag = 0;                                    // activations: step + 2
+  int lk = 0, lg = 0;                                    // weights: feature block and group of step + 3
+  int ak = 0, ag = 0;                                    // activations: the same for step + 2
   int l_state = 0;                                       // 1: the weight loads are in the next unit, 2: held at the last step
   int a_frozen = 0;
   auto set_bases = [&](const RowsUnit& u) {
@@ -185,16 +191,23 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     Ln = (const uint8_t*)pw.norms + (g_base * pw.n_total + row0) * 2;
   };
   auto stage_rows = [&](const RowsUnit& u, int (&ri)[CPT]) {
+    // (the first row goes through an empty asm: the per-chunk row numbers are cheap to recompute and
+    // would otherwise be kept, and spilled, across the whole call)
+    int row0 = wave * (4 * TT) + q;
+    asm volatile("" : "+v"(row0));
+    const int* const rix = pw.row_index;
+    if (rix) {
 #pragma unroll
-    for (int c = 0; c < CPT; ++c) {
-      const int srow = wave * (4 * TT) + c * 4 + q;
-      const int s_rlog = min(u.r_first + srow, u.r_end - 1);
-      ri[c] = pw.row_index ? pw.row_index[s_rlog] : s_rlog;
+      for (int c = 0; c < CPT; ++c) ri[c] = rix[min(u.r_first + row0 + c * 4, u.r_end - 1)];
+    } else {
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) ri[c] = min(u.r_first + row0 + c * 4, u.r_end - 1);
     }
   };
   auto lanes_from_rows = [&](const int (&ri)[CPT], uint32_t (&al)[CPT]) {
 #pragma unroll
-    for (int c = 0; c < CPT; ++c) al[c] = (uint32_t)ri[c] * (uint32_t)p.act_row_bytes + l16 * 16;
+    for (int c = 0; c < CPT; ++c)
+      al[c] = (uint32_t)ri[c] * (uint32_t)p.act_row_bytes + (uint32_t)((l16 ^ ((wave * (4 * TT) + c * 4 + q) & 15)) * 16);
   };
 
   float4_t acc[NT][TT];
@@ -205,7 +218,6 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
 
   uint32_t pk[4][NT][WW];            // packed weights of four consecutive group steps
   uint32_t nh[4][NT];                // norm of the lane's weight row
-  uint4_t ar[CPT];                   // activation chunks on their way to LDS
   uint32_t raw[NT][4];               // looked-up operand words on their way to being scaled (one MFMA step)
   uint4_t aop[2][NT];                // scaled weight operands of the current / next MFMA step
   uint4_t bf[4];                     // activation operands, three micro-steps ahead of their MFMAs
@@ -221,8 +233,18 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     dmq_load_words<WW>(wb + lane_off(w_lane[j]), d);
     n = *(const uint16_t*)(nb + lane_off(n_lane[j]));
   };
-  auto load_a = [&](int c) -> uint4_t {
-    return *(const uint4_t*)(act_p + (long)ag * AB + lane_off(a_lane[c]));
+  // chunk c of the activation tile of the activation-side position, straight into LDS buffer buf_off
+  auto load_a = [&](int c, uint32_t buf_off) {
+    const uint32_t m0v = stage_lds + buf_off + (uint32_t)((wave_u * (4 * TT) + c * 4) * AB);
+    const uint8_t* src = act_p + (long)ag * AB;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(m0v), "v"(a_lane[c]), "s"(src) : "m0");
+  };
+  // every vector memory operation issued before the last `younger` ones has completed
+  auto wait_loads = [](auto nc) {
+    constexpr int younger = decltype(nc)::value;
+    static_assert(younger >= 0 && younger < 64, "6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(younger) : "memory");
   };
   auto look = [&](auto sc_, const uint32_t (&pkj)[WW], uint32_t (&w)[4]) {
     constexpr int s = decltype(sc_)::value;
@@ -272,7 +294,9 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     } else {
       if (DMQ_UNI(nxt.valid && nxt.cls == my_cls && nxt.pool == my_pool)) {
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) nxt_ri[c] = (int)((uint32_t)nxt_ri[c] * (uint32_t)p.act_row_bytes + l16 * 16);
+        for (int c = 0; c < CPT; ++c)
+          nxt_ri[c] = (int)((uint32_t)nxt_ri[c] * (uint32_t)p.act_row_bytes +
+                            (uint32_t)((l16 ^ ((wave * (4 * TT) + c * 4 + q) & 15)) * 16));
         nxt_ready = 1;
       }
     }
@@ -310,8 +334,7 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     }
   };
 
-  // ---- empty pipeline: table, steps 0..2 of the weights, activation tiles 0 and 1 in LDS, tile 2
-  // on its way
+  // ---- empty pipeline: table, steps 0..2 of the weights, activation tiles 0 and 1 in LDS
   {
     int ri[CPT];
     stage_rows(cur, ri);
@@ -320,14 +343,13 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     const bool build = __builtin_amdgcn_readfirstlane(lut_pool) != cur.pool;
     if (build) dmq_lut_fetch<BIT, 2>(pw.lut, threadIdx.x, lutw);
     lanes_from_rows(ri, a_lane);
-    uint4_t a1[CPT];
 #pragma unroll
-    for (int c = 0; c < CPT; ++c) ar[c] = load_a(c);
+    for (int c = 0; c < CPT; ++c) load_a(c, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) load_w(j, pk[0][j], nh[0][j]);
     lg = 1; ag = 1;
 #pragma unroll
-    for (int c = 0; c < CPT; ++c) a1[c] = load_a(c);
+    for (int c = 0; c < CPT; ++c) load_a(c, SLOT);
 #pragma unroll
     for (int j = 0; j < NT; ++j) load_w(j, pk[1][j], nh[1][j]);
     lg = 2; ag = 2;
@@ -339,10 +361,7 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
       dmq_lut_store_wave<BIT, 2>(tbl, wave, lutw);
       lut_pool = cur.pool;
     }
-#pragma unroll
-    for (int c = 0; c < CPT; ++c) *(uint4_t*)(stage + a_dst[c]) = ar[c];
-#pragma unroll
-    for (int c = 0; c < CPT; ++c) *(uint4_t*)(stage + SLOT + a_dst[c]) = a1[c];
+    wait_loads(std::integral_constant<int, 0>{});        // both tiles have landed
     __syncthreads();
   }
   uint32_t cur_off = 0, nxt_off = SLOT, wr_off = 2 * SLOT;
@@ -529,8 +548,8 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
         else look(std::integral_constant<int, (s + 2) & 3>{}, pk[(GI + 1) & 3][j], raw[j]);
         if constexpr (s == 1) load_w(j, pk[(GI + 3) & 3][j], nh[(GI + 3) & 3][j]);   // three steps ahead
       }
-      if constexpr (s == 0) ar[t] = load_a(t);                                     // tile of step st + 2
-      if constexpr (s == 3) *(uint4_t*)(stage + wr_off + a_dst[t]) = ar[t];        // ... into its buffer
+      // the activation tile of step st + 2, into the buffer that the previous step has released
+      if constexpr (s == 0) load_a(t, wr_off);
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
@@ -554,13 +573,24 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
         micro(sc_, std::integral_constant<int, 7>{});
       }
     };
+    // The last three micro-steps of this step already read operands of the next step's tile, so
+    // that tile is published inside the step (in front of MFMA step 3; with two row tiles MFMA
+    // step 2 holds one of those micro-steps, so in front of that), not at its end: it was requested
+    // at the head of the previous step, and since then this wave has issued 8 weight loads, the TT
+    // loads of the tile after it and 8 more weight loads.
+    auto publish_next_tile = [&]() {
+      wait_loads(std::integral_constant<int, 16 + TT>{});
+      __syncthreads();
+    };
     mfma_step(std::integral_constant<int, 0>{});
     mfma_step(std::integral_constant<int, 1>{});
+    if constexpr (TT < 3) publish_next_tile();
     mfma_step(std::integral_constant<int, 2>{});
+    if constexpr (TT >= 3) publish_next_tile();
     mfma_step(std::integral_constant<int, 3>{});
     advance_load();
     advance_act();
-    __syncthreads();
+    __syncthreads();                          // every wave is done with this step's tile: its buffer is free
     const uint32_t o = cur_off; cur_off = nxt_off; nxt_off = wr_off; wr_off = o;
   };
 
@@ -580,6 +610,9 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     kb = cur.kb0;
     l_state = 0;
   }
+  // tile loads of the last steps are still on their way to LDS buffers that the next call lays
+  // out differently
+  wait_loads(std::integral_constant<int, 0>{});
   // the unit after this call: the one already drawn (another class or pool), or a fresh draw
   if (DMQ_UNI(nxt.valid)) cur_io = nxt;
   else sc.fetch_sync(cur_io);
@@ -602,21 +635,34 @@ __global__ __launch_bounds__(256) void dmq_gemm_rows_kernel(GemmParams p, int* q
   const int n_items = min(p.n_items[0], DMQ_ROWS_MAX_ITEMS);
   const int ipt = (n_items + 255) >> 8;                  // items per thread, contiguous
   constexpr int IPT_MAX = DMQ_ROWS_MAX_ITEMS / 256;
+  // which pools this launch serves (fp16 activations, 1/2/4-bit indices), one bit per pool
+  unsigned elig = 0;
+#pragma unroll
+  for (int q = 0; q < DMQ_MAX_POOLS; ++q)
+    elig |= (p.pool[q].mode == DMQ_MODE_A16 && p.pool[q].bit != 8) ? 1u << q : 0u;
+  // all records are requested before any is looked at (positions past the list repeat its last
+  // record: the loads are unconditional)
+  int rpool[IPT_MAX], rtile[IPT_MAX], rcount[IPT_MAX];
+#pragma unroll
+  for (int k = 0; k < IPT_MAX; ++k) {
+    rpool[k] = 0; rtile[k] = 0; rcount[k] = 0;
+    if (k < ipt) {                                       // uniform
+      const int i = max(min(tid * ipt + k, n_items - 1), 0);
+      const int4_t r0 = *(const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * i);
+      rpool[k] = r0[0]; rtile[k] = r0[2];
+      rcount[k] = p.items[(long)DMQ_ITEM_WORDS * i + 4];
+    }
+  }
   int cls[IPT_MAX];
   unsigned long long cnt = 0;                            // three 16-bit counters
 #pragma unroll
   for (int k = 0; k < IPT_MAX; ++k) {
     cls[k] = 3;
     const int i = tid * ipt + k;
-    if (k < ipt && i < n_items) {
-      const int4_t r0 = *(const int4_t*)(p.items + (long)DMQ_ITEM_WORDS * i);
-      const int tc = p.items[(long)DMQ_ITEM_WORDS * i + 4];
-      const int rows = tc - r0[2] * DMQ_ROWS_TILE;
-      const PoolW& pw = p.pool[r0[0] & (DMQ_MAX_POOLS - 1)];
-      if (rows > 0 && pw.mode == DMQ_MODE_A16 && pw.bit != 8) {
-        cls[k] = rows > 64 ? 0 : (rows > 32 ? 1 : 2);
-        cnt += 1ull << (16 * cls[k]);
-      }
+    const int rows = rcount[k] - rtile[k] * DMQ_ROWS_TILE;
+    if (k < ipt && i < n_items && rows > 0 && ((elig >> (rpool[k] & (DMQ_MAX_POOLS - 1))) & 1u)) {
+      cls[k] = rows > 64 ? 0 : (rows > 32 ? 1 : 2);
+      cnt += 1ull << (16 * cls[k]);
     }
   }
   unsigned long long incl = cnt;

@@ -155,3 +155,62 @@ def test_rows_argument_errors():
     with pytest.raises(ValueError):            # a block of the plain-store epilogue is 256 features
         ops.matmul_merged(A16, 2, STORE, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info,
                           groups=4, n_out=128, slice_is_groups=False, rows_total=16, tt=ROWS_TT)
+
+
+@pytest.mark.parametrize("epi", ["store", "silu_rot", "scatter"])
+def test_rows_many_units_keep_the_pipeline_full(epi):
+    """Several hundred work items of every tile class, so that workgroups run many units one after
+    the other (loads of a unit's last steps go to the next unit, units drawn from the queues while
+    the previous one runs, other workgroups' queues emptied at the end): bits of the 32-row kernel."""
+    from dartmoq_hip import ops
+    from dartmoq_hip._lib import EPI_SILU_ROT
+    bit = 2
+    g = torch.Generator().manual_seed(91)
+    n_exp = 300
+    counts = torch.randint(0, 260, (n_exp,), generator=g).tolist()
+    counts[7] = 1500                                     # one expert with many full stretches
+    starts, rows_total = _starts(counts)
+    if epi == "scatter":                                 # down shape: slices in groups, K = 512, 1024 features out
+        k, hidden = 512, 1024
+        didx, dnorms, dcb = _pool(bit, hidden, k * n_exp, 41)
+        dinfo = torch.tensor([(starts[e], counts[e], e * (k // 128), k // 128) for e in range(n_exp)],
+                             dtype=torch.int32).cuda()
+        a = (torch.randn(rows_total, k, generator=g) * 0.5).half().cuda()
+        slot = torch.randperm(rows_total, generator=g).int().cuda()
+        wts = torch.rand(rows_total, generator=g).cuda()
+        outs = []
+        for tt in (2, ROWS_TT):
+            slots = torch.full((rows_total, hidden), float("nan"), dtype=torch.float16, device="cuda")
+            ops.matmul_merged(A16, bit, SCATTER, a, None, didx.cuda(), dnorms.cuda(), dcb.cuda(), dinfo,
+                              groups=k // 128, n_out=hidden, slice_is_groups=True, rows_total=rows_total,
+                              out=slots, out_stride=hidden, row_weight=wts, row_slot=slot, tt=tt)
+            torch.cuda.synchronize()
+            outs.append(slots.cpu())
+        assert not torch.isnan(outs[0].float()).any()
+        assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+        return
+    k, inter = 1024, 256
+    n_rows = (inter if epi == "store" else 2 * inter) * n_exp
+    idx_gf, norms_gf, cb = _pool(bit, n_rows, k, 43)
+    x = (torch.randn(rows_total, k, generator=g) * 0.5).half().cuda()
+    width = n_rows // n_exp
+    info = torch.tensor([(starts[e], counts[e], e * width, width) for e in range(n_exp)],
+                        dtype=torch.int32).cuda()
+    tens = (x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info)
+    outs = []
+    for tt in (2, ROWS_TT):
+        if epi == "store":
+            out = ops.matmul_merged(A16, bit, STORE, *tens, groups=k // 128, n_out=inter,
+                                    slice_is_groups=False, rows_total=rows_total, tt=tt)
+        else:
+            rot = (torch.randn(n_exp * inter // 128, 128, 128, generator=torch.Generator().manual_seed(5))
+                   / 128 ** 0.5).half().cuda()
+            out = torch.full((rows_total, inter), float("nan"), dtype=torch.float16, device="cuda")
+            dummy = torch.empty((rows_total, inter), dtype=torch.float16, device="cuda")
+            ops.matmul_merged(A16, bit, EPI_SILU_ROT, *tens, groups=k // 128, n_out=inter, half_width=inter,
+                              slice_is_groups=False, rows_total=rows_total, tt=tt, out=dummy,
+                              out_stride=inter, post=dict(rot=[rot], extra=[1.0], out=out, scale=None))
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    assert not torch.isnan(outs[0].float()).any()
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))

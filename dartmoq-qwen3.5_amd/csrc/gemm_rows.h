@@ -123,7 +123,7 @@ struct RowsSched {
 
 template <int BIT, int TT, int EPI>
 __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc, RowsUnit& cur_io,
-                                              int& lut_pool, uint8_t* tbl, uint8_t* stage) {
+                                              int& lut_key, uint8_t* lds) {
   RowsUnit cur = cur_io.uniform();
   constexpr int MODE = DMQ_MODE_A16;
   constexpr int NT = 4;
@@ -134,6 +134,12 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
   constexpr bool SILU = (EPI == DMQ_EPI_SILU || EPI == DMQ_EPI_SILU_ROT);
   constexpr int FPB = SILU ? 128 : 256;                  // output features per block
   constexpr int CPT = TT;                                // 16-byte chunks a thread stages per group
+  constexpr int DMA_STEP = (TT < 3) ? 2 : 3;             // MFMA step behind the barrier of a group step
+  // Table rows of 256 bytes (the address of a look-up is one byte permute) where the three
+  // activation buffers leave the room: up to 64 rows.  128-row units keep 128-byte rows.
+  constexpr int ROW = (TT <= 4) ? 256 : DMQ_LUT_ROW;
+  uint8_t* const tbl = lds;
+  uint8_t* const stage = lds + 256 * ROW;
 
   // The kernel holds nine instances of this body in one loop.  The thread index goes through an
   // empty asm so that the lane constants below are computed here, per call: hoisted out of that
@@ -144,7 +150,7 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
   const int wave = tidv >> 6;
   const int l16 = lane & 15;
   const int q = lane >> 4;
-  const uint32_t lane_base = dmq_lut_lane_base<BIT, 2>(lane);
+  const uint32_t lane_base = dmq_lut_lane_base<BIT, 2, ROW>(lane);
   // every unit of this call is of this pool and class (both the same for every lane)
   const int my_pool = __builtin_amdgcn_readfirstlane(cur.pool), my_cls = __builtin_amdgcn_readfirstlane(cur.cls);
   const PoolW& pw = p.pool[my_pool];
@@ -248,7 +254,7 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
   };
   auto look = [&](auto sc_, const uint32_t (&pkj)[WW], uint32_t (&w)[4]) {
     constexpr int s = decltype(sc_)::value;
-    dmq_dequant_step<MODE, BIT, s>(tbl, lane_base, pkj, w);
+    dmq_dequant_step<MODE, BIT, s, false, ROW>(tbl, lane_base, pkj, w);
   };
   auto read_b = [&](uint32_t buf_off, int s, int t) -> uint4_t {
     return *(const uint4_t*)(stage + buf_off + b_off[s] + t * (16 * AB));
@@ -340,7 +346,8 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     stage_rows(cur, ri);
     set_bases(cur);
     uint32_t lutw[4];
-    const bool build = __builtin_amdgcn_readfirstlane(lut_pool) != cur.pool;
+    const int my_key = cur.pool * 2 + (ROW == 256 ? 1 : 0);   // the table in LDS: pool and row size
+    const bool build = __builtin_amdgcn_readfirstlane(lut_key) != my_key;
     if (build) dmq_lut_fetch<BIT, 2>(pw.lut, threadIdx.x, lutw);
     lanes_from_rows(ri, a_lane);
 #pragma unroll
@@ -358,8 +365,8 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     lg = 3;
     if (build) {
       __syncthreads();                                   // nobody reads the old table any more
-      dmq_lut_store_wave<BIT, 2>(tbl, wave, lutw);
-      lut_pool = cur.pool;
+      dmq_lut_store_wave<BIT, 2, ROW>(tbl, wave, lutw);
+      lut_key = my_key;
     }
     wait_loads(std::integral_constant<int, 0>{});        // both tiles have landed
     __syncthreads();
@@ -440,16 +447,16 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
       }
     } else {
       // SiLU * up rows of the block (one group of the down projection) -> rotation of that group by
-      // the expert's matrix -> fp16 rows.  The tile meets in the LDS buffer that the finished step
-      // has consumed (every wave is past this step's barrier), every wave rotates it onto 32 of the
-      // 128 outputs with its quarter of the matrix: the arithmetic of the stand-alone rotation
-      // kernel, in its order.  The buffer is written again in the next step: a barrier ends the
-      // epilogue.
+      // the expert's matrix -> fp16 rows.  The tile meets in the LDS buffer of the finished step
+      // (once every wave is done reading it: a barrier), every wave rotates it onto 32 of the 128
+      // outputs with its quarter of the matrix: the arithmetic of the stand-alone rotation kernel,
+      // in its order.  The buffer is next written behind the following step's barrier.
       constexpr int PITCH = 256;
       const int blk = kb * FPB;
       uint8_t* tile = stage + wr_off;
       const __half* prot = pw.post_rot + (long)(cur.post_slice + blk / DMQ_GS) * (DMQ_GS * DMQ_GS) +
                            (long)(32 * wave + l16) * DMQ_GS + 8 * q;
+      __syncthreads();
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
         const int row = t * 16 + l16;
@@ -492,7 +499,6 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
           *(half4_t*)(orow + (col0 + 16 * jt) * 2) = h;
         }
       }
-      __syncthreads();
     }
 #pragma unroll
     for (int j = 0; j < NT; ++j)
@@ -548,17 +554,14 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
         else look(std::integral_constant<int, (s + 2) & 3>{}, pk[(GI + 1) & 3][j], raw[j]);
         if constexpr (s == 1) load_w(j, pk[(GI + 3) & 3][j], nh[(GI + 3) & 3][j]);   // three steps ahead
       }
-      // the activation tile of step st + 2, into the buffer that the previous step has released
-      if constexpr (s == 0) load_a(t, wr_off);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, TT >= 8 ? 2 : (TT == 4 ? 3 : 6), 0);   // VALU
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                          // one LDS read
-        if (j == 3) __builtin_amdgcn_sched_group_barrier(0x220, 1, 0);              // memory / LDS write
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      // the activation tile of step st + 2, into the buffer the previous step has read: requested
+      // behind the barrier of this step, which every wave passes only when it is done with that one
+      if constexpr (s == DMA_STEP) load_a(t, wr_off);
     };
+    // The issue order inside an MFMA step: a wave alone on its SIMD issues at most one instruction
+    // every four cycles and an MFMA keeps the matrix pipe for sixteen, so up to three other
+    // instructions fit behind each MFMA for free, and none of this step's other work depends on
+    // this step's MFMAs: one MFMA, then up to three vector / scalar / LDS / memory instructions.
     auto mfma_step = [&](auto sc_) {
       micro(sc_, std::integral_constant<int, 0>{});
       micro(sc_, std::integral_constant<int, 1>{});
@@ -572,14 +575,22 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
         micro(sc_, std::integral_constant<int, 6>{});
         micro(sc_, std::integral_constant<int, 7>{});
       }
+#pragma unroll
+      for (int i = 0; i < 4 * TT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x326, TT >= 8 ? 3 : (TT == 4 ? 5 : 10), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     };
-    // The last three micro-steps of this step already read operands of the next step's tile, so
-    // that tile is published inside the step (in front of MFMA step 3; with two row tiles MFMA
-    // step 2 holds one of those micro-steps, so in front of that), not at its end: it was requested
-    // at the head of the previous step, and since then this wave has issued 8 weight loads, the TT
-    // loads of the tile after it and 8 more weight loads.
+    // One barrier per step.  The last three micro-steps of a step already read operands of the
+    // next step's tile, so the barrier stands inside the step: in front of MFMA step 3 (with two
+    // row tiles MFMA step 2 holds one of those micro-steps: in front of that).  It publishes the
+    // next step's tile, requested behind the previous step's barrier (since then this wave has
+    // issued the 8 weight loads of this step, in MFMA step 1, and nothing else), and a wave that
+    // has passed it knows every wave done with the previous step, whose buffer takes the tile after
+    // next.
     auto publish_next_tile = [&]() {
-      wait_loads(std::integral_constant<int, 16 + TT>{});
+      wait_loads(std::integral_constant<int, 8>{});
       __syncthreads();
     };
     mfma_step(std::integral_constant<int, 0>{});
@@ -590,7 +601,6 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
     mfma_step(std::integral_constant<int, 3>{});
     advance_load();
     advance_act();
-    __syncthreads();                          // every wave is done with this step's tile: its buffer is free
     const uint32_t o = cur_off; cur_off = nxt_off; nxt_off = wr_off; wr_off = o;
   };
 
@@ -623,8 +633,7 @@ __device__ __forceinline__ void dmq_rows_body(const GemmParams& p, RowsSched& sc
 template <int EPI>
 __global__ __launch_bounds__(256) void dmq_gemm_rows_kernel(GemmParams p, int* queue, int nbl) {
   extern __shared__ __attribute__((aligned(16))) uint8_t dmq_rows_lds[];
-  uint8_t* tbl = dmq_rows_lds;
-  uint8_t* stage = dmq_rows_lds + DMQ_LUT_BYTES;
+  uint8_t* stage = dmq_rows_lds + DMQ_LUT_BYTES;         // scratch of the sort below
   uint16_t* order = (uint16_t*)(dmq_rows_lds + DMQ_ROWS_ORDER_OFF);
   int* mail = (int*)(dmq_rows_lds + DMQ_ROWS_MAIL_OFF);
   const int tid = threadIdx.x;
@@ -718,10 +727,10 @@ __global__ __launch_bounds__(256) void dmq_gemm_rows_kernel(GemmParams p, int* q
       sc.fetch_sync(cur);
     }
   }
-  int lut_pool = -1;
+  int lut_key = -1;
   while (cur.valid) {
     const int bit = p.pool[cur.pool].bit;
-#define DMQ_ROWS_CALL(BIT, TT) dmq_rows_body<BIT, TT, EPI>(p, sc, cur, lut_pool, tbl, stage)
+#define DMQ_ROWS_CALL(BIT, TT) dmq_rows_body<BIT, TT, EPI>(p, sc, cur, lut_key, dmq_rows_lds)
 #define DMQ_ROWS_BIT(TT) \
     if (bit == 1) DMQ_ROWS_CALL(1, TT); else if (bit == 2) DMQ_ROWS_CALL(2, TT); else DMQ_ROWS_CALL(4, TT);
     if (cur.cls == 0) { DMQ_ROWS_BIT(8) }

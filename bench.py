@@ -8,7 +8,10 @@ dequant-GEMM + SiLU*up, per-expert rotation, down dequant-GEMM + scatter-add, fp
 one batch of synthetic tokens of BASELINE configs[1]: H=2048, 256 experts, top-8, I=512, WxA16
 with mixed bit pools at ~2 bpw and Zipf(1.1)-skewed routing.  Inputs are resident in HBM when
 the timed region starts.  The 2 bpw layer (~216 MB packed) fits in the 256 MB Infinity Cache, so
-the steps rotate through three independent copies of the layer.
+the steps rotate through three independent copies of the layer; a small batch touches few
+experts, so its steps also cycle through router logits with the expert axis rolled until the
+distinct weights of one cycle exceed twice that cache (`weight_copies_rotated`, `logit_variants`,
+`cycle_weight_bytes` of every entry).
 
 Defaults: 50 untimed warm-up steps and 500 timed ones (about 0.15 s of GPU work).  The GPU takes
 tens of milliseconds of sustained load to reach its working clocks, so every measurement starts
@@ -19,9 +22,11 @@ short and long runs then read the same time per step.
 WxA8, configs[4] WxFP8 and WxFP4; the all-4-bit layer, uniform routing) at 2048 and 64 tokens, each
 with the roofline of its gate_up launch; `sweep` the decode sizes of the main configuration.
 
-Prints ONE JSON line.  `roofline` describes the dominant kernel (the gate_up dequant-GEMM of the
-largest bit pool, which also rotates its output rows for the down projection), timed live with
-events on the stream it runs on; `cpu_baseline` is the CPU
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the merged gate_up dequant-GEMM),
+timed live with events on the stream it runs on, on its algorithmic bytes and flops: packed
+indices, norms and activation rows; the down-projection rotation the same launch performs is
+listed beside them as `extra_bytes` / `extra_flops`.  `roofline_down` is the same for the down
+dequant-GEMM.  `cpu_baseline` is the CPU
 oracle (dequantize-then-matmul, fp32) timed on the host cores on a bounded sample.
 """
 
@@ -61,6 +66,8 @@ def layer_bytes(mod, counts):
 
 
 PRELUDE_S = 0.5
+MALL_BYTES = 256 << 20     # Infinity Cache of the MI355X
+MAX_LOGIT_VARIANTS = 256
 
 
 def settle_clocks(mods, x, logits, seconds):
@@ -68,103 +75,169 @@ def settle_clocks(mods, x, logits, seconds):
     sustained work to reach its working clocks (and drops them again while the host is busy), so
     without it a 20-step run reads 15 % slower than a 500-step run of the same thing."""
     import torch
-    n = len(mods)
+    n, v = len(mods), len(logits)
     t0 = time.perf_counter()
     s = 0
     while time.perf_counter() - t0 < seconds:
         for _ in range(20):
-            mods[s % n].forward(x, router_logits=logits)
+            mods[s % n].forward(x, router_logits=logits[s % v])
             s += 1
         torch.cuda.synchronize()
     return time.perf_counter() - t0
 
 
 def time_steps(mods, x, logits, steps, warmup):
+    """Step s runs weight copy s % copies on router logits s % variants."""
     import torch
-    n = len(mods)
+    n, v = len(mods), len(logits)
     settle_clocks(mods, x, logits, PRELUDE_S)
     for s in range(warmup):
-        mods[s % n].forward(x, router_logits=logits)
+        mods[s % n].forward(x, router_logits=logits[s % v])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(steps):
-        mods[s % n].forward(x, router_logits=logits)
+        mods[s % n].forward(x, router_logits=logits[s % v])
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps
 
 
+def pick_rotation(mods, x, base_logits):
+    """Router logits for the timed steps such that no weight can stay in the Infinity Cache from
+    one use to the next.  A small batch touches a few experts only, so three copies of them fit
+    the cache; the steps therefore also cycle through variants of the logits with the expert axis
+    rolled (the same distribution of routed rows under another expert numbering), as many as it
+    takes for the distinct (copy, expert) weights of one cycle to exceed twice the cache.  Returns
+    the logits, the routed-row counts of each variant and the description of the cycle."""
+    import math
+    import torch
+    from dartmoq_hip.moe import forward_staged
+    mod, copies = mods[0], len(mods)
+    n_exp = mod.num_experts + mod.n_shared
+    experts = base_logits.shape[1]
+    counts_of = {}
+    variants = 1
+    while True:
+        shifts = [v * (experts // variants) for v in range(variants)]
+        for sh in shifts:
+            if sh not in counts_of:
+                lg = torch.roll(base_logits, shifts=sh, dims=1).contiguous()
+                _o, _s, aux = forward_staged(mod, x, router_logits=lg, profile=False)
+                counts_of[sh] = (lg, aux["counts"].cpu().tolist())
+        cycle = math.lcm(copies, variants)
+        weight_bytes = 0
+        for c in range(copies):
+            union = [0] * n_exp
+            for s in range(c, cycle, copies):
+                cnt = counts_of[shifts[s % variants]][1]
+                union = [u or int(k > 0) for u, k in zip(union, cnt)]
+            weight_bytes += layer_bytes(mod, union)[0]
+        if weight_bytes >= 2 * MALL_BYTES or variants >= MAX_LOGIT_VARIANTS:
+            break
+        variants *= 2
+    logits = [counts_of[sh][0] for sh in shifts]
+    counts = [counts_of[sh][1] for sh in shifts]
+    return logits, counts, {"weight_copies_rotated": copies, "logit_variants": variants,
+                            "cycle_steps": cycle, "cycle_weight_bytes": weight_bytes,
+                            "exceeds_twice_infinity_cache": weight_bytes >= 2 * MALL_BYTES}
+
+
+def kernel_work(mod, counts, tokens, fused_pools):
+    """Algorithmic work of one forward with these routed-row counts: the layer's bytes, and for
+    the gate_up and the down launch the packed indices + fp16 norms of the distinct routed experts
+    and the activation rows in and out (bytes) and the GEMM itself (flops).  What the gate_up
+    launch does on top for the pools in `fused_pools` (it rotates its SiLU*up rows for the down
+    projection: 2*I*128 flop per row, one 32 KiB matrix per distinct expert and down group) is
+    kept apart as extra_*."""
+    h, i = mod.hidden_size, mod.intermediate_size
+    layer_total, per_pool = layer_bytes(mod, counts)
+    w = {"layer_bytes": layer_total + 2 * tokens * h * 2, "gu_bytes": 0, "gu_flops": 0.0,
+         "gu_extra_bytes": 0, "gu_extra_flops": 0.0, "dn_bytes": tokens * h * 2, "dn_flops": 0.0,
+         "rows": 0, "distinct": 0}
+    for p, (_key, (d_b, r_b, bit_b)) in enumerate(per_pool.items()):
+        w["gu_bytes"] += d_b * (2 * h * i * bit_b // 8 + 4 * h * i // 128)
+        w["gu_bytes"] += (tokens if r_b else 0) * h * 2 + r_b * i * 2
+        w["gu_flops"] += 2.0 * r_b * h * 2 * i
+        w["dn_bytes"] += d_b * (h * i * bit_b // 8 + 2 * h * i // 128) + r_b * i * 2
+        w["dn_flops"] += 2.0 * r_b * i * h
+        if fused_pools >> p & 1:
+            w["gu_extra_flops"] += 2.0 * r_b * i * 128
+            w["gu_extra_bytes"] += d_b * (i // 128) * 128 * 128 * 2
+        w["rows"] += r_b
+        w["distinct"] += d_b
+    return w
+
+
+def roofline_of(nbytes, flops, ms, mode):
+    """The binding roofline of a launch of `nbytes` algorithmic bytes and `flops` algorithmic
+    flops that took `ms`."""
+    t_hbm, t_mfma = nbytes / HBM_PEAK, flops / MFMA_PEAK[mode]
+    if t_hbm >= t_mfma:
+        roof = {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
+                "unit": "GB/s"}
+    else:
+        roof = {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12,
+                "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    return roof
+
+
 def measure(mods, tokens, steps, warmup, seed, zipf, mode):
-    """Throughput of the full layer plus the live timing of its dominant kernel."""
+    """Throughput of the full layer plus the live timing of its two GEMM launches."""
     import torch
     from dartmoq_hip import synthetic
     from dartmoq_hip.moe import forward_staged
     mod = mods[0]
-    h, i, k = mod.hidden_size, mod.intermediate_size, mod.top_k
-    x = torch.randn(tokens, h, generator=torch.Generator().manual_seed(seed)).half().cuda()
-    logits = synthetic.zipf_logits(tokens, mod.num_experts, seed, skew=zipf).cuda()
+    x = torch.randn(tokens, mod.hidden_size, generator=torch.Generator().manual_seed(seed)).half().cuda()
+    base = synthetic.zipf_logits(tokens, mod.num_experts, seed, skew=zipf).cuda()
+    logits, counts, rotation = pick_rotation(mods, x, base)
     sec = time_steps(mods, x, logits, steps, warmup)
 
-    # stage timing (events on the launch stream), rotating the copies like the timed loop
-    reps = max(3, min(steps, 20))
+    # stage timing (events on the launch stream), copies and logits rotating like the timed loop,
+    # every variant of the logits the same number of times
+    n_var = len(logits)
+    reps = n_var * -(-max(3, min(steps, 20)) // n_var)
     acc = {}
     aux = None
-    for r in range(reps + 1):
-        _out, stats, aux = forward_staged(mods[r % len(mods)], x, router_logits=logits)
-        if r == 0:
+    for r in range(-1, reps):
+        _out, stats, aux = forward_staged(mods[r % len(mods)], x, router_logits=logits[r % n_var])
+        if r < 0:
             continue                                   # first pass warms the allocator
         for name, ms in stats.items():
             acc[name] = acc.get(name, 0.0) + ms
     stage_ms = {n: v / reps for n, v in acc.items()}
-    counts = aux["counts"].cpu().tolist()
-    bytes_total, per_pool = layer_bytes(mod, counts)
-    bytes_total += 2 * tokens * h * 2                  # x in, y out (fp16)
+    fused = aux["fused_rot_pools"]
+    work = [kernel_work(mod, c, tokens, fused) for c in counts]
+    avg = {key: sum(w[key] for w in work) / len(work) for key in work[0]}
     flops = tokens * mod.flops_per_token()
 
-    # dominant kernel: the merged gate_up dequant-GEMM (one launch over all bit pools).
-    # algorithmic bytes = packed gate_up indices + fp16 norms of the distinct routed experts,
-    # the rotated activations read once per token and pool, and the SiLU*up rows written
-    gu_bytes = 0
-    rows = 0
-    distinct = 0
-    for _key, (d_b, r_b, bit_b) in per_pool.items():
-        gu_bytes += d_b * (2 * h * i * bit_b // 8 + 4 * h * i // 128)
-        gu_bytes += (tokens if r_b else 0) * h * 2 + r_b * i * 2
-        rows += r_b
-        distinct += d_b
-    gu_flops = 2.0 * rows * h * 2 * i
-    # without a K split the same launch also rotates its SiLU*up rows for the down projection:
-    # 2*I*128 flop per row and one 32 KiB matrix per (distinct expert, down group)
-    fused_rot = aux["ks"] in (1, -2, -4) and all(bw.bit != 8 for bw in mod.bit_weights.values())
-    if fused_rot:
-        gu_flops += 2.0 * rows * i * 128
-        gu_bytes += distinct * (i // 128) * 128 * 128 * 2
+    # dominant kernel: the merged gate_up dequant-GEMM (one launch over all bit pools)
     gu_ms = stage_ms["merged_gate_up"]
-    t_hbm, t_mfma = gu_bytes / HBM_PEAK, gu_flops / MFMA_PEAK[mode]
-    if t_hbm >= t_mfma:
-        roof = {"bound": "hbm", "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
-                "unit": "GB/s"}
-    else:
-        roof = {"bound": "mfma", "achieved": gu_flops / (gu_ms * 1e-3) / 1e12,
-                "peak": MFMA_PEAK[mode] / 1e12, "unit": "TFLOP/s"}
-    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof = roofline_of(avg["gu_bytes"], avg["gu_flops"], gu_ms, mode)
     roof["traffic"] = None
     shared_k = f", K shared by {-aux['ks']} workgroups" if aux["ks"] < 0 else ""
     roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={max(aux['ks'], 1)},"
-                       f"{'SILU_ROT' if fused_rot else 'SILU'}> merged gate_up"
-                       f"{' + down rotation' if fused_rot else ''}, nbl={min(aux['nbl'], 2)}{shared_k}",
+                       f"{'SILU_ROT' if fused else 'SILU'}> merged gate_up"
+                       f"{' + down rotation' if fused else ''}, nbl={min(aux['nbl'], 2)}{shared_k}",
                 launch_ms=gu_ms,
-                algorithmic_bytes=gu_bytes, algorithmic_flops=gu_flops,
-                distinct_experts=distinct, routed_rows=rows)
+                algorithmic_bytes=avg["gu_bytes"], algorithmic_flops=avg["gu_flops"],
+                extra_bytes=avg["gu_extra_bytes"], extra_flops=avg["gu_extra_flops"],
+                distinct_experts=avg["distinct"], routed_rows=avg["rows"])
+    dn_ms = stage_ms["merged_down"]
+    roof_down = roofline_of(avg["dn_bytes"], avg["dn_flops"], dn_ms, mode)
+    roof_down.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['down_tt']},SCATTER> merged down",
+                     launch_ms=dn_ms, algorithmic_bytes=avg["dn_bytes"],
+                     algorithmic_flops=avg["dn_flops"])
     return {
         "tokens": tokens, "ms_per_step": sec * 1e3, "tokens_per_s": tokens / sec,
         "eff_tflops": flops / sec / 1e12,
-        "layer_hbm_frac": bytes_total / HBM_PEAK / sec,
+        "layer_hbm_frac": avg["layer_bytes"] / HBM_PEAK / sec,
         "layer_mfma_frac": flops / MFMA_PEAK[mode] / sec,
-        "layer_algorithmic_bytes": bytes_total,
+        "layer_algorithmic_bytes": avg["layer_bytes"],
         "gpu_stage_ms": {n: round(v, 4) for n, v in stage_ms.items()},
         "gpu_stage_sum_ms": round(sum(stage_ms.values()), 4),
         "tt": aux["tt"], "ks": aux["ks"], "nbl": aux["nbl"], "work_items": aux["n_items"],
-    }, roof
+        **rotation,
+    }, roof, roof_down
 
 
 def measured_traffic(config, mode, tokens):
@@ -367,16 +440,17 @@ def main():
         torch.cuda.synchronize()
         del probe
 
-    main_res, roof = measure(mods, args.tokens, args.steps, args.warmup, args.seed, spec["zipf"],
-                             args.mode)
+    main_res, roof, roof_down = measure(mods, args.tokens, args.steps, args.warmup, args.seed,
+                                        spec["zipf"], args.mode)
     roof["traffic"] = measured_traffic(args.config, args.mode, args.tokens)
     sweep = []
     for t in [int(v) for v in args.sweep.split(",") if v]:
         if t == args.tokens:
             continue
-        res, r = measure(mods, t, args.steps, args.warmup, args.seed, spec["zipf"], args.mode)
+        res, r, rd = measure(mods, t, args.steps, args.warmup, args.seed, spec["zipf"], args.mode)
         r["traffic"] = measured_traffic(args.config, args.mode, t)
         res["roofline"] = r
+        res["roofline_down"] = rd
         sweep.append(res)
     del mods
 
@@ -388,14 +462,20 @@ def main():
         sp = synthetic.CONFIGS[cfg_m]
         mm = modules(cfg_m, mode_s)
         for t in [int(v) for v in tok_s.split("/")]:
-            res, r = measure(mm, t, args.steps, args.warmup, args.seed, sp["zipf"], mode_s)
+            res, r, rd = measure(mm, t, args.steps, args.warmup, args.seed, sp["zipf"], mode_s)
             r["traffic"] = measured_traffic(cfg_m, mode_s, t)
             mode_results.append({"config": cfg_m, "mode": mode_s, "dtype": DTYPE[mode_s], "tokens": t,
                                  "value": res["tokens_per_s"], "unit": "tokens/s",
                                  "ms_per_step": res["ms_per_step"], "eff_tflops": res["eff_tflops"],
                                  "layer_hbm_frac": res["layer_hbm_frac"],
                                  "layer_mfma_frac": res["layer_mfma_frac"],
-                                 "gpu_stage_ms": res["gpu_stage_ms"], "roofline": r})
+                                 "gpu_stage_ms": res["gpu_stage_ms"],
+                                 "weight_copies_rotated": res["weight_copies_rotated"],
+                                 "logit_variants": res["logit_variants"],
+                                 "cycle_steps": res["cycle_steps"],
+                                 "cycle_weight_bytes": res["cycle_weight_bytes"],
+                                 "exceeds_twice_infinity_cache": res["exceeds_twice_infinity_cache"],
+                                 "roofline": r, "roofline_down": rd})
         del mm
         torch.cuda.empty_cache()
 
@@ -426,11 +506,14 @@ def main():
                            if shared is not None else "") +
                         f"group 128, T={args.tokens} tokens, "
                         f"{'Zipf(1.1)-skewed' if spec['zipf'] else 'uniform'} randn router logits",
-            "tokens": args.tokens, "mode": args.mode, "weight_copies_rotated": N_COPIES,
+            "tokens": args.tokens, "mode": args.mode,
+            "weight_copies_rotated": main_res["weight_copies_rotated"],
+            "logit_variants": main_res["logit_variants"],
         },
         "eff_tflops": main_res["eff_tflops"],
         "layer": main_res,
         "roofline": roof,
+        "roofline_down": roof_down,
         "cpu_baseline": cpu,
         "sweep": sweep,
         "modes": mode_results,

@@ -192,7 +192,8 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
 // Scratch of dmq_route_permute_static: the per-chunk expert histograms of the counting sort at their
 // largest (DMQ_SORT_MAX_CHUNKS chunks x DMQ_SORT_MAX_EXPERTS experts), one copy per GPU, held until the
 // process ends.  Host code never uses the array's name as an address: the device address is looked
-// up once per device (with that device current) and cached.
+// up once per device (with that device current) and cached.  Two host threads making the first
+// call on a device at once both look it up and store the same value.
 #define DMQ_STATIC_SCRATCH_BYTES (DMQ_SORT_MAX_CHUNKS * DMQ_SORT_MAX_EXPERTS * 4)
 #define DMQ_STATIC_MAX_DEVICES 64
 static __device__ __align__(256) unsigned char dmq_static_scratch[DMQ_STATIC_SCRATCH_BYTES];
@@ -967,6 +968,14 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   const bool widths_apart = tt != 1 || (long)tokens * K > 1280;
   bool fuse_rot[DMQ_MAX_POOLS];
   for (int mi = 0; mi < n_modes; ++mi) fuse_rot[mi] = (ks == 1);
+  if (aux_out) {
+    // which pools get their SiLU*up rows rotated inside the gate_up launch (bit i: pool i)
+    long mask = 0;
+    for (int mi = 0; mi < n_modes; ++mi)
+      for (int i = 0; i < P; ++i)
+        if (fuse_rot[mi] && layer->pool[i].mode == modes[mi]) mask |= 1L << i;
+    ((long*)aux_out)[6] = mask;
+  }
 
   // Which pools rotate every token once instead of their routed rows: the caller's choice (pools
   // expected to see more routed rows than tokens) and, for small batches, all of them: rotating a
@@ -1249,6 +1258,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     const long avg_rows = (long)tokens * K / E;
     const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
     d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = w.tile_rows; d.roomy = roomy;
+    if (aux_out && mi == 0) ((long*)aux_out)[7] = down_tt;
     d.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
     d.widths_apart = widths_apart;
     d.ks = ks; d.n_pools = P;

@@ -290,7 +290,10 @@ class WxA16BitPartitionedGroupMoE:
         their own rule (qwen35_quant_io.py:416-532): a WxA16 layer keeps them fp16; the other
         modes move an 8-bit Linear to int8 only when its codebook is the uniform grid (a Lloyd-Max
         codebook would lose levels on the int8 grid) and never to fp8 unless asked to
-        (attn="wxfp8"); anything else stays on the fp16 path."""
+        (attn="wxfp8"); anything else stays on the fp16 path.  The reference decides per Linear;
+        a pool has one mode for its gate_up and its down projection, so a shared expert with one
+        uniform and one Lloyd-Max codebook runs both projections in fp16 here (the reference would
+        run the uniform one in int8)."""
         mode = MODE_BY_NAME[self.MODE]
         if mode == MODE_A16 or self.shared_attn == "wxa16" or bw.bit != 8:
             return MODE_A16
@@ -587,4 +590,4 @@ def forward_staged(moe: WxA16BitPartitionedGroupMoE, x: torch.Tensor,
     counts = ws[aux[2]:aux[2] + 4 * (moe.num_experts + moe.n_shared)].view(torch.int32).clone()
     n_items = int(ws[aux[4]:aux[4] + 4].view(torch.int32).item())
     return out, stats, {"counts": counts, "tt": int(aux[0]), "ks": int(aux[1]), "nbl": int(aux[5]),
-                        "n_items": n_items}
+                        "n_items": n_items, "fused_rot_pools": int(aux[6]), "down_tt": int(aux[7])}

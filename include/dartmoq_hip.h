@@ -146,8 +146,10 @@ int dmq_route_permute(const void* topk_idx, const void* topk_w, int tokens, int 
  * library, one copy per GPU, held until the process ends; its size covers every accepted call
  * (any number of tokens, experts <= 2048; larger problems return DMQ_ERR_LIMIT).  The call
  * allocates nothing.  All calls on one GPU share that array: calls that overlap on a GPU (two
- * streams, two threads) race; calls ordered on one stream do not.  Arguments and outputs as
- * dmq_route_permute. */
+ * streams, two threads) race; calls ordered on one stream do not.  The first call on a GPU looks
+ * the array's address up (hipGetSymbolAddress, which may load the code object): make that call
+ * outside any stream capture; later calls on that GPU only launch kernels.  Arguments and outputs
+ * as dmq_route_permute. */
 int dmq_route_permute_static(const void* topk_idx, const void* topk_w, int tokens, int k,
                              int experts, int pools, const void* slice_start,
                              const void* slice_count, int tile_rows, int max_items, void* counts,
@@ -447,7 +449,8 @@ int dmq_moe_ffn_forward(const dmq_layer_desc* layer, const void* x, const void* 
  * hipEvent_t recorded on `stream` before the first launch and after each stage (sort_prep,
  * rotation, merged_gate_up, act_quant_down, merged_down, combine); aux_out (optional) is a host
  * long[8] that receives tt, ks, the byte offset of counts[experts] inside the workspace,
- * max_items, the byte offset of n_items and nbl. */
+ * max_items, the byte offset of n_items, nbl, the mask of pools whose SiLU*up rows the gate_up
+ * launch rotates itself (bit i: pool i) and the tt of the first down launch. */
 int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const void* topk_idx,
                                const void* topk_w, int tokens, const void* add_f16, void* out,
                                void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,

@@ -149,9 +149,18 @@ def test_fused_rotate_quantize_exact_rotations(mode, rows, tt):
         assert torch.equal(codes.cpu(), p_ref)
 
 
+def _flips(a, b):
+    return (a != b).float().mean().item()
+
+
 @pytest.mark.parametrize("mode", [0, A8, FP8, FP4])
 def test_fused_rotate_quantize_haar(mode):
-    """Haar rotations: values agree to accumulation round-off, codes to one rounding step."""
+    """Haar rotations: the kernel accumulates the rotation in another order than the fp32 matmul of
+    the oracle, so a value that sits within round-off of a rounding boundary may land on the other
+    side.  Measured on MI355X over three seeds and three shapes (up to 2048 x 2048 values): int8
+    codes differ at 0.5 - 1.1e-5 of the positions (always by one step), fp8 codes at 0.4 - 1.5e-5,
+    e2m1 bytes at 0 - 1.0e-5, the fp16 scales of a group at 0 - 2.8e-4 (one ulp), e2m1 scale bytes
+    never, fp16 rows at 1.0e-3 (one ulp).  The bounds below are three times the largest rate."""
     from dartmoq_hip import ops
     rows, k = 257, 2048
     x = _inputs(rows, k, 11)
@@ -161,23 +170,25 @@ def test_fused_rotate_quantize_haar(mode):
     codes, scale = ops.rotate(mode, x.cuda(), rot.cuda(), extra_scale=0.0118931, tt=4)
     if mode == 0:
         torch.testing.assert_close(codes.cpu().float(), x_rot, rtol=2e-3, atol=2e-3)
+        assert _flips(codes.cpu().view(torch.int16), x_rot.half().view(torch.int16)) < 3.3e-3
         return
     if mode == A8:
         q_ref, s_ref = actquant.quantize_act_int8(x_rot, 128, 0.0118931)
         diff = (codes.cpu().int() - q_ref.int()).abs()
         assert diff.max() <= 1
-        assert (diff != 0).float().mean() < 2e-3
-        torch.testing.assert_close(scale.cpu().float(), s_ref, rtol=2e-3, atol=1e-9)
+        assert (diff != 0).float().mean() < 3.5e-5
+        assert _flips(scale.cpu().view(torch.int16), s_ref.half().view(torch.int16)) < 8.5e-4
+        torch.testing.assert_close(scale.cpu().float(), s_ref, rtol=1e-3, atol=1e-9)
     elif mode == FP8:
         q_ref, s_ref = actquant.quantize_act_fp8(x_rot, 128, 0.0118931)
-        same = codes.cpu().view(torch.uint8) == q_ref.view(torch.uint8)
-        assert (~same).float().mean() < 2e-3
+        assert _flips(codes.cpu().view(torch.uint8), q_ref.view(torch.uint8)) < 4.6e-5
         torch.testing.assert_close(codes.cpu().float(), q_ref.float(), rtol=0.13, atol=2 ** -9)
-        torch.testing.assert_close(scale.cpu().float(), s_ref, rtol=2e-3, atol=1e-9)
+        assert _flips(scale.cpu().view(torch.int16), s_ref.half().view(torch.int16)) < 8.5e-4
+        torch.testing.assert_close(scale.cpu().float(), s_ref, rtol=1e-3, atol=1e-9)
     else:
         p_ref, sb_ref = actquant.quantize_act_e2m1(x_rot)
-        assert (scale.cpu() != sb_ref).float().mean() < 1e-3
-        assert (codes.cpu() != p_ref).float().mean() < 5e-3
+        assert torch.equal(scale.cpu(), sb_ref)
+        assert _flips(codes.cpu(), p_ref) < 3.1e-5
 
 
 def test_rotate_rejects_bad_shapes():

@@ -52,12 +52,17 @@ def _compare(tokens, experts, k, tile_rows, seed):
 
 
 def test_static_scratch_two_calls_in_a_row():
-    # 4096 tokens x 8: the three-launch path whose histograms live in the scratch (64 chunks)
+    # 4096 tokens x 8 = 32768 routed rows: the chunked path whose per-chunk histograms live in the
+    # scratch (64 chunks, 256 experts)
     _compare(4096, 256, 8, 32, seed=1)
-    # a smaller input right after: fewer chunks, fewer experts; the array still holds the first
-    # call's histograms
-    _compare(600, 48, 4, 16, seed=2)
-    # and a batch small enough for the one-launch path, which never touches the scratch
+    # a smaller input right after, still beyond 16384 routed rows: fewer chunks and fewer experts
+    # over the histograms the first call left behind
+    _compare(3000, 100, 8, 32, seed=2)
+    # more than 512 experts: the plan step rewrites the histograms in place before the fill step
+    # reads them, here over the stale contents of the two calls before
+    _compare(2500, 1000, 8, 16, seed=4)
+    # batches small enough for the paths that never touch the scratch
+    _compare(600, 48, 4, 16, seed=5)
     _compare(16, 48, 4, 16, seed=3)
 
 

@@ -107,6 +107,30 @@ def test_e2m1_power_of_two_edges_and_ties():
     assert torch.equal(p.cpu(), p_ref)
 
 
+def test_quantizers_match_reference_written_vectors():
+    """The reference's own torch quantizers on inputs with ties, all-zero and tiny groups
+    (tests/golden/actquant_fixtures.json, written by make_actquant_fixtures.py): the kernels
+    return the same codes, and the same fp32 scales where they offer fp32 scales."""
+    import json
+    import os
+    from dartmoq_hip import ops
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "actquant_fixtures.json")
+    with open(path) as fh:
+        gold = json.load(fh)
+    for rec in gold["act"]:
+        x = torch.tensor(rec["x_fp32_bits"], dtype=torch.int32).view(torch.float32)
+        x = x.reshape(rec["rows"], rec["k"]).cuda()
+        q, s = ops.quantize_act(A8, x, rec["extra_scale"], scale_fp32=True)
+        assert q.cpu().flatten().tolist() == rec["int8"]
+        assert s.cpu().view(torch.int32).flatten().tolist() == rec["int8_scale_fp32_bits"]
+        q, s = ops.quantize_act(FP8, x, rec["extra_scale"], scale_fp32=True)
+        assert q.cpu().view(torch.uint8).flatten().tolist() == rec["e4m3_bytes"]
+        assert s.cpu().view(torch.int32).flatten().tolist() == rec["e4m3_scale_fp32_bits"]
+        p, sb = ops.quantize_act(FP4, x)
+        assert sb.cpu().flatten().tolist() == rec["e2m1_scale_bytes"]
+        assert p.cpu().flatten().tolist() == rec["e2m1_packed"]
+
+
 def _exact_rotations(groups, seed):
     """Rotations whose products are exact in fp32 in any summation order: a signed permutation
     composed with a block-diagonal 4x4 Hadamard / 2 (entries 0, +-1/2)."""

@@ -2,6 +2,7 @@
 #include "params.h"
 #include "topk.h"
 #include "gemm_dispatch.h"
+#include "router.h"
 
 __global__ __launch_bounds__(256) void dmq_fill_zero_kernel(uint32_t* p, long n_words) {
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_words;
@@ -57,7 +58,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 19; }
+int dmq_abi_version(void) { return 20; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -723,6 +724,7 @@ struct MoeWorkspace {
   float* split_partial;              // gate_up K range shared between workgroups: fp32 sums
   int* split_counter;
   int* rows_queue;                   // queue words of the persistent gate_up and down launches
+  __half* router_logits;             // [16, experts] logits of the router workgroups (pre-norm entry)
   int split_rows, split_counters;
   void* sort_scratch;
   size_t sort_scratch_bytes;
@@ -769,6 +771,7 @@ static MoeWorkspace carve(const dmq_layer_desc* L, int tokens, int tt, uint8_t* 
   w.dn_info = (int*)take(P * E * 16);
   w.n_items = (int*)take(16);
   w.rows_queue = (int*)take(2 * DMQ_ROWS_QUEUE_WORDS * 4);
+  w.router_logits = (__half*)take((size_t)DMQ_PRENORM_MAX_TOKENS * E * 2);
   w.sort_scratch_bytes = dmq_route_scratch_bytes(tokens, L->top_k, L->experts);
   w.sort_scratch = take(w.sort_scratch_bytes);
   w.items = (int*)take((size_t)w.max_items * DMQ_ITEM_WORDS * sizeof(int));
@@ -818,12 +821,42 @@ int dmq_moe_ffn_forward_staged(const dmq_layer_desc* layer, const void* x, const
                                     tt, ks, nbl, stage_events, aux_out, stream);
 }
 
+// pre != NULL: x holds the block's pre-norm input; the first launch normalizes it, projects it onto
+// the router and runs the top-k (dmq_moe_ffn_forward_prenorm)
+static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_args* router,
+                               const dmq_prenorm_args* pre, const void* x, int tokens,
+                               const void* add_f16, void* out, void* workspace,
+                               size_t workspace_bytes, int tt, int ks, int nbl,
+                               void* const* stage_events, void* aux_out, void* stream);
+
 int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_args* router,
                                const void* x, int tokens, const void* add_f16, void* out,
                                void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
                                void* const* stage_events, void* aux_out, void* stream) {
-  if (!layer || !router || !x || !out || !workspace || !layer->pool) return DMQ_ERR_NULL;
+  if (!router) return DMQ_ERR_NULL;
   if (!router->logits && (!router->topk_idx || !router->topk_w)) return DMQ_ERR_NULL;
+  return forward_routed_impl(layer, router, nullptr, x, tokens, add_f16, out, workspace, workspace_bytes,
+                             tt, ks, nbl, stage_events, aux_out, stream);
+}
+
+int dmq_moe_ffn_forward_prenorm(const dmq_layer_desc* layer, const dmq_router_args* router,
+                                const dmq_prenorm_args* pre, const void* h, int tokens,
+                                const void* add_f16, void* out, void* workspace,
+                                size_t workspace_bytes, int tt, int ks, int nbl,
+                                void* const* stage_events, void* aux_out, void* stream) {
+  if (!router || !pre || !pre->norm_weight || !pre->gate_weight || !pre->state) return DMQ_ERR_NULL;
+  if (router->logits || router->topk_idx || router->topk_w) return DMQ_ERR_MODE;   // the launch makes them
+  if (tokens > DMQ_PRENORM_MAX_TOKENS) return DMQ_ERR_LIMIT;
+  return forward_routed_impl(layer, router, pre, h, tokens, add_f16, out, workspace, workspace_bytes,
+                             tt, ks, nbl, stage_events, aux_out, stream);
+}
+
+static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_args* router,
+                               const dmq_prenorm_args* pre, const void* x, int tokens,
+                               const void* add_f16, void* out, void* workspace,
+                               size_t workspace_bytes, int tt, int ks, int nbl,
+                               void* const* stage_events, void* aux_out, void* stream) {
+  if (!layer || !router || !x || !out || !workspace || !layer->pool) return DMQ_ERR_NULL;
   const int n_shared = router->n_shared;
   if (n_shared < 0 || n_shared >= layer->top_k || n_shared >= layer->experts) return DMQ_ERR_SHAPE;
   if (n_shared > 0 && !router->shared_gate_row) return DMQ_ERR_NULL;
@@ -1011,13 +1044,16 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   bool whole_done[DMQ_MAX_POOLS] = {false, false, false, false};   // per mode
   int a16_mi = -1;
   for (int mi = 0; mi < n_modes; ++mi) if (modes[mi] == DMQ_MODE_A16) a16_mi = mi;
+  PreNorm pn{};
+  if (pre) pn = PreNorm{pre->norm_weight, pre->norm_weight_fp32, pre->eps, 1};
   auto rotate_gate_up_input = [&](int mode, bool whole, bool tiled, const TopkParams* tp,
-                                  int tp_fp16) -> int {
+                                  int tp_fp16, const RouterParams* rt = nullptr) -> int {
     // the whole-batch pools of the fp16 mode ride the main mode's launch (see `dual`): same
     // rotation, their rows are stored as fp16 instead of going through the quantizer
     const bool with_f16 = dual && mode == main_mode && whole && !whole_done[a16_mi];
     RotParams rp{};
     rp.x = (const __half*)x; rp.x_stride = H; rp.row_index = w.sorted_tokens;
+    rp.pn = pn;
     rp.rows = tokens; rp.groups = H / DMQ_GS;
     rp.items = w.items; rp.n_items = w.n_items; rp.tile_rows = w.tile_rows; rp.scale_fp32 = 0;
     rp.items_prefix = 1;
@@ -1045,11 +1081,13 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
     else rp.items = nullptr;
     if (rp.n_hoisted == 0 && !any_tiled && !tp) return DMQ_OK;
     rp.also_f16 = with_f16 ? 1 : 0;
-    const int rc_rot = dmq_rotate_dispatch(mode, rp, n, rtt, st, tp, tp_fp16);
+    if (pn.on && (any_tiled || (!rt && rp.n_hoisted == 0))) return any_tiled ? DMQ_ERR_MODE : DMQ_OK;
+    const int rc_rot = rt ? dmq_rotate_router_dispatch(mode, rp, *rt, st)
+                          : dmq_rotate_dispatch(mode, rp, n, rtt, st, tp, tp_fp16);
     if (!rc_rot && with_f16) whole_done[a16_mi] = true;   // fp16 pools rotated per work item keep their own pass
     return rc_rot;
   };
-  const bool route_small = (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
+  const bool route_small = !pre && (long)tokens * K <= DMQ_ROUTE_SMALL_ROWS && E <= DMQ_ROUTE_SMALL_EXPERTS &&
                            K <= 64 && (!router->logits || tokens <= DMQ_ROUTE_SMALL_TOKENS);
   // When the top-k is a launch of its own (logits, more than 16 tokens) it shares the launch of the
   // whole-batch rotation of the first mode: neither needs the other, both are short.
@@ -1062,12 +1100,14 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
                 R <= w.max_items && K <= 64 &&
                 (wsplit_eff == 1 || R * (I / DMQ_GS) <= w.split_counters);
   bool direct_done = false;
-  if (direct || (!route_small && router->logits)) {
+  if (direct || (!route_small && router->logits) || pre) {
     bool any_whole = false;
     for (int i = 0; i < P; ++i) any_whole |= (whole_batch[i] && layer->pool[i].mode == modes[0]);
     const int rk = K - n_shared, re = E - n_shared;
-    if (any_whole && re <= 1024 && rk <= 64 && rk <= re && rk > 0 && n_shared <= 64) {
-      const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
+    const bool topk_fits = any_whole && re <= 1024 && rk <= 64 && rk <= re && rk > 0 && n_shared <= 64;
+    if (pre && (!topk_fits || sub || re % 4)) return DMQ_ERR_LIMIT;
+    if (topk_fits) {
+      const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared, pn, nullptr};
       TopkParams tp{router->logits, tokens, re, rk, router->renorm, w.topk_w, w.topk_idx, sg,
                     (tokens + 3) / 4, DirectPlan{}, (const int*)router->topk_idx,
                     (const float*)router->topk_w};
@@ -1083,7 +1123,18 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
         if (wsplit_eff > 1) { dp.clear_words = w.split_counter; dp.clear_count = w.split_counters; }
         direct_done = true;
       }
-      rc = rotate_gate_up_input(modes[0], true, false, &tp, router->logits_fp16);
+      if (pre) {
+        RouterParams rt{};
+        rt.h = (const __half*)x; rt.h_stride = H; rt.tokens = tokens; rt.hidden = H; rt.pn = pn;
+        rt.gate_w = (const __half*)pre->gate_weight; rt.experts = re;
+        rt.logits = w.router_logits; rt.ticket = (int*)pre->state;
+        rt.x_norm_out = (__half*)pre->x_norm_out; rt.logits_out = (__half*)pre->logits_out;
+        rt.blocks = (re + 15) / 16;
+        rt.tp = tp;
+        rc = rotate_gate_up_input(modes[0], true, false, nullptr, 0, &rt);
+      } else {
+        rc = rotate_gate_up_input(modes[0], true, false, &tp, router->logits_fp16);
+      }
       if (rc) return rc;
       whole_done[0] = true;
       topk_done = true;
@@ -1094,7 +1145,7 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
   //    expert_info, work items: one launch for small batches
   {
     const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
-    const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared};
+    const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared, pn, nullptr};
     // up to DMQ_ROUTE_RANK_ROWS (128) routed rows with the top-k at hand: the one-row-per-thread ranking kernel
     const int* rank_idx = topk_done ? w.topk_idx
                                     : ((!router->logits && n_shared == 0) ? (const int*)router->topk_idx : nullptr);

@@ -2,6 +2,7 @@
 // * (1 + weight), everything in fp32 with one final rounding to the activation type.  One wave per
 // row; the row is read twice (the second time from cache) and written once.  HBM-bound byte mover.
 #include "params.h"
+#include "prenorm.h"
 #include <hip/hip_bf16.h>
 
 template <typename T> __device__ __forceinline__ float norm_to_f32(T v);
@@ -21,16 +22,8 @@ void dmq_rms_norm_kernel(const T* x, const W* weight, long rows, int n, long x_s
   if (row >= rows) return;
   const T* xr = x + row * x_stride;
   T* orow = out + row * out_stride;
-  float sumsq = 0.f;
-  for (int c = lane * 8; c < n; c += 512) {
-    const uint4_t raw = *(const uint4_t*)(xr + c);
-    const T* v = (const T*)&raw;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { const float f = norm_to_f32<T>(v[i]); sumsq += f * f; }
-  }
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) sumsq += __shfl_xor(sumsq, m, 64);
-  const float rstd = rsqrtf(sumsq / (float)n + eps);
+  const float sumsq = dmq_row_sumsq<T>(xr, n, lane, [](T v) { return norm_to_f32<T>(v); });
+  const float rstd = dmq_rstd(sumsq, n, eps);
   for (int c = lane * 8; c < n; c += 512) {
     const uint4_t raw = *(const uint4_t*)(xr + c);
     const T* v = (const T*)&raw;
@@ -38,7 +31,7 @@ void dmq_rms_norm_kernel(const T* x, const W* weight, long rows, int n, long x_s
     T* o = (T*)&packed;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      o[i] = norm_from_f32<T>(norm_to_f32<T>(v[i]) * rstd * (1.0f + norm_to_f32<W>(weight[c + i])));
+      o[i] = norm_from_f32<T>(dmq_norm_value(norm_to_f32<T>(v[i]), rstd, norm_to_f32<W>(weight[c + i])));
     *(uint4_t*)(orow + c) = packed;
   }
 }

@@ -32,6 +32,16 @@ struct LinearPrep {
   int zero_count;
 };
 
+// RMSNorm folded into a consumer of the layer input: the rows handed over are the block's
+// pre-norm input h, and every consumer forms x = fp16(h * rstd(row) * (1 + weight)) itself, with
+// the arithmetic of dmq_rms_norm_kernel (same bits as the stand-alone kernel's output).
+struct PreNorm {
+  const void* weight;      // [hidden] fp16 or fp32
+  int weight_fp32;
+  float eps;
+  int on;
+};
+
 struct RotParams {
   RotPool pool[DMQ_MAX_POOLS];
   const __half* x;         // [*, x_stride] fp16
@@ -51,6 +61,7 @@ struct RotParams {
   int items_prefix;        // 1: only the first n_items[1] items belong to tiled pools
   int also_f16;            // 1: whole-batch pools of mode DMQ_MODE_A16 are served too (rows stored as fp16)
   LinearPrep prep;
+  PreNorm pn;              // on: x holds pre-norm rows (whole-batch pools, 16-row tiles only)
 };
 
 struct QuantParams {
@@ -85,6 +96,8 @@ struct SharedGate {
   const __half* gate_row;        // [hidden]
   int hidden;
   int n_shared;
+  PreNorm pn;                    // on: x holds pre-norm rows, row_rstd their rsqrt(mean square + eps)
+  const float* row_rstd;         // [tokens]
 };
 
 struct PlanParams {
@@ -166,6 +179,8 @@ struct TopkParams;
 // tp != NULL: the launch also runs the router's top-k (workgroups in front; logits fp16 or fp32)
 int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream,
                         const TopkParams* tp = nullptr, int topk_fp16 = 0);
+struct RouterParams;
+int dmq_rotate_router_dispatch(int mode, const RotParams& p, const RouterParams& rt, hipStream_t stream);
 int dmq_quantize_dispatch(int mode, const QuantParams& p, hipStream_t stream);
 
 // int8 GEMM of a Linear with 8-bit weights on a uniform grid (w = idx - 128), 128 x 128 tiles

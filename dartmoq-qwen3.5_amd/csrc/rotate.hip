@@ -20,6 +20,7 @@
 // expert (the down rotations).
 #include "params.h"
 #include "topk.h"
+#include "router.h"
 #include <type_traits>
 
 __device__ __forceinline__ float wave_max16x4(float v) {
@@ -137,6 +138,21 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
 #pragma unroll
     for (int t = 0; t < TT; ++t)
       xraw[s][t] = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
+  if (TT == 1 && p.pn.on && staged) {
+    // pre-norm rows: the workgroup's four waves hold 64 consecutive rows; their rstd is computed
+    // by all four waves together (also by those whose tile lies past the last row), then every
+    // lane normalizes the pieces it holds
+    __shared__ float s_rstd[64];
+    const int row0 = r_first - wave * ROWS_PER_ITEM;
+    dmq_wg_rstd(p.x, p.x_stride, row0, p.rows, p.groups * DMQ_GS, p.pn.eps, s_rstd);
+    const float rstd = s_rstd[wave * 16 + l16];
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      float w8[8];
+      dmq_norm_weights8(p.pn, cg * DMQ_GS + 8 * q + 32 * s4, w8);
+      xraw[s4][0] = dmq_norm8(xraw[s4][0], rstd, w8);
+    }
+  }
   const bool stage_now = staged || (tiled_wg && stage_pool >= 0);   // uniform over the workgroup
   if (stage_now) {
     // 2048 chunks of 16 bytes, eight per thread; chunk c of row r sits at position c ^ (r % 16) so
@@ -303,6 +319,17 @@ void dmq_rotate_topk_kernel(RotParams p, TopkParams tp) {
   else dmq_rotate_wg<MODE, TT>(p, (int)blockIdx.x - tp.blocks, mat);
 }
 
+// The launch of a decode step that starts from the block's pre-norm input: workgroups
+// [0, rt.blocks) are the router (RMSNorm, projection, top-k; see router.h), the rest rotate the
+// whole-batch pools and normalize their rows on the way in (RotParams.pn).
+template <int MODE>
+__global__ __launch_bounds__(256)
+void dmq_rotate_router_kernel(RotParams p, RouterParams rt) {
+  __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
+  if ((int)blockIdx.x < rt.blocks) dmq_router_wg(rt, blockIdx.x, mat);
+  else dmq_rotate_wg<MODE, 1>(p, (int)blockIdx.x - rt.blocks, mat);
+}
+
 // Quantization of activations that are already rotated (no matrix product): one wave per
 // (row, group), two consecutive features per lane.
 template <int MODE>
@@ -408,6 +435,32 @@ static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStr
   else if (tt == 2) hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 2>), dim3(grid), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 1>), dim3(grid), dim3(256), 0, stream, p);
   return dmq_check_launch();
+}
+
+template <int MODE>
+static int launch_rotate_router(const RotParams& p_in, const RouterParams& rt, hipStream_t stream) {
+  RotParams p = p_in;
+  const long row_tiles = ((long)p.rows + 15) / 16;
+  p.hoisted_staged = 1;
+  p.hoisted_wgs_per_pool = (int)(((row_tiles + 3) / 4) * p.groups);
+  p.tiled_staged = 1;
+  p.items = nullptr;
+  const long total = (long)p.n_hoisted * p.hoisted_wgs_per_pool + rt.blocks;
+  hipLaunchKernelGGL((dmq_rotate_router_kernel<MODE>), dim3((int)total), dim3(256), 0, stream, p, rt);
+  return dmq_check_launch();
+}
+
+int dmq_rotate_router_dispatch(int mode, const RotParams& p, const RouterParams& rt, hipStream_t stream) {
+  if (!p.pn.on || rt.tokens <= 0 || rt.tokens > DMQ_PRENORM_MAX_TOKENS || p.rows != rt.tokens)
+    return DMQ_ERR_LIMIT;
+  if (rt.hidden % DMQ_GS || rt.experts % 4 || rt.experts > 1024 || rt.h_stride % 8) return DMQ_ERR_ALIGN;
+  switch (mode) {
+    case DMQ_MODE_A16: return launch_rotate_router<DMQ_MODE_A16>(p, rt, stream);
+    case DMQ_MODE_A8: return launch_rotate_router<DMQ_MODE_A8>(p, rt, stream);
+    case DMQ_MODE_FP8: return launch_rotate_router<DMQ_MODE_FP8>(p, rt, stream);
+    case DMQ_MODE_FP4: return launch_rotate_router<DMQ_MODE_FP4>(p, rt, stream);
+  }
+  return DMQ_ERR_MODE;
 }
 
 int dmq_rotate_dispatch(int mode, const RotParams& p, long tiled_waves, int tt, hipStream_t stream,

@@ -1,6 +1,7 @@
 // Top-k routing device code shared by the routing kernels and the fused rotation + top-k launch.
 #pragma once
 #include "params.h"
+#include "prenorm.h"
 
 // ------------------------------------------------------------------------------ top-k
 // Wave-wide max / min through data-parallel lane moves: xor 1, xor 2, mirror within 8 and within
@@ -36,8 +37,15 @@ template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return _
 __device__ __forceinline__ float dmq_shared_gate_value(const SharedGate& sg, int tok, int lane) {
   const __half* xr = sg.x + (long)tok * sg.hidden;
   float dot = 0.f;
+  const float rstd = sg.pn.on ? sg.row_rstd[tok] : 0.f;
   for (int h = lane * 8; h < sg.hidden; h += 512) {
-    const half8_t a = *(const half8_t*)(xr + h);
+    uint4_t raw = *(const uint4_t*)(xr + h);
+    if (sg.pn.on) {                      // pre-norm rows: normalize the piece first
+      float w[8];
+      dmq_norm_weights8(sg.pn, h, w);
+      raw = dmq_norm8(raw, rstd, w);
+    }
+    const half8_t a = __builtin_bit_cast(half8_t, raw);
     const half8_t b = *(const half8_t*)(sg.gate_row + h);
 #pragma unroll
     for (int c = 0; c < 8; ++c) dot += (float)a[c] * (float)b[c];

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 19
+ABI_VERSION = 20
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER, EPI_SILU_ROT = 0, 1, 2, 3
@@ -92,6 +92,14 @@ class RouterArgs(Structure):
     ]
 
 
+class PrenormArgs(Structure):
+    _fields_ = [
+        ("norm_weight", c_void_p), ("norm_weight_fp32", c_int), ("eps", ctypes.c_float),
+        ("gate_weight", c_void_p), ("state", c_void_p), ("x_norm_out", c_void_p),
+        ("logits_out", c_void_p),
+    ]
+
+
 # name -> (restype, argtypes); the single source for the symbol-export test as well
 PROTOTYPES = {
     "dmq_abi_version": (c_int, []),
@@ -142,6 +150,10 @@ PROTOTYPES = {
     "dmq_moe_ffn_forward_routed": (c_int, [POINTER(LayerDesc), POINTER(RouterArgs), c_void_p, c_int,
                                            c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int,
                                            c_int, POINTER(c_void_p), POINTER(c_long), c_void_p]),
+    "dmq_moe_ffn_forward_prenorm": (c_int, [POINTER(LayerDesc), POINTER(RouterArgs), POINTER(PrenormArgs),
+                                            c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t,
+                                            c_int, c_int, c_int, POINTER(c_void_p), POINTER(c_long),
+                                            c_void_p]),
 }
 
 _lib = None

@@ -18,7 +18,7 @@ import torch
 
 from . import hostprep, ops
 from ._lib import (MODE_A16, MODE_A8, MODE_BY_NAME, MODE_FP4, MODE_FP8, LayerDesc, PoolDesc,
-                   RouterArgs, check, load)
+                   PrenormArgs, RouterArgs, check, load)
 
 GROUP_SIZE = 128
 
@@ -125,6 +125,8 @@ class WxA16BitPartitionedGroupMoE:
         self.shared_gate_row = None
         self._desc = None
         self._workspace = None
+        self._gate_f16 = None       # fp16 copy of gate_weight and the state word of forward_prenorm
+        self._prenorm_state = None
         self.tt_override = 0        # activation tiles of 16 rows per wave (0 = pick from tokens)
         self.ks_override = 0        # waves splitting K inside a workgroup (0 = pick from tt)
         self.nbl_override = 0       # feature blocks per workgroup of the GEMMs (0 = pick from tokens)
@@ -468,6 +470,82 @@ class WxA16BitPartitionedGroupMoE:
         return out.reshape(shape)
 
     __call__ = forward
+
+    PRENORM_MAX_TOKENS = 16
+
+    @torch.no_grad()
+    def forward_prenorm(self, hidden_states_prenorm: torch.Tensor, norm_weight: torch.Tensor,
+                        eps: float = 1e-6, residual: torch.Tensor | None = None,
+                        return_normed: bool = False, logits_out: torch.Tensor | None = None):
+        """The layer from the block's pre-norm hidden states for a decode step of at most 16
+        tokens: RMSNorm (out = h * rsqrt(mean(h^2) + eps) * (1 + weight),
+        turboquant_utils/norm_kernels.py:79-117), the router projection with this module's
+        ``gate_weight``, softmax + top-k (quantization/wxa16/bit_partitioned_moe.py:1112-1120) and
+        the rotation of the gate_up input are one launch (dmq_moe_ffn_forward_prenorm); no norm
+        kernel and no router GEMM run in front of the layer.  More tokens take the separate steps
+        (ops.rms_norm, then forward).  Returns the output, or (output, normalized input) with
+        ``return_normed``.  ``logits_out`` (fp16 [tokens, num_experts], optional) receives the
+        router logits."""
+        shape = hidden_states_prenorm.shape
+        h = hidden_states_prenorm.reshape(-1, shape[-1])
+        if not h.is_cuda:
+            raise RuntimeError("dartmoq_hip layers run on the GPU only (no CPU fallback)")
+        if self.gate_weight is None:
+            raise ValueError("forward_prenorm needs the module's gate_weight")
+        orig_dtype = h.dtype
+        tokens = h.shape[0]
+        if tokens == 0:
+            empty = torch.empty(shape, dtype=orig_dtype, device=h.device)
+            return (empty, empty.clone()) if return_normed else empty
+        if tokens > self.PRENORM_MAX_TOKENS:
+            x = ops.rms_norm(h, norm_weight, eps)
+            logits = torch.matmul(x, self.gate_weight.t().to(x.dtype))
+            if logits_out is not None:
+                logits_out.copy_(logits)
+            out = self.forward(x.reshape(shape), router_logits=logits, residual=residual)
+            return (out, x.reshape(shape)) if return_normed else out
+        if h.dtype != torch.float16:
+            h = h.half()
+        h = h.contiguous()
+        if norm_weight.dtype not in (torch.float16, torch.float32):
+            norm_weight = norm_weight.float()
+        norm_weight = norm_weight.to(h.device).contiguous()
+        if self._gate_f16 is None:
+            self._gate_f16 = self.gate_weight.to(device=h.device, dtype=torch.float16).contiguous()
+            self._prenorm_state = torch.zeros(64, dtype=torch.int32, device=h.device)
+        router = RouterArgs()
+        router.renorm = int(self.renormalize)
+        if self.n_shared:
+            router.shared_gate_row = self.shared_gate_row.data_ptr()
+            router.n_shared = self.n_shared
+        x_norm = torch.empty_like(h) if return_normed else None
+        pre = PrenormArgs()
+        pre.norm_weight = norm_weight.data_ptr()
+        pre.norm_weight_fp32 = int(norm_weight.dtype == torch.float32)
+        pre.eps = float(eps)
+        pre.gate_weight = self._gate_f16.data_ptr()
+        pre.state = self._prenorm_state.data_ptr()
+        pre.x_norm_out = None if x_norm is None else x_norm.data_ptr()
+        if logits_out is not None:
+            if (logits_out.dtype != torch.float16 or not logits_out.is_contiguous()
+                    or tuple(logits_out.shape) != (tokens, self.num_experts)):
+                raise ValueError("logits_out must be a contiguous fp16 [tokens, num_experts] tensor")
+            pre.logits_out = logits_out.data_ptr()
+        desc = self._descriptor()[0]
+        ws = self._get_workspace(tokens)
+        out = torch.empty_like(h)
+        add = None if residual is None else residual.reshape(-1, shape[-1]).half().contiguous()
+        stream = ctypes.c_void_p(torch.cuda.current_stream(h.device).cuda_stream)
+        check(load().dmq_moe_ffn_forward_prenorm(
+            ctypes.byref(desc), ctypes.byref(router), ctypes.byref(pre), h.data_ptr(), tokens,
+            None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
+            int(self.tt_override), int(self.ks_override), int(self.nbl_override), None, None, stream),
+            "moe_ffn_forward_prenorm")
+        if orig_dtype != torch.float16:
+            out = out.to(orig_dtype)
+            x_norm = None if x_norm is None else x_norm.to(orig_dtype)
+        out = out.reshape(shape)
+        return (out, x_norm.reshape(shape)) if return_normed else out
 
     # ------------------------------------------------------------------ accounting
     def weight_bytes_per_expert(self, bit: int) -> int:

@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 18). */
+/* Library / build identification: returns the ABI version (currently 20). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -481,6 +481,37 @@ int dmq_moe_ffn_forward_routed(const dmq_layer_desc* layer, const dmq_router_arg
                                const void* x, int tokens, const void* add_f16, void* out,
                                void* workspace, size_t workspace_bytes, int tt, int ks, int nbl,
                                void* const* stage_events, void* aux_out, void* stream);
+
+/* What dmq_moe_ffn_forward_prenorm needs on top of the layer: the RMSNorm in front of the block
+ * (turboquant_utils/norm_kernels.py:79-117: x = h * rsqrt(mean(h^2) + eps) * (1 + weight), fp32
+ * arithmetic, one rounding to fp16) and the router projection (the `gate` Linear of
+ * quantization/wxa16/bit_partitioned_moe.py:1112-1120). */
+typedef struct {
+  const void* norm_weight;      /* [hidden] fp16 or fp32 */
+  int norm_weight_fp32;
+  float eps;
+  const void* gate_weight;      /* fp16 [experts - n_shared, hidden], row-major */
+  void* state;                  /* device int32[1], zero before the first call; every call leaves it
+                                   zero.  Calls that overlap on the GPU need separate words. */
+  void* x_norm_out;             /* optional fp16 [tokens, hidden]: the normalized rows (same bits as
+                                   dmq_rms_norm) */
+  void* logits_out;             /* optional fp16 [tokens, experts - n_shared]: the router logits the
+                                   top-k was taken from */
+} dmq_prenorm_args;
+
+/* dmq_moe_ffn_forward_routed for a decode step of at most 16 tokens that starts from the block's
+ * pre-norm input h (fp16 [tokens, hidden]): the first launch computes the RMSNorm, the router
+ * logits (fp32 accumulation, rounded to fp16 like an fp16 Linear), softmax + top-k and, for up to
+ * 4 tokens, the routing step, next to the rotation of the gate_up input, which normalizes its
+ * rows itself.  No norm launch, no router GEMM.  router carries renorm, n_shared and
+ * shared_gate_row only (logits / topk_* must be NULL).  More than 16 tokens, more than 1024
+ * routed experts, experts % 4 != 0 or a sub-expert layer return DMQ_ERR_LIMIT: such callers run
+ * dmq_rms_norm, their router and dmq_moe_ffn_forward_routed. */
+int dmq_moe_ffn_forward_prenorm(const dmq_layer_desc* layer, const dmq_router_args* router,
+                                const dmq_prenorm_args* pre, const void* h, int tokens,
+                                const void* add_f16, void* out, void* workspace,
+                                size_t workspace_bytes, int tt, int ks, int nbl,
+                                void* const* stage_events, void* aux_out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/dartmoq_hip.h but not exported"
     assert set(declared) == set(_lib.PROTOTYPES), "ctypes prototypes and header disagree"
-    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 19
+    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 20
     assert lib.dmq_status_string(0) == b"ok"
     assert b"bit width" in lib.dmq_status_string(1)
 
@@ -269,7 +269,8 @@ def test_ctypes_structs_match_the_header_layout(tmp_path):
         pytest.skip("no C compiler")
     pairs = [("dmq_gemm_pool", _lib.GemmPool), ("dmq_gemm_args", _lib.GemmArgs),
              ("dmq_pool_desc", _lib.PoolDesc), ("dmq_linear_desc", _lib.LinearDesc),
-             ("dmq_layer_desc", _lib.LayerDesc), ("dmq_router_args", _lib.RouterArgs)]
+             ("dmq_layer_desc", _lib.LayerDesc), ("dmq_router_args", _lib.RouterArgs),
+             ("dmq_prenorm_args", _lib.PrenormArgs)]
     lines = ['#include "dartmoq_hip.h"', "#include <stdio.h>", "#include <stddef.h>", "int main(void) {"]
     for cname, cls in pairs:
         last = cls._fields_[-1][0]

@@ -240,6 +240,56 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     }, roof, roof_down
 
 
+def measure_prenorm(mods, tokens, steps, warmup, seed, variants=64):
+    """A decode step that starts from the block's pre-norm hidden states: RMSNorm, router
+    projection (randn * 0.02 gate weight: near-uniform routing) and top-k inside the layer's
+    first launch (`forward_prenorm`) against the same step as three pieces (norm kernel, router
+    GEMM by torch, `forward` from logits).  The steps cycle through the weight copies and through
+    `variants` different hidden states, so consecutive uses of a weight are a full cycle apart."""
+    import torch
+    from dartmoq_hip import ops
+    mod = mods[0]
+    hdim, e = mod.hidden_size, mod.num_experts
+    g = torch.Generator().manual_seed(seed + 31)
+    wn = (torch.randn(hdim, generator=g) * 0.1).half().cuda()
+    wg = (torch.randn(e, hdim, generator=g) * 0.02).half().cuda()
+    hs = [(torch.randn(tokens, hdim, generator=g) * 2.0).half().cuda() for _ in range(variants)]
+    for m in mods:
+        m.gate_weight = wg
+        m._gate_f16 = None
+    n, v = len(mods), len(hs)
+
+    def fused(s):
+        return mods[s % n].forward_prenorm(hs[s % v], wn, 1e-6, fused=True)
+
+    def separate(s):
+        x = ops.rms_norm(hs[s % v], wn, 1e-6)
+        return mods[s % n].forward(x, router_logits=torch.matmul(x, wg.t()))
+
+    res = {"tokens": tokens, "hidden_state_variants": variants, "weight_copies_rotated": n}
+    same = all(torch.equal(fused(s), separate(s)) for s in range(3))
+    for name, fn in (("fused", fused), ("separate", separate)):
+        t0 = time.perf_counter()
+        s = 0
+        while time.perf_counter() - t0 < PRELUDE_S / 2:
+            for _ in range(20):
+                fn(s)
+                s += 1
+            torch.cuda.synchronize()
+        for s in range(warmup):
+            fn(s)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for s in range(steps):
+            fn(s)
+        torch.cuda.synchronize()
+        res[f"{name}_ms_per_step"] = (time.perf_counter() - t0) / steps * 1e3
+    res["launches_fused"] = "norm + router + top-k (+ routing up to 4 tokens) + rotation, [routing], gate_up, down, combine"
+    res["launches_separate"] = "norm, router GEMM (torch), top-k + rotation, [routing], gate_up, down, combine"
+    res["outputs_equal_on_first_3_steps"] = bool(same)
+    return res
+
+
 def measured_traffic(config, mode, tokens):
     """HBM bytes per launch of the dominant kernel from the committed counter runs
     (profiles/gate_up_hbm_traffic.json: FETCH_SIZE + WRITE_SIZE, calibrated on a copy of known
@@ -378,6 +428,9 @@ def main():
     ap.add_argument("--modes", type=str, default="2:wxa8:2048/64,4:wxfp8:2048/64,4:wxfp4:2048/64,3:wxa8:64/8/1",
                     help='extra entries of the "modes" array, "config:mode:tokens[/tokens...]" comma '
                          'separated ("" for none)')
+    ap.add_argument("--prenorm", type=str, default="1,8",
+                    help='token counts of the "prenorm" entries (decode steps that start from pre-norm '
+                         'hidden states; "" for none)')
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch dmq_finalize_kernel on 64 Mi fp32 elements (256 MiB read, "
                          "128 MiB written): the known-size kernel that calibrates FETCH_SIZE / "
@@ -452,6 +505,9 @@ def main():
         res["roofline"] = r
         res["roofline_down"] = rd
         sweep.append(res)
+    prenorm = []
+    for t in [int(v) for v in args.prenorm.split(",") if v]:
+        prenorm.append(measure_prenorm(mods, t, args.steps, args.warmup, args.seed))
     del mods
 
     # the activation-quantized modes on the configurations BASELINE names for them
@@ -516,6 +572,7 @@ def main():
         "roofline_down": roof_down,
         "cpu_baseline": cpu,
         "sweep": sweep,
+        "prenorm": prenorm,
         "modes": mode_results,
         "clock_prelude_s": PRELUDE_S,
     }

@@ -3,6 +3,14 @@
 #pragma once
 #include "params.h"
 
+// acc + f * f as one fp32 FMA.  The value passes through an empty asm so that the compiler cannot
+// merge neighbouring squares into a packed dot product in one caller and not in another: every
+// user of these helpers adds the same squares with the same roundings.
+__device__ __forceinline__ float dmq_sq_acc(float f, float acc) {
+  asm volatile("" : "+v"(f));
+  return __builtin_fmaf(f, f, acc);
+}
+
 // Sum of squares of a row of n values (n % 8 == 0) by one wave: lane l takes the 8-value pieces
 // l, l + 64, ... in order, then the lanes are folded pairwise (xor 1, 2, ... 32).  Uniform result.
 template <typename T, typename F>
@@ -12,7 +20,7 @@ __device__ __forceinline__ float dmq_row_sumsq(const T* xr, int n, int lane, F t
     const uint4_t raw = *(const uint4_t*)(xr + c);
     const T* v = (const T*)&raw;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { const float f = to_f32(v[i]); sumsq = __builtin_fmaf(f, f, sumsq); }
+    for (int i = 0; i < 8; ++i) sumsq = dmq_sq_acc(to_f32(v[i]), sumsq);
   }
 #pragma unroll
   for (int m = 1; m < 64; m <<= 1) sumsq += __shfl_xor(sumsq, m, 64);
@@ -25,7 +33,10 @@ __device__ __forceinline__ float dmq_rstd(float sumsq, int n, float eps) {
 
 // One normalized value: h * rstd * (1 + w), rounded once by the caller.
 __device__ __forceinline__ float dmq_norm_value(float h, float rstd, float w) {
-  return h * rstd * (1.0f + w);
+  float t = h * rstd;
+  float u = 1.0f + w;
+  asm volatile("" : "+v"(t), "+v"(u));               // two roundings, then the product: in every caller
+  return t * u;
 }
 
 // The same sum for four fp16 rows at once (their pieces are requested together, NCH pieces per
@@ -50,8 +61,7 @@ __device__ __forceinline__ void dmq_rows_sumsq4(const __half* const (&xr)[4], in
       const __half* v = (const __half*)&raw[r][ch];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const float f = in ? __half2float(v[i]) : 0.f;
-        sumsq = __builtin_fmaf(f, f, sumsq);
+        sumsq = dmq_sq_acc(in ? __half2float(v[i]) : 0.f, sumsq);
       }
     }
 #pragma unroll

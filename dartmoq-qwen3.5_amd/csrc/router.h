@@ -24,6 +24,61 @@ struct RouterParams {
   TopkParams tp;                 // what the last workgroup runs (logits taken from LDS)
 };
 
+// The logits of 16 experts x 16 tokens: wave w contracts the w-th quarter of the hidden dimension
+// in NS steps of 32 (NS = 0: any length, loads inside the loop).  With NS known every load of the
+// wave for router rows and pre-norm rows is requested before the row statistics are
+// computed, so the whole contraction waits on memory once.
+template <int NS>
+__device__ __forceinline__ float4_t dmq_router_logits(const RouterParams& rp, int block, float* s_rstd) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int l16 = lane & 15;
+  const int q = lane >> 4;
+  const int e0 = block * 16;
+  const int erow = min(e0 + l16, rp.experts - 1);
+  const int trow = min(l16, rp.tokens - 1);
+  const int kq = rp.hidden / 4;
+  const int col0 = wave * kq + 8 * q;
+  const __half* wp = rp.gate_w + (long)erow * rp.hidden + col0;
+  const __half* hp = rp.h + (long)trow * rp.h_stride + col0;
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  auto step = [&](int k, uint4_t a, uint4_t raw, const float (&w8)[8], float rstd) {
+    const uint4_t xn = dmq_norm8(raw, rstd, w8);
+    if (block == 0 && rp.x_norm_out && l16 < rp.tokens)
+      *(uint4_t*)(rp.x_norm_out + (long)l16 * rp.hidden + col0 + k) = xn;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                 __builtin_bit_cast(half8_t, xn), acc, 0, 0, 0);
+  };
+  if constexpr (NS > 0) {
+    uint4_t a[NS], raw[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      a[s] = *(const uint4_t*)(wp + 32 * s);
+      raw[s] = *(const uint4_t*)(hp + 32 * s);
+    }
+    dmq_wg_rstd(rp.h, rp.h_stride, 0, rp.tokens, rp.hidden, rp.pn.eps, s_rstd);
+    const float rstd = s_rstd[trow];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      float w8[8];
+      dmq_norm_weights8(rp.pn, col0 + 32 * s, w8);
+      step(32 * s, a[s], raw[s], w8, rstd);
+    }
+  } else {
+    dmq_wg_rstd(rp.h, rp.h_stride, 0, rp.tokens, rp.hidden, rp.pn.eps, s_rstd);
+    const float rstd = s_rstd[trow];
+#pragma unroll 4
+    for (int k = 0; k < kq; k += 32) {
+      const uint4_t a = *(const uint4_t*)(wp + k);
+      const uint4_t raw = *(const uint4_t*)(hp + k);
+      float w8[8];
+      dmq_norm_weights8(rp.pn, col0 + k, w8);
+      step(k, a, raw, w8, rstd);
+    }
+  }
+  return acc;
+}
+
 // `lds`: 32 KiB of LDS the caller does not need while this runs.
 __device__ __forceinline__ void dmq_router_wg(const RouterParams& rp, const int block, uint8_t* lds) {
   using u64 = unsigned long long;
@@ -33,29 +88,11 @@ __device__ __forceinline__ void dmq_router_wg(const RouterParams& rp, const int 
   const int wave = threadIdx.x >> 6;
   const int l16 = lane & 15;
   const int q = lane >> 4;
-  dmq_wg_rstd(rp.h, rp.h_stride, 0, rp.tokens, rp.hidden, rp.pn.eps, s_rstd);
-
-  // logits of 16 experts x 16 tokens: wave w contracts the w-th quarter of the hidden dimension
   const int e0 = block * 16;
-  const int erow = min(e0 + l16, rp.experts - 1);
-  const int trow = min(l16, rp.tokens - 1);
-  const float rstd = s_rstd[trow];
-  const int kq = rp.hidden / 4;
-  const __half* wp = rp.gate_w + (long)erow * rp.hidden + wave * kq + 8 * q;
-  const __half* hp = rp.h + (long)trow * rp.h_stride + wave * kq + 8 * q;
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int k = 0; k < kq; k += 32) {
-    const uint4_t a = *(const uint4_t*)(wp + k);
-    const uint4_t raw = *(const uint4_t*)(hp + k);
-    float w8[8];
-    dmq_norm_weights8(rp.pn, wave * kq + 8 * q + k, w8);
-    const uint4_t xn = dmq_norm8(raw, rstd, w8);
-    if (block == 0 && rp.x_norm_out && l16 < rp.tokens)
-      *(uint4_t*)(rp.x_norm_out + (long)l16 * rp.hidden + wave * kq + 8 * q + k) = xn;
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
-                                                 __builtin_bit_cast(half8_t, xn), acc, 0, 0, 0);
-  }
+  float4_t acc;
+  if (rp.hidden == 2048) acc = dmq_router_logits<16>(rp, block, s_rstd);
+  else if (rp.hidden == 3072) acc = dmq_router_logits<24>(rp, block, s_rstd);
+  else acc = dmq_router_logits<0>(rp, block, s_rstd);
   float* part = (float*)lds;                           // [4 waves][64 lanes][4]
   *(float4_t*)(part + (wave * 64 + lane) * 4) = acc;
   __syncthreads();

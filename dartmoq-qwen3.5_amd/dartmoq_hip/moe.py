@@ -471,19 +471,25 @@ class WxA16BitPartitionedGroupMoE:
 
     __call__ = forward
 
-    PRENORM_MAX_TOKENS = 16
+    PRENORM_MAX_TOKENS = 16      # what dmq_moe_ffn_forward_prenorm takes
+    PRENORM_AUTO_TOKENS = 8      # up to here forward_prenorm picks it by itself (measured: H=2048,
+                                 # 256 experts, top-8: 1 token 57.7 -> 39.7 us, 4 tokens 54.6 -> 46.8,
+                                 # 8 tokens 61.7 -> 60.1, 16 tokens 81.8 -> 86.3: the last router
+                                 # workgroup takes the top-k of four tokens at a time)
 
     @torch.no_grad()
     def forward_prenorm(self, hidden_states_prenorm: torch.Tensor, norm_weight: torch.Tensor,
                         eps: float = 1e-6, residual: torch.Tensor | None = None,
-                        return_normed: bool = False, logits_out: torch.Tensor | None = None):
+                        return_normed: bool = False, logits_out: torch.Tensor | None = None,
+                        fused: bool | None = None):
         """The layer from the block's pre-norm hidden states for a decode step of at most 16
         tokens: RMSNorm (out = h * rsqrt(mean(h^2) + eps) * (1 + weight),
         turboquant_utils/norm_kernels.py:79-117), the router projection with this module's
         ``gate_weight``, softmax + top-k (quantization/wxa16/bit_partitioned_moe.py:1112-1120) and
         the rotation of the gate_up input are one launch (dmq_moe_ffn_forward_prenorm); no norm
-        kernel and no router GEMM run in front of the layer.  More tokens take the separate steps
-        (ops.rms_norm, then forward).  Returns the output, or (output, normalized input) with
+        kernel and no router GEMM run in front of the layer.  ``fused`` None picks that launch up
+        to 8 tokens, True up to 16; more tokens (or False) take the separate steps (ops.rms_norm,
+        the router GEMM, forward).  Returns the output, or (output, normalized input) with
         ``return_normed``.  ``logits_out`` (fp16 [tokens, num_experts], optional) receives the
         router logits."""
         shape = hidden_states_prenorm.shape
@@ -497,7 +503,8 @@ class WxA16BitPartitionedGroupMoE:
         if tokens == 0:
             empty = torch.empty(shape, dtype=orig_dtype, device=h.device)
             return (empty, empty.clone()) if return_normed else empty
-        if tokens > self.PRENORM_MAX_TOKENS:
+        limit = self.PRENORM_AUTO_TOKENS if fused is None else (self.PRENORM_MAX_TOKENS if fused else 0)
+        if tokens > limit:
             x = ops.rms_norm(h, norm_weight, eps)
             logits = torch.matmul(x, self.gate_weight.t().to(x.dtype))
             if logits_out is not None:

@@ -38,7 +38,7 @@ def _run(layer, mode, tokens, seed, weight_dtype=torch.float16):
     mod = make_module(layer, mode)
     mod.gate_weight = wg.cuda()
     logits = torch.empty(tokens, layer.num_experts, dtype=torch.float16, device="cuda")
-    out, xn = mod.forward_prenorm(h.cuda(), wn.cuda(), EPS, return_normed=True, logits_out=logits)
+    out, xn = mod.forward_prenorm(h.cuda(), wn.cuda(), EPS, return_normed=True, logits_out=logits, fused=True)
     torch.cuda.synchronize()
     # the stand-alone kernel's bits
     xk = ops.rms_norm(h.cuda(), wn.cuda(), EPS)

@@ -419,6 +419,11 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.home_filter = a->width_filter != 0 ? a->home_filter : -1;
   p.accumulate = (a->epi == DMQ_EPI_SCATTER && a->accumulate) ? 1 : 0;
   p.wsplit = wsplit;
+  p.split_items = 0;
+  if (wsplit > 1 && a->k_split_items > 0) {
+    if (a->spread || subs > 1 || rows_kernel) return DMQ_ERR_MODE;
+    p.split_items = a->k_split_items < a->max_items ? a->k_split_items : a->max_items;
+  }
   p.spread = a->spread != 0;
   p.subs = subs;
   p.split_rows = a->split_rows;
@@ -463,6 +468,7 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     // several blocks per workgroup: the tail of every XCD's share is cut into single blocks
     p.tail_slots = (nbl > 1 && wsplit == 1 && p.n_blocks % nbl == 0) ? DMQ_TAIL_SLOTS : 0;
     L.p = p;
+    if (spread_l) L.p.split_items = 0;                 // items dealt out: every item shares K
     L.ks = lks;
     L.wide = both_widths ? 2 : wide;
     long work;
@@ -475,6 +481,12 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
                                   : (long)a->max_items * subs;
       work = units * ((p.n_blocks + nbl - 1) / nbl) * wsplit;
       work = (work + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;    // every XCD gets the same number of slots
+      if (L.p.split_items > 0) {
+        // the shared items in front (their bound), then one workgroup per block for the rest
+        const long head = ((long)L.p.split_items * p.n_blocks * wsplit + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;
+        const long bulk = ((long)a->max_items * p.n_blocks + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;
+        work = head + bulk;
+      }
     }
     if (work > 0x7fffffffL) return DMQ_ERR_LIMIT;
     L.grid = (int)work;
@@ -890,6 +902,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   }
   if (tt == DMQ_ROWS_TT && !rows_ok) tt = 4;
   if (tt != 1 && tt != 2 && tt != 4 && tt != DMQ_ROWS_TT) return DMQ_ERR_MODE;
+  const bool ks_auto = ks == 0;
   if (ks == 0) {
     ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
     // an 8-bit pool on the fp16 path (a shared expert with a 256-entry table) makes few, long work
@@ -918,6 +931,30 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     ks = 1;
   }
   const int wsplit_eff = sub ? 1 : wsplit;
+  // Few long work items next to many short ones: with 16-row tiles every workgroup of the gate_up
+  // launch is resident from the start, so the launch ends with its slowest item.  The items of a
+  // pool that holds a small share of the experts (the 4-bit and 1-bit pools of a 2 bpw layer: twice
+  // the bytes per step, or a table that takes longer to build) are therefore shared by four
+  // workgroups each while the bulk keeps one per block (configs[3] wxa8 64 tokens: the 4-bit
+  // item ran 47 us, the 1-bit one 40, the median 2-bit one 30).
+  bool rare_pool[DMQ_MAX_POOLS] = {false, false, false, false};
+  int n_rare = 0, wsplit_launch = wsplit_eff;
+  long rare_items = 0;                                   // bound on the work items of those pools
+  if (ks_auto && wsplit_eff == 1 && !sub && tt == 1 && ks == 1 && (long)tokens * K <= DMQ_SPLIT_MAX_ROWS &&
+      tokens <= DMQ_HOIST_ALL_TOKENS) {
+    const int s = (H / DMQ_GS) % 4 == 0 ? 4 : ((H / DMQ_GS) % 2 == 0 ? 2 : 1);
+    for (int i = 0; i < P; ++i) {
+      const long members = layer->pool[i].n_gate_up / (2L * I);
+      rare_pool[i] = members * 8 <= E;
+      if (rare_pool[i]) {
+        ++n_rare;
+        const long by_tokens = members * ((tokens + 15) / 16), by_rows = members + (long)tokens * K / 16;
+        rare_items += by_tokens < by_rows ? by_tokens : by_rows;
+      }
+    }
+    if (s > 1 && n_rare > 0 && n_rare < P) wsplit_launch = s;
+    else { n_rare = 0; for (int i = 0; i < P; ++i) rare_pool[i] = false; }
+  }
   if (tt == DMQ_ROWS_TT ? ks != 1 : !dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   const bool nbl_auto = nbl <= 0;
   if (nbl_auto) nbl = pick_nbl((long)tokens * K, tt > 4 ? 4 : tt);
@@ -1024,8 +1061,11 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   {
     int n = 0;
     for (int i = 0; i < P; ++i) if (!whole_batch[i]) pool_order[n++] = i;
+    // (every pool rotates by token when some pools' items share K, see rare_pool: the prefix then
+    // counts the items of those pools instead)
+    if (n_rare > 0) for (int i = 0; i < P; ++i) if (rare_pool[i]) pool_order[n++] = i;
     lead_pools = n;
-    for (int i = 0; i < P; ++i) if (whole_batch[i]) pool_order[n++] = i;
+    for (int i = 0; i < P; ++i) if (whole_batch[i] && !rare_pool[i]) pool_order[n++] = i;
     // Among the whole-batch pools the ones with the longest work items go first (the order of the
     // list is the order in which workgroups get their slots): 4-bit weights cost twice the look-ups
     // of 2-bit ones, fp16 activations more than quantized ones.  A 4-bit fp16 shared expert at the
@@ -1120,7 +1160,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
         dp.items = w.items; dp.n_items = w.n_items; dp.counts = w.counts;
         dp.sorted_tokens = w.sorted_tokens; dp.sorted_weights = w.sorted_weights;
         dp.sorted_rows = w.sorted_rows;
-        if (wsplit_eff > 1) { dp.clear_words = w.split_counter; dp.clear_count = w.split_counters; }
+        if (wsplit_launch > 1) { dp.clear_words = w.split_counter; dp.clear_count = w.split_counters; }
         direct_done = true;
       }
       if (pre) {
@@ -1163,7 +1203,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
       rr.counts = w.counts; rr.n_items = w.n_items; rr.items = w.items;
       rr.sorted_tokens = w.sorted_tokens; rr.sorted_weights = w.sorted_weights;
       rr.sorted_rows = w.sorted_rows;
-      if (wsplit_eff > 1) { rr.clear_words = w.split_counter; rr.clear_count = w.split_counters; }
+      if (wsplit_launch > 1) { rr.clear_words = w.split_counter; rr.clear_count = w.split_counters; }
       rc = dmq_route_rank_launch(rr, st);
     } else if (route_small) {
       RouteSmallParams sp{};
@@ -1183,7 +1223,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
       plan.lead_pools = lead_pools;
       sp.sorted_tokens = w.sorted_tokens; sp.sorted_weights = w.sorted_weights;
       sp.sorted_rows = w.sorted_rows;
-      if (wsplit_eff > 1) { sp.clear_words = w.split_counter; sp.clear_count = w.split_counters; }
+      if (wsplit_launch > 1) { sp.clear_words = w.split_counter; sp.clear_count = w.split_counters; }
       rc = dmq_route_small_launch(sp, st);
     } else {
       const void* tk_idx = router->topk_idx;
@@ -1203,7 +1243,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
                                  w.items, w.sort_scratch, w.sort_scratch_bytes, pool_order,
                                  lead_pools, stream, tt == DMQ_ROWS_TT ? w.rows_queue : nullptr,
                                  2 * DMQ_ROWS_QUEUE_WORDS);
-      if (!rc && wsplit_eff > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
+      if (!rc && wsplit_launch > 1) rc = dmq_fill_zero(w.split_counter, (long)w.split_counters * 4, stream);
     }
   }
   if (rc) return rc;
@@ -1254,8 +1294,9 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     g.post_out = actq_of(mode); g.post_row_bytes = (long)I * 2;
     g.post_scale = actq_scale_of(mode); g.post_scale_stride = scale_stride_for(mode, I);
     g.rows_queue = w.rows_queue;
-    if (wsplit_eff > 1) {
-      g.k_split = wsplit_eff; g.split_rows = w.split_rows;
+    if (wsplit_launch > 1) {
+      g.k_split = wsplit_launch; g.split_rows = w.split_rows;
+      if (n_rare > 0) g.k_split_items = (int)(rare_items < w.max_items ? rare_items : w.max_items);
       g.split_partial = w.split_partial; g.split_counter = w.split_counter;
     }
     if (!sub) {

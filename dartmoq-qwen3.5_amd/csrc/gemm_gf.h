@@ -97,6 +97,7 @@ struct GemmParams {
   int home_filter;
   int accumulate;
   int wsplit;                  // 1, 2, 4, 8 or 16
+  int split_items;             // > 0: only the first min(n_items[1], split_items) items share K
   int spread;                  // work item i on XCD i % 8 instead of a contiguous share per XCD (nbl == 1)
   int split_rows;              // rows of one plane
   float* split_partial;        // fp32 [wsplit, split_rows, 2 * n_out (SiLU) or n_out (store)]
@@ -225,6 +226,9 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
                                               int token_count, int slice_start, int post_slice,
                                               int ttile, int nb, int nbc, int split, int* ticket,
                                               int* wg_flag, int col0) {
+  // split: index of this workgroup among those sharing the K range (low byte) and their number
+  const int nsplit_in = split >> 8;
+  split &= 0xff;
   using T = ModeTraits<MODE>;
   using acc_t = typename T::acc_t;
   using GG = GemmGeom<MODE, NT, TT, KS>;
@@ -950,7 +954,7 @@ __device__ __forceinline__ void dmq_gemm_body(const GemmParams& p, const PoolW& 
     static_assert(D % 2 == 0, "the LDS slot of a ring entry is fixed by its parity");
     uint32_t pkb[D][NT][WW];
     Staged srb[D];
-    const int nsplit = XSPLIT ? p.wsplit : 1;
+    const int nsplit = XSPLIT ? nsplit_in : 1;
     const int G = XSPLIT ? p.groups / nsplit : g_hi;   // groups this workgroup contracts
     const int g_first = XSPLIT ? split * G : 0;
     const int steps = nbc * G;
@@ -1100,7 +1104,33 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   __shared__ int wg_flag;
   const int wsplit = XSPLIT ? p.wsplit : 1;
   int item, nb, nbc, split = 0;
-  if (p.tail_slots > 0) {
+  int ns = wsplit;                                       // workgroups sharing this one's K range
+  if (XSPLIT && p.split_items > 0) {
+    // The list begins with a few long items (their number: n_items[1], at most split_items): those
+    // share K between wsplit workgroups and take the first workgroups of the launch, every other
+    // item gets one workgroup per block, each XCD a contiguous range of them as below.
+    const int nsp = min(p.n_items[1], p.split_items);
+    const int wpi = p.n_blocks * wsplit;                 // workgroups of a shared item
+    const int head = (p.split_items * wpi + DMQ_XCDS - 1) / DMQ_XCDS * DMQ_XCDS;
+    if ((int)blockIdx.x < head) {
+      item = blockIdx.x / wpi;
+      if (item >= nsp) return;
+      const int sub = blockIdx.x - item * wpi;
+      split = sub % wsplit;
+      nb = sub / wsplit;
+    } else {
+      const int b = blockIdx.x - head;
+      const int total = (p.n_items[0] - nsp) * p.n_blocks;
+      const int per_xcd = (total + DMQ_XCDS - 1) / DMQ_XCDS;
+      const int slot = b / DMQ_XCDS;
+      const int unit = (b % DMQ_XCDS) * per_xcd + slot;
+      if (slot >= per_xcd || unit >= total) return;
+      item = nsp + unit / p.n_blocks;
+      nb = unit % p.n_blocks;
+      ns = 1;
+    }
+    nbc = 1;
+  } else if (p.tail_slots > 0) {
     // Workgroups are dispatched in index order as slots free up, so the order of the list is the
     // schedule: the head of an XCD's share goes nbl blocks per workgroup (loads stay in flight
     // across blocks, one table build for several blocks), its last tail_slots blocks one per
@@ -1171,23 +1201,23 @@ void dmq_gemm_gf_kernel(GemmParams p) {
   auto run = [&](auto mode_tag) __attribute__((always_inline)) {
     constexpr int M = decltype(mode_tag)::value;
     if constexpr (M == DMQ_MODE_FP4) {
-      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+      dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split | (ns << 8), ticket, &wg_flag, col0);
       return;
     }
     if constexpr (M != DMQ_MODE_FP4 && WIDE != 0) {
       if (WIDE == 1 || pw.bit == 8) {                    // uniform over the workgroup
         if (M == DMQ_MODE_A8 && pw.lut == nullptr)       // uniform codebook: no table
-          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, M == DMQ_MODE_A8, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split | (ns << 8), ticket, &wg_flag, col0);
         else
-          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0);
+          dmq_gemm_body<M, 8, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split | (ns << 8), ticket, &wg_flag, col0);
         return;
       }
     }
     if constexpr (M != DMQ_MODE_FP4 && WIDE != 1) {
       switch (pw.bit) {
-        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
-        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split, ticket, &wg_flag, col0); break;
+        case 1: dmq_gemm_body<M, 1, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split | (ns << 8), ticket, &wg_flag, col0); break;
+        case 2: dmq_gemm_body<M, 2, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split | (ns << 8), ticket, &wg_flag, col0); break;
+        default: dmq_gemm_body<M, 4, NT, TT, EPI, KS, DBG, false, ROW, ROOMY>(p, pw, tbl, smem2, smem_post, token_start, token_count, slice_start, post_slice, ttile, nb, nbc, split | (ns << 8), ticket, &wg_flag, col0); break;
       }
     }
   };

@@ -321,6 +321,13 @@ typedef struct {
    * device memory, zero before the launch; the launch leaves them zero.  Same results, bit for bit,
    * as tt == 2 and tt == 4. */
   void* rows_queue;
+  /* With k_split > 1 and k_split_items > 0: only the first min(n_items[1], k_split_items) work
+   * items of the list share their K range between k_split workgroups; the rest run one workgroup
+   * per feature block.  For lists that begin with a few long items (pools with a wider index or a
+   * table that takes longer to build, ordered first by dmq_route_permute's pool order, their
+   * number written to n_items[1]): the launch then ends with the bulk instead of with them.
+   * k_split_items bounds that number from the host; not with spread or item_tile_rows. */
+  int k_split_items;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

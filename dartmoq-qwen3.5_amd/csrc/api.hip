@@ -758,7 +758,14 @@ static int pick_tt(int tokens, int top_k, int experts, int weights) {
   // 12 rows per expert on (-5 % at 24, -6 % at 32, -3 % at 64).  The down GEMM keeps 32-row tiles
   // on those items (down_tt below).
   const long min4 = weights == 2 ? 10 : (weights == 1 ? 40 : DMQ_TT4_MIN_AVG);
-  if (avg <= (weights == 1 ? 12 : 8)) return 1;   // 4-bit look-up layers: 16-row tiles 3 % ahead at 12 rows per expert
+  // 16-row tiles: 4-bit look-up layers (uniform routing) keep them up to 12 rows per expert (3 %
+  // ahead there), FP4 up to 8.  Layers of narrow pools are measured under Zipf routing, where the
+  // hot experts fill several 16-row tiles long before the average does, each of them streaming
+  // the expert's weights again: 32-row tiles from 2 rows per expert on (H = 2048, I = 512, 256
+  // experts, top-8, whole forward: 64 tokens 73.2 -> 69.3 us, 128 tokens equal, 256 tokens
+  // 92.8 -> 86.2; H = 3072, I = 1024 with a shared expert, wxa8: 64 tokens 108 -> 102, 128 tokens
+  // 133 -> 128, 256 tokens 183 -> 164; at 1 row per expert 16-row tiles are 2-7 % ahead).
+  if (weights == 0 ? avg < 2 : avg <= (weights == 1 ? 12 : 8)) return 1;
   return avg <= min4 ? 2 : 4;
 }
 

@@ -304,7 +304,7 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
-                 row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, rows_total=None,
+                 row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, k_split_items=0, rows_total=None,
                  item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None, widths_apart=0):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
@@ -374,6 +374,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
             partial = torch.empty((k_split, rows_total, width), dtype=torch.float32, device=dev)
             counter = torch.zeros(n_counters, dtype=torch.int32, device=dev)
         a.k_split, a.split_rows = k_split, rows_total
+        a.k_split_items = int(k_split_items)
         a.split_partial, a.split_counter = partial.data_ptr(), counter.data_ptr()
     check(load().dmq_matmul_merged_gf(ctypes.byref(a), _stream(dev)), "matmul_merged_gf")
     return out

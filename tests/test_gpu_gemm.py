@@ -242,6 +242,61 @@ def test_both_index_widths_in_one_launch_give_the_bits_of_two_launches(mode, roo
                                        atol=2e-3 * one.float().abs().max().item())
 
 
+@pytest.mark.parametrize("mode", [A16, A8])
+def test_k_shared_for_the_leading_items_only(mode):
+    """16-row tiles, a list that begins with the items of a 4-bit pool (n_items[1] of them) followed
+    by those of a 2-bit pool: with k_split_items the leading items share K between four workgroups
+    and give the bits of a launch that shares every item, the others run one workgroup per block
+    and give the bits of a launch that shares nothing."""
+    from dartmoq_hip import ops
+    k, inter = 1024, 256
+    counts0, counts1 = [3, 0, 20], [5, 40, 0, 17, 1]
+    r0, r1 = sum(counts0), sum(counts1)
+    rows = r0 + r1
+    g = torch.Generator().manual_seed(17 + mode)
+    x_rot = torch.randn(rows, k, generator=g) * 0.7
+    pools, infos = [], []
+    act = scale = None
+    for pi, (bit, counts, first_row) in enumerate([(4, counts0, 0), (2, counts1, r0)]):
+        cb = codebook.get_codebook(bit)[0].half()
+        act, scale, _, _, lut, _, _, _, wsb = _mode_inputs(mode, x_rot, cb)
+        idx_gf, norms_gf, _ = _pool(bit, 2 * inter * len(counts), k, 500 + pi)
+        starts = [first_row + sum(counts[:e]) for e in range(len(counts))]
+        info = torch.tensor([(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(len(counts))],
+                            dtype=torch.int32).cuda()
+        infos.append(info)
+        pools.append(dict(w=idx_gf.cuda(), norms=norms_gf.cuda(), lut=lut.cuda(), expert_info=info,
+                          act=act.cuda(), act_scale=None if scale is None else scale.cuda(),
+                          row_index=None, bit=bit, mode=mode, w_scale_byte=wsb))
+    lists = [ops.build_tiles(infos[pi], rows, 16, pool=pi) for pi in range(2)]
+    n = [int(l[0][0]) for l in lists]
+    items = torch.cat([lists[0][1][:n[0]], lists[1][1][:n[1]]]).contiguous()
+    n_items = torch.tensor([n[0] + n[1], n[0], 0, 0], dtype=torch.int32).cuda()
+    common = dict(groups=k // 128, n_out=inter, half_width=inter, slice_is_groups=False, tt=1,
+                  out_stride=inter, act_row_bytes=act.element_size() * k,
+                  act_scale_stride=0 if scale is None else scale.stride(0))
+
+    def run(**kw):
+        out = torch.full((rows, inter), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul_pools(mode, SILU, pools, items, n_items, items.shape[0] + 3, out=out, **common, **kw)
+        torch.cuda.synchronize()
+        assert not torch.isnan(out.float()).any()
+        return out
+
+    none = run()
+    every = run(k_split=4, rows_total=rows)
+    for bound in (n[0], n[0] + 2, 1):
+        lead = run(k_split=4, rows_total=rows, k_split_items=bound)
+        if bound >= n[0]:
+            assert torch.equal(lead[:r0], every[:r0])
+            assert torch.equal(lead[r0:], none[r0:])
+        else:        # a bound below the prefix count: only that many items are shared
+            first = int(items[0, 4])                       # rows of the first item
+            assert torch.equal(lead[:first], every[:first])
+            assert torch.equal(lead[first:], none[first:])
+    torch.testing.assert_close(every.float(), none.float(), rtol=2e-3, atol=2e-3 * none.float().abs().max().item())
+
+
 @pytest.mark.parametrize("mode", [A16, A8, FP8, FP4])
 @pytest.mark.parametrize("bit", [1, 2, 4])
 def test_merged_in_features_down(mode, bit):

@@ -89,25 +89,31 @@ def is_uniform_codebook(codebook: torch.Tensor, rel_tol: float = 1e-2) -> bool:
     return bool((d - d.mean()).abs().max() < rel_tol * mean)
 
 
-def build_int8_lut(codebook: torch.Tensor):
+def build_int8_lut(codebook: torch.Tensor, round_lloyd_max_8bit: bool = False):
     """int8 look-up table and step of a codebook for the int8 path: the rounded table of
-    build_int8_codebook for 1/2/4-bit codebooks; for 8-bit codebooks the identity w = idx - 128
-    with the uniform step, which is what the reference's IDENTITY_CB kernels compute
-    (quantization/wxa8/linear.py:130-159) and needs a uniform codebook (:79-98)."""
+    build_int8_codebook for 1/2/4-bit codebooks; for uniform 8-bit codebooks the identity
+    w = idx - 128 with the uniform step, which is what the reference's IDENTITY_CB kernels compute
+    (quantization/wxa8/linear.py:130-159).  A Lloyd-Max 8-bit codebook is refused for a Linear, as
+    in the reference (:79-98); the bit pools of a MoE layer pass ``round_lloyd_max_8bit``: the
+    reference rounds the codebook of every pool to int8 whatever its width
+    (quantization/wxa8/bit_partitioned_moe.py:78-82), levels near zero merging
+    (triton_kernels_a8.py:539-542)."""
     if codebook.numel() == 256:
-        if not is_uniform_codebook(codebook):
+        if is_uniform_codebook(codebook):
+            q = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8)
+            return q, uniform_codebook_step(codebook)
+        if not round_lloyd_max_8bit:
             raise ValueError("the int8 path takes 8-bit weights only with a uniform codebook")
-        q = (torch.arange(256, dtype=torch.int16) - 128).to(torch.int8)
-        return q, uniform_codebook_step(codebook)
     return build_int8_codebook(codebook)
 
 
-def int8_lut_for_launch(codebook: torch.Tensor, device):
+def int8_lut_for_launch(codebook: torch.Tensor, device, round_lloyd_max_8bit: bool = False):
     """(table or None, step) as the int8 GEMM launches take it: 8-bit uniform codebooks pass no
     table (the kernels compute w = idx - 128 from the index bytes), everything else its rounded
     int8 table on the device."""
-    q, step = build_int8_lut(codebook)
-    return (None if codebook.numel() == 256 else q.to(device)), step
+    q, step = build_int8_lut(codebook, round_lloyd_max_8bit)
+    identity = codebook.numel() == 256 and is_uniform_codebook(codebook)
+    return (None if identity else q.to(device)), step
 
 
 def build_fp8_codebook(codebook: torch.Tensor, n_coarse: int = 512):

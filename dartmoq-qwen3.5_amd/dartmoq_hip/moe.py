@@ -69,8 +69,8 @@ class BitPoolWeights:
         if mode == MODE_A16:
             ctx["gu_lut"], ctx["dn_lut"] = self.gu_codebook, self.dn_codebook
         elif mode == MODE_A8:
-            gq, gstep = hostprep.int8_lut_for_launch(self.gu_codebook, dev)
-            dq, dstep = hostprep.int8_lut_for_launch(self.dn_codebook, dev)
+            gq, gstep = hostprep.int8_lut_for_launch(self.gu_codebook, dev, round_lloyd_max_8bit=True)
+            dq, dstep = hostprep.int8_lut_for_launch(self.dn_codebook, dev, round_lloyd_max_8bit=True)
             ctx.update(gu_lut=gq, dn_lut=dq, gu_extra=gstep, dn_extra=dstep)
         elif mode == MODE_FP8:
             gq, gs_ = hostprep.build_fp8_codebook(self.gu_codebook)

@@ -246,14 +246,20 @@ def sliced_layer(request):
 def test_sub_expert_layer_matches_oracles(sliced_layer, mode, tokens, tt):
     """Experts spread over several bit pools (the reference's --slices layout): the output of an
     expert is the sum over its pools."""
-    if "8" in sliced_layer.pools and mode in ("wxa8", "wxfp4"):
-        pytest.skip("a Lloyd-Max 8-bit pool has no int8 form (int8 takes the uniform 8-bit grid only)")
     x, idx, w, out = _run(sliced_layer, mode, tokens, seed=tokens, tt=tt)
     ideal = moe.quantized_forward(sliced_layer, x, idx, w, mode)
     tight = {"wxa16": 3e-3, "wxa8": 6e-3, "wxfp8": 2e-2, "wxfp4": 6e-2}[mode]
     assert relerr(out, ideal) < tight, (mode, relerr(out, ideal))
     ref = moe.reference_forward(sliced_layer, x, idx, w)
-    assert relerr(out, ref) < MODE_BOUND[mode], (mode, relerr(out, ref))
+    bound = MODE_BOUND[mode]
+    if "8" in sliced_layer.pools and mode in ("wxa8", "wxfp4"):
+        # a Lloyd-Max 8-bit pool on the int8 path: its 256 levels are rounded to the int8 grid like
+        # every pool's codebook (quantization/wxa8/bit_partitioned_moe.py:78-82), which the
+        # reference measures at 0.0128 for such a matrix against 0.00075 in fp16
+        # (triton_kernels_a8.py:539-542); the tight bound above already holds the kernels to that
+        # dataflow
+        bound *= 1.5
+    assert relerr(out, ref) < bound, (mode, relerr(out, ref))
 
 
 @pytest.mark.parametrize("tokens", [1, 3, 40, 200])

@@ -31,7 +31,9 @@ __device__ __forceinline__ float wave_max16x4(float v) {
 
 // One workgroup of the rotation launch (`block` = its index among the rotation workgroups, `mat` =
 // 32 KiB of LDS for the staged matrix).
-template <int MODE, int TT>
+// PN: the rows are pre-norm (RotParams.pn): instances of their own, so that the others keep their
+// registers (the row statistics hold a few dozen loads in flight).
+template <int MODE, int TT, bool PN = false>
 __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int block, uint8_t* mat) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -138,7 +140,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
 #pragma unroll
     for (int t = 0; t < TT; ++t)
       xraw[s][t] = valid[t] ? *(const uint4_t*)(xrow[t] + 32 * s) : (uint4_t){0u, 0u, 0u, 0u};
-  if (TT == 1 && p.pn.on && staged) {
+  if constexpr (PN && TT == 1) if (staged) {
     // pre-norm rows: the workgroup's four waves hold 64 consecutive rows; their rstd is computed
     // by all four waves together (also by those whose tile lies past the last row), then every
     // lane normalizes the pieces it holds
@@ -287,7 +289,7 @@ __device__ __forceinline__ void dmq_rotate_wg(const RotParams& p, const int bloc
 }
 
 // --------------------------------------------------------------------------------------------
-template <int MODE, int TT>
+template <int MODE, int TT, bool PN = false>
 __global__ __launch_bounds__(256)
 void dmq_rotate_kernel(RotParams p) {
   __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
@@ -305,7 +307,7 @@ void dmq_rotate_kernel(RotParams p) {
       *(int4_t*)lp.info = (int4_t){0, lp.rows, 0, lp.n_out};
     }
   }
-  dmq_rotate_wg<MODE, TT>(p, blockIdx.x, mat);
+  dmq_rotate_wg<MODE, TT, PN>(p, blockIdx.x, mat);
 }
 
 // The same launch with the router's top-k in front: workgroups [0, tp.blocks) take four tokens
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(256)
 void dmq_rotate_router_kernel(RotParams p, RouterParams rt) {
   __shared__ __attribute__((aligned(16))) uint8_t mat[DMQ_GS * DMQ_GS * 2];
   if ((int)blockIdx.x < rt.blocks) dmq_router_wg(rt, blockIdx.x, mat);
-  else dmq_rotate_wg<MODE, 1>(p, (int)blockIdx.x - rt.blocks, mat);
+  else dmq_rotate_wg<MODE, 1, true>(p, (int)blockIdx.x - rt.blocks, mat);
 }
 
 // Quantization of activations that are already rotated (no matrix product): one wave per
@@ -418,6 +420,11 @@ static int launch_rotate(const RotParams& p_in, long tiled_waves, int tt, hipStr
   if (total > 0x7fffffffL) return DMQ_ERR_LIMIT;
   const int grid = (int)total;
   if (grid <= 0) return DMQ_OK;
+  if (p.pn.on) {                       // pre-norm rows: whole-batch pools, 16-row tiles, no top-k part
+    if (tt != 1 || tp || tiled_wgs > 0) return DMQ_ERR_MODE;
+    hipLaunchKernelGGL((dmq_rotate_kernel<MODE, 1, true>), dim3(grid), dim3(256), 0, stream, p);
+    return dmq_check_launch();
+  }
   if (tp) {
     auto go = [&](auto tt_tag) {
       constexpr int T_ = decltype(tt_tag)::value;

@@ -256,7 +256,6 @@ def measure_prenorm(mods, tokens, steps, warmup, seed, variants=64):
     hs = [(torch.randn(tokens, hdim, generator=g) * 2.0).half().cuda() for _ in range(variants)]
     for m in mods:
         m.gate_weight = wg
-        m._gate_f16 = None
     n, v = len(mods), len(hs)
 
     def fused(s):

@@ -126,6 +126,7 @@ class WxA16BitPartitionedGroupMoE:
         self._desc = None
         self._workspace = None
         self._gate_f16 = None       # fp16 copy of gate_weight and the state word of forward_prenorm
+        self._gate_src = None
         self._prenorm_state = None
         self.tt_override = 0        # activation tiles of 16 rows per wave (0 = pick from tokens)
         self.ks_override = 0        # waves splitting K inside a workgroup (0 = pick from tt)
@@ -517,8 +518,10 @@ class WxA16BitPartitionedGroupMoE:
         if norm_weight.dtype not in (torch.float16, torch.float32):
             norm_weight = norm_weight.float()
         norm_weight = norm_weight.to(h.device).contiguous()
-        if self._gate_f16 is None:
+        if self._gate_f16 is None or self._gate_src is not self.gate_weight:
+            self._gate_src = self.gate_weight          # a new gate_weight tensor refreshes the copy
             self._gate_f16 = self.gate_weight.to(device=h.device, dtype=torch.float16).contiguous()
+        if self._prenorm_state is None:
             self._prenorm_state = torch.zeros(64, dtype=torch.int32, device=h.device)
         router = RouterArgs()
         router.renorm = int(self.renormalize)

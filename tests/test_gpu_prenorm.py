@@ -93,6 +93,13 @@ def test_prenorm_forward_twice_and_beyond_the_limit(small_layer):
     torch.cuda.synchronize()
     assert torch.equal(a, b) and torch.equal(a[:2], c)
     assert int(mod._prenorm_state.abs().sum()) == 0
+    # a replaced gate weight is picked up (the module keeps an fp16 copy of it)
+    wg2 = wg.flip(0).contiguous()
+    mod.gate_weight = wg2.cuda()
+    lg = torch.empty(6, small_layer.num_experts, dtype=torch.float16, device="cuda")
+    _o, xn6 = mod.forward_prenorm(h.cuda(), wn.cuda(), EPS, return_normed=True, logits_out=lg)
+    torch.testing.assert_close(lg.float().cpu(), xn6.float().cpu() @ wg2.float().t(), rtol=2e-3, atol=2e-3)
+    mod.gate_weight = wg.cuda()
     h40, _wn, _wg = _case(small_layer, 40, 6)
     out, xn = mod.forward_prenorm(h40.cuda(), wn.cuda(), EPS, return_normed=True)
     want = mod.forward(xn, router_logits=torch.matmul(xn, wg.cuda().t()))

@@ -132,3 +132,34 @@ def test_prenorm_entry_rejects_what_it_does_not_take(small_layer):
         ctypes.byref(desc), ctypes.byref(router), ctypes.byref(pre), hd.data_ptr(), 4, None,
         out.data_ptr(), ws.data_ptr(), ws.numel(), 0, 0, 0, None, None, None)
     assert rc != 0                                             # no state word
+
+
+@pytest.mark.parametrize("tokens", [2, 7])
+def test_prenorm_forward_is_graph_capturable(small_layer, tokens):
+    """The pre-norm forward allocates nothing, never synchronises and leaves its state word zero,
+    so it can be captured in a HIP graph: every replay, with eager work of the same module in
+    between, reproduces the eager result bit for bit."""
+    h, wn, wg = _case(small_layer, tokens, 40 + tokens)
+    mod = make_module(small_layer, "wxa8")
+    mod.gate_weight = wg.cuda()
+    hd, wnd = h.cuda(), wn.cuda()
+    ref = mod.forward_prenorm(hd, wnd, EPS, fused=True).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            mod.forward_prenorm(hd, wnd, EPS, fused=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = mod.forward_prenorm(hd, wnd, EPS, fused=True)
+    for _ in range(4):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, ref)
+        other = mod.forward_prenorm(hd.flip(0).contiguous(), wnd, EPS, fused=True)
+        torch.cuda.synchronize()
+        assert torch.equal(other.flip(0), ref)
+    assert int(mod._prenorm_state.abs().sum()) == 0

@@ -60,7 +60,7 @@ static inline int pick_nbl(long rows, int tt) {
 
 extern "C" {
 
-int dmq_abi_version(void) { return 20; }
+int dmq_abi_version(void) { return 21; }
 
 const char* dmq_status_string(int status) {
   switch (status) {
@@ -431,6 +431,16 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
   p.split_rows = a->split_rows;
   p.split_partial = (float*)a->split_partial;
   p.split_counter = (int*)a->split_counter;
+  if (a->gemv) {
+    if (a->mode != DMQ_MODE_A16 || a->tt != 1 || ks != 1 || wsplit > 1 || mode2 >= 0 || a->dbg_acc ||
+        a->width_filter != 0 || a->accumulate || rows_kernel)
+      return DMQ_ERR_MODE;
+    if (a->epi != DMQ_EPI_SILU && a->epi != DMQ_EPI_SCATTER) return DMQ_ERR_MODE;
+    for (int i = 0; i < a->n_pools; ++i)
+      if (a->pool[i].mode == DMQ_MODE_A16 && a->pool[i].bit > 4) return DMQ_ERR_BIT;
+    if (!dmq_gemv_shape_ok(a->groups, a->n_out)) return DMQ_ERR_SHAPE;
+    return dmq_gemv_launch(p, a->epi == DMQ_EPI_SILU, a->max_items, (hipStream_t)stream);
+  }
   L.epi = a->epi;
   L.tt = a->tt;
   L.nt = one_tile ? 1 : 4;

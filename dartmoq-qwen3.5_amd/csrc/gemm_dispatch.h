@@ -123,3 +123,7 @@ int dmq_gemm_launch_fp4(const GemmLaunch& L);
 // persistent launch over work items of 128 rows, fp16 pools of 1/2/4-bit indices (gemm_rows.h);
 // nbl: feature blocks per unit; queue: DMQ_ROWS_QUEUE_WORDS zeroed device words
 int dmq_gemm_rows_launch(const GemmParams& p, int epi, int* queue, int nbl, hipStream_t stream);
+
+// dot-product launch for work items of at most four rows (csrc/gemv.hip)
+bool dmq_gemv_shape_ok(int groups, int n_out);
+int dmq_gemv_launch(const GemmParams& p, int silu, int max_items, hipStream_t stream);

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdartmoq_hip.so")
 
 OK = 0
-ABI_VERSION = 20
+ABI_VERSION = 21
 MAX_POOLS = 4
 MODE_A16, MODE_A8, MODE_FP8, MODE_FP4 = 0, 1, 2, 3
 EPI_STORE, EPI_SILU, EPI_SCATTER, EPI_SILU_ROT = 0, 1, 2, 3
@@ -52,7 +52,7 @@ class GemmArgs(Structure):
         ("item_tile_rows", c_int),
         ("nt", c_int),
         ("width_filter", c_int), ("home_filter", c_int), ("accumulate", c_int), ("roomy", c_int), ("spread", c_int), ("mode2_on", c_int), ("mode2", c_int), ("widths_apart", c_int),
-        ("rows_queue", c_void_p), ("k_split_items", c_int),
+        ("rows_queue", c_void_p), ("k_split_items", c_int), ("gemv", c_int),
     ]
 
 

@@ -305,7 +305,7 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, k_split_items=0, rows_total=None,
-                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None, widths_apart=0):
+                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None, widths_apart=0, gemv=False):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
     out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 (plain-store
@@ -314,7 +314,9 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     routed row indices and ``split_ws`` = (fp32 planes, zeroed int32 counters) may bring the
     scratch tensors in (allocated per call otherwise).  ``nt`` = 1: one n-tile per wave (plain
     store, tt = 1, ks = 4; any bit width): the launch of a Linear with a handful of rows.  ``item_tile_rows``: rows per work item
-    when the list was built for a larger tile than 16 * tt."""
+    when the list was built for a larger tile than 16 * tt.  ``gemv``: work items of at most four
+    rows as dot products on the vector ALU (fp16 activations, 1/2/4-bit pools, SiLU or scatter
+    epilogue)."""
     a = GemmArgs()
     a.mode, a.epi, a.tt, a.ks, a.nbl, a.n_pools = mode, epi, tt, ks, nbl, len(pools)
     dev = None
@@ -358,6 +360,7 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.mode2_on = 0 if mode2 is None else 1
     a.mode2 = 0 if mode2 is None else int(mode2)
     a.widths_apart = int(widths_apart)
+    a.gemv = int(bool(gemv))
     if tt == ROWS_TT:       # the persistent launch over 128-row work items: its queue words start at zero
         rows_queue = torch.zeros(16, dtype=torch.int32, device=dev)
         a.rows_queue = rows_queue.data_ptr()
@@ -384,7 +387,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
                   tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0, split_ws=None, nt=0,
-                  roomy=0, spread=0, widths_apart=0):
+                  roomy=0, spread=0, widths_apart=0, gemv=False):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -405,7 +408,8 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         out_stride=out_stride if out_stride is not None else out.stride(0),
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
                         dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total,
-                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy, spread=spread, widths_apart=widths_apart)
+                        item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy, spread=spread, widths_apart=widths_apart,
+                        gemv=gemv)
 
 
 def linear_gemm_i8(x_i8: torch.Tensor, x_scale: torch.Tensor, indices_gf: torch.Tensor,

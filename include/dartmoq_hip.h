@@ -51,7 +51,7 @@ enum { DMQ_EPI_STORE = 0, DMQ_EPI_SILU = 1, DMQ_EPI_SCATTER = 2, DMQ_EPI_SILU_RO
 #define DMQ_MAX_POOLS 4
 #define DMQ_ITEM_WORDS 8
 
-/* Library / build identification: returns the ABI version (currently 20). */
+/* Library / build identification: returns the ABI version (currently 21). */
 int dmq_abi_version(void);
 /* Human-readable text for a status code (static storage). */
 const char* dmq_status_string(int status);
@@ -328,6 +328,14 @@ typedef struct {
    * number written to n_items[1]): the launch then ends with the bulk instead of with them.
    * k_split_items bounds that number from the host; not with spread or item_tile_rows. */
   int k_split_items;
+  /* gemv != 0: work items of at most 4 rows each (a decode step of at most 4 tokens: one row per
+   * token and expert) run as dot products on the vector ALU instead of MFMA tiles: DMQ_MODE_A16,
+   * 1/2/4-bit pools, epi DMQ_EPI_SILU or DMQ_EPI_SCATTER, tt == 1, groups a multiple of 4 with
+   * groups / 4 in {1, 2, 4, 6, 8}, n_out % 16 == 0; no ks, k_split, mode2, dbg_acc, width_filter or
+   * accumulate.  Rows of an item beyond the fourth are not computed.  Same outputs as the MFMA
+   * launch up to the order of the fp32 sums (the norm multiplies the fp32 sum of a quarter group
+   * instead of the fp16 operand). */
+  int gemv;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

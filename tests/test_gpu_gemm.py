@@ -552,3 +552,71 @@ def test_work_items_larger_than_the_launch_tile(mode, tt, item_rows):
     assert torch.equal(own, big)
     with pytest.raises(ValueError):                 # not a multiple of the launch tile
         ops.matmul_merged(*args, item_tile_rows=48, **dict(kw, tt=2))
+
+
+@pytest.mark.parametrize("bit", [1, 2, 4])
+@pytest.mark.parametrize("k,inter", [(512, 128), (1024, 256), (2048, 512), (3072, 256), (4096, 128)])
+def test_dot_product_launch_for_a_few_rows_per_expert(bit, k, inter):
+    """Decode steps of at most four tokens: the vector-ALU launch (gemv) against the MFMA launch and
+    against fp32 maths, gate_up with SiLU * up and down with weight + scatter.  Experts with one to
+    four rows and an expert with none."""
+    from dartmoq_hip import ops
+    counts = [1, 4, 0, 2, 3, 1]
+    n_exp = len(counts)
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(100 + bit + k)
+    idx_gf, norms_gf, cb = _pool(bit, 2 * inter * n_exp, k, 7 + bit)
+    x = (torch.randn(rows_total, k, generator=g) * 0.5).half()
+    info = [(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(n_exp)]
+    info_dev = torch.tensor(info, dtype=torch.int32).cuda()
+    args = (A16, bit, SILU, x.cuda(), None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev)
+    common = dict(groups=k // 128, slice_is_groups=False, rows_total=rows_total, tt=1, n_out=inter,
+                  half_width=inter)
+    mfma = ops.matmul_merged(*args, **common).float().cpu()
+    got = ops.matmul_merged(*args, gemv=True, **common).float().cpu()
+    w = (cb.float()[packing.unpack_nbit(idx_gf, bit, 128).long()] * norms_gf.float().unsqueeze(-1))
+    ref = torch.zeros(rows_total, inter)
+    for e, (ts, cnt, ss, sc) in enumerate(info):
+        we = w[:, ss:ss + sc].permute(1, 0, 2).reshape(sc, k)
+        gu = x[ts:ts + cnt].float() @ we.t()
+        ref[ts:ts + cnt] = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    scale = ref.abs().max().item()
+    torch.testing.assert_close(got, ref, rtol=2e-3, atol=2e-3 * scale)
+    torch.testing.assert_close(got, mfma, rtol=4e-3, atol=4e-3 * scale)
+
+    # down: K = k again (groups of the expert's slice), n_out = 256 features, scattered
+    hidden, top_k = 256, 1
+    didx, dnorms, dcb = _pool(bit, hidden, k * n_exp, 9 + bit)
+    a = (torch.randn(rows_total, k, generator=g) * 0.5).half()
+    dinfo = [(starts[e], counts[e], e * (k // 128), k // 128) for e in range(n_exp)]
+    dinfo_dev = torch.tensor(dinfo, dtype=torch.int32).cuda()
+    slot = torch.randperm(rows_total, generator=g).int()
+    wts = torch.rand(rows_total, generator=g)
+    dargs = (A16, bit, SCATTER, a.cuda(), None, didx.cuda(), dnorms.cuda(), dcb.cuda(), dinfo_dev)
+    dcommon = dict(groups=k // 128, n_out=hidden, slice_is_groups=True, rows_total=rows_total, tt=1,
+                   out_stride=hidden, row_weight=wts.cuda(), row_slot=slot.cuda())
+    outs = []
+    for gemv in (False, True):
+        slots = torch.full((rows_total, hidden), float("nan"), dtype=torch.float16, device="cuda")
+        ops.matmul_merged(*dargs, out=slots, gemv=gemv, **dcommon)
+        outs.append(slots.float().cpu())
+    dw = (dcb.float()[packing.unpack_nbit(didx, bit, 128).long()] * dnorms.float().unsqueeze(-1))
+    dref = torch.zeros(rows_total, hidden)
+    for e, (ts, cnt, ss, sc) in enumerate(dinfo):
+        we = dw[ss:ss + sc].permute(1, 0, 2).reshape(hidden, k)
+        dref[slot[ts:ts + cnt].long()] = (a[ts:ts + cnt].float() @ we.t()) * wts[ts:ts + cnt].unsqueeze(1)
+    dscale = dref.abs().max().item()
+    torch.testing.assert_close(outs[1], dref, rtol=2e-3, atol=2e-3 * dscale)
+    torch.testing.assert_close(outs[1], outs[0], rtol=4e-3, atol=4e-3 * dscale)
+
+
+def test_dot_product_launch_rejects_what_it_does_not_cover():
+    from dartmoq_hip import ops
+    bit, k, inter = 2, 640, 128                               # 5 groups: not a multiple of 4
+    idx_gf, norms_gf, cb = _pool(bit, 2 * inter, k, 3)
+    x = torch.zeros(1, k).half().cuda()
+    info_dev = torch.tensor([(0, 1, 0, 2 * inter)], dtype=torch.int32).cuda()
+    with pytest.raises(ValueError):
+        ops.matmul_merged(A16, bit, SILU, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev,
+                          groups=k // 128, slice_is_groups=False, rows_total=1, tt=1, n_out=inter,
+                          half_width=inter, gemv=True)

@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/dartmoq_hip.h but not exported"
     assert set(declared) == set(_lib.PROTOTYPES), "ctypes prototypes and header disagree"
-    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 20
+    assert lib.dmq_abi_version() == _lib.ABI_VERSION == 21
     assert lib.dmq_status_string(0) == b"ok"
     assert b"bit width" in lib.dmq_status_string(1)
 

@@ -215,16 +215,22 @@ def measure(mods, tokens, steps, warmup, seed, zipf, mode):
     roof = roofline_of(avg["gu_bytes"], avg["gu_flops"], gu_ms, mode)
     roof["traffic"] = None
     shared_k = f", K shared by {-aux['ks']} workgroups" if aux["ks"] < 0 else ""
-    roof.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={max(aux['ks'], 1)},"
-                       f"{'SILU_ROT' if fused else 'SILU'}> merged gate_up"
-                       f"{' + down rotation' if fused else ''}, nbl={min(aux['nbl'], 2)}{shared_k}",
-                launch_ms=gu_ms,
+    gemv = aux["tt"] == 0                        # at most four tokens: dot products on the vector ALU
+    gu_kernel = (f"dmq_gemm_gf_kernel<tt={aux['tt']},ks={max(aux['ks'], 1)},"
+                 f"{'SILU_ROT' if fused else 'SILU'}> merged gate_up"
+                 f"{' + down rotation' if fused else ''}, nbl={min(aux['nbl'], 2)}{shared_k}")
+    if gemv:
+        gu_kernel = f"dmq_gemv_kernel<{mod.hidden_size // 512},SILU> merged gate_up"
+    roof.update(kernel=gu_kernel, launch_ms=gu_ms,
                 algorithmic_bytes=avg["gu_bytes"], algorithmic_flops=avg["gu_flops"],
                 extra_bytes=avg["gu_extra_bytes"], extra_flops=avg["gu_extra_flops"],
                 distinct_experts=avg["distinct"], routed_rows=avg["rows"])
     dn_ms = stage_ms["merged_down"]
     roof_down = roofline_of(avg["dn_bytes"], avg["dn_flops"], dn_ms, mode)
-    roof_down.update(kernel=f"dmq_gemm_gf_kernel<tt={aux['down_tt']},SCATTER> merged down",
+    dn_kernel = f"dmq_gemm_gf_kernel<tt={aux['down_tt']},SCATTER> merged down"
+    if gemv:
+        dn_kernel = f"dmq_gemv_kernel<{mod.intermediate_size // 512},SCATTER> merged down"
+    roof_down.update(kernel=dn_kernel,
                      launch_ms=dn_ms, algorithmic_bytes=avg["dn_bytes"],
                      algorithmic_flops=avg["dn_flops"])
     return {

@@ -435,11 +435,18 @@ int dmq_matmul_merged_gf(const dmq_gemm_args* a, void* stream) {
     if (a->mode != DMQ_MODE_A16 || a->tt != 1 || ks != 1 || wsplit > 1 || mode2 >= 0 || a->dbg_acc ||
         a->width_filter != 0 || a->accumulate || rows_kernel)
       return DMQ_ERR_MODE;
-    if (a->epi != DMQ_EPI_SILU && a->epi != DMQ_EPI_SCATTER) return DMQ_ERR_MODE;
+    const bool rot = a->epi == DMQ_EPI_SILU_ROT, scatter = a->epi == DMQ_EPI_SCATTER;
+    if (!rot && !scatter && a->epi != DMQ_EPI_SILU) return DMQ_ERR_MODE;
     for (int i = 0; i < a->n_pools; ++i)
       if (a->pool[i].mode == DMQ_MODE_A16 && a->pool[i].bit > 4) return DMQ_ERR_BIT;
-    if (!dmq_gemv_shape_ok(a->groups, a->n_out)) return DMQ_ERR_SHAPE;
-    return dmq_gemv_launch(p, a->epi == DMQ_EPI_SILU, a->max_items, (hipStream_t)stream);
+    if (!dmq_gemv_shape_ok(a->groups, a->n_out, rot)) return DMQ_ERR_SHAPE;
+    const bool planes = rot || (scatter && a->gemv_planes > 0);
+    if (planes && (!a->split_partial || a->split_rows <= 0)) return DMQ_ERR_NULL;
+    if (scatter && a->gemv_planes > 8) return DMQ_ERR_LIMIT;
+    p.split_partial = planes ? (float*)a->split_partial : nullptr;
+    p.split_rows = a->split_rows;
+    p.wsplit = scatter ? a->gemv_planes : dmq_gemv_planes(a->groups);
+    return dmq_gemv_launch(p, !scatter, a->max_items, (hipStream_t)stream);
   }
   L.epi = a->epi;
   L.tt = a->tt;
@@ -915,13 +922,21 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
                  ((long)tokens * K + (long)E * DMQ_ROWS_TILE) * 2 * (H > I ? H : I) <= 0xffffffffL;
   for (int i = 0; i < P; ++i)
     rows_ok = rows_ok && layer->pool[i].mode == DMQ_MODE_A16 && layer->pool[i].bit != 8;
+  // A decode step of at most four tokens on an fp16 layer of 1/2/4-bit pools (every expert then has
+  // at most four rows): both GEMMs as dot products on the vector ALU (csrc/gemv.hip) unless the
+  // caller names a tiling.  The down input is rotated by a launch of its own.
+  bool gemv = tt <= 0 && ks == 0 && tokens <= DMQ_GEMV_MAX_TOKENS && layer->n_widths == 0 &&
+              dmq_gemv_shape_ok(H / DMQ_GS, I, 1) && dmq_gemv_shape_ok(I / DMQ_GS, H, 0);
+  for (int i = 0; i < P; ++i)
+    gemv = gemv && layer->pool[i].mode == DMQ_MODE_A16 && layer->pool[i].bit <= 4;
+  if (gemv) { tt = 1; ks = 1; }
   if (tt <= 0) {
     tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
     if (rows_ok && (long)tokens * K >= DMQ_ROWS_MIN_ROUTED) tt = DMQ_ROWS_TT;
   }
   if (tt == DMQ_ROWS_TT && !rows_ok) tt = 4;
   if (tt != 1 && tt != 2 && tt != 4 && tt != DMQ_ROWS_TT) return DMQ_ERR_MODE;
-  const bool ks_auto = ks == 0;
+  const bool ks_auto = ks == 0;            // (not for the dot-product launches: no K sharing)
   if (ks == 0) {
     ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
     // an 8-bit pool on the fp16 path (a shared expert with a 256-entry table) makes few, long work
@@ -993,7 +1008,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   int rc;
   if (aux_out) {
     long* aux = (long*)aux_out;
-    aux[0] = tt; aux[1] = wsplit_eff > 1 ? -wsplit_eff : ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
+    aux[0] = gemv ? 0 : tt; aux[1] = wsplit_eff > 1 ? -wsplit_eff : ks; aux[2] = (long)((uint8_t*)w.counts - (uint8_t*)workspace);
     aux[3] = w.max_items; aux[4] = (long)((uint8_t*)w.n_items - (uint8_t*)workspace);
     aux[5] = nbl;
   }
@@ -1056,7 +1071,9 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   // 196 -> 240, so beyond 1280 routed rows the widths keep their own launches).
   const bool widths_apart = tt != 1 || (long)tokens * K > 1280;
   bool fuse_rot[DMQ_MAX_POOLS];
-  for (int mi = 0; mi < n_modes; ++mi) fuse_rot[mi] = (ks == 1);
+  // (dot-product launches: the rotated rows travel as fp32 planes of partial sums)
+  const bool gemv_rot = gemv && (long)tokens * K <= w.split_rows;
+  for (int mi = 0; mi < n_modes; ++mi) fuse_rot[mi] = (ks == 1) && (!gemv || gemv_rot);
   if (aux_out) {
     // which pools get their SiLU*up rows rotated inside the gate_up launch (bit i: pool i)
     long mask = 0;
@@ -1283,6 +1300,10 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     if (dual && mode == DMQ_MODE_A16) continue;        // rides the main mode's launch
     dmq_gemm_args g{};
     g.mode = mode; g.epi = fuse_rot[mi] ? DMQ_EPI_SILU_ROT : DMQ_EPI_SILU;
+    g.gemv = gemv;
+    if (gemv_rot) { g.split_partial = w.split_partial; g.split_rows = w.split_rows; }
+    // (every record of such a step holds at least one routed row: no more than R of them)
+    if (gemv && R < g.max_items) g.max_items = (int)R;
     if (dual && mode == main_mode) { g.mode2_on = 1; g.mode2 = DMQ_MODE_A16; }
     // the gate_up blocks are four times as long as the down blocks (K = H against K = I) and end in
     // the rotation epilogue: more than two per workgroup costs more in balance than it saves
@@ -1372,7 +1393,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     if (aux_out && mi == 0) ((long*)aux_out)[7] = down_tt;
     d.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;
     d.widths_apart = widths_apart;
-    d.ks = ks; d.n_pools = P;
+    d.ks = ks; d.n_pools = P; d.gemv = gemv;
     d.nbl = (nbl_auto && down_tt != tt) ? pick_nbl((long)tokens * K, down_tt) : nbl;   // by its own tile count
     for (int i = 0; i < P; ++i) {
       const dmq_pool_desc& pd = layer->pool[i];
@@ -1387,6 +1408,11 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     d.out = w.slots; d.out_stride = H;
     d.row_weight = w.sorted_weights; d.row_slot = w.sorted_rows;
     d.rows_queue = w.rows_queue + DMQ_ROWS_QUEUE_WORDS;
+    if (gemv && R < d.max_items) d.max_items = (int)R;
+    if (gemv_rot) {
+      d.gemv_planes = dmq_gemv_planes(H / DMQ_GS);
+      d.split_partial = w.split_partial; d.split_rows = w.split_rows;
+    }
     if (!sub) {
       rc = dmq_matmul_merged_gf(&d, stream);
       if (rc) return rc;

@@ -52,7 +52,7 @@ class GemmArgs(Structure):
         ("item_tile_rows", c_int),
         ("nt", c_int),
         ("width_filter", c_int), ("home_filter", c_int), ("accumulate", c_int), ("roomy", c_int), ("spread", c_int), ("mode2_on", c_int), ("mode2", c_int), ("widths_apart", c_int),
-        ("rows_queue", c_void_p), ("k_split_items", c_int), ("gemv", c_int),
+        ("rows_queue", c_void_p), ("k_split_items", c_int), ("gemv", c_int), ("gemv_planes", c_int),
     ]
 
 

@@ -296,6 +296,12 @@ def pick_ks(tt: int, rows_total: int) -> int:
     return 4 if (tt == 1 and rows_total <= 16) else 1
 
 
+def gemv_plane_count(groups: int) -> int:
+    """Planes a rotating dot-product gate_up launch over ``groups`` groups of 128 writes."""
+    nit = groups // 4
+    return 128 // (16 * (1 if nit >= 4 else 4 // max(nit, 1)))
+
+
 def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=None, w_scale_byte=127):
     """One pool entry of a merged launch (a dict of device tensors and scalars)."""
     return dict(mode=mode, bit=bit, act=act, act_scale=act_scale, w=w, norms=norms, lut=lut,
@@ -305,7 +311,8 @@ def gemm_pool(mode, bit, act, act_scale, w, norms, lut, expert_info, row_index=N
 def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, slice_is_groups,
                  tt, ks=0, nbl=0, out, out_stride, half_width=0, act_row_bytes=None, act_scale_stride=None,
                  row_weight=None, row_slot=None, dbg_acc=None, post=None, k_split=0, k_split_items=0, rows_total=None,
-                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None, widths_apart=0, gemv=False):
+                 item_tile_rows=0, split_ws=None, nt=0, roomy=0, spread=0, mode2=None, widths_apart=0, gemv=False,
+                 gemv_planes=None):
     """Merged dequant-GEMM launch over up to four pools sharing one work-item list.  ``post``
     (EPI_SILU_ROT) = dict(rot=[per-pool fp16 rotation matrices], extra=[per-pool scale factors],
     out=codes tensor [rows, *], scale=scale tensor or None).  ``k_split`` = 2 or 4 (plain-store
@@ -315,8 +322,8 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     scratch tensors in (allocated per call otherwise).  ``nt`` = 1: one n-tile per wave (plain
     store, tt = 1, ks = 4; any bit width): the launch of a Linear with a handful of rows.  ``item_tile_rows``: rows per work item
     when the list was built for a larger tile than 16 * tt.  ``gemv``: work items of at most four
-    rows as dot products on the vector ALU (fp16 activations, 1/2/4-bit pools, SiLU or scatter
-    epilogue)."""
+    rows as dot products on the vector ALU (fp16 activations, 1/2/4-bit pools; SiLU, scatter, or,
+    with ``gemv_planes``, SiLU + down rotation handed to the scatter launch as fp32 planes)."""
     a = GemmArgs()
     a.mode, a.epi, a.tt, a.ks, a.nbl, a.n_pools = mode, epi, tt, ks, nbl, len(pools)
     dev = None
@@ -361,6 +368,17 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
     a.mode2 = 0 if mode2 is None else int(mode2)
     a.widths_apart = int(widths_apart)
     a.gemv = int(bool(gemv))
+    if gemv and gemv_planes is not None:
+        # fp32 planes [n_planes, rows, width] of partial sums of the rotated SiLU*up rows: written by
+        # the gate_up launch (EPI_SILU_ROT, width = n_out), read by the down launch (EPI_SCATTER,
+        # width = 128 * groups)
+        if gemv_planes.dtype != torch.float32 or gemv_planes.dim() != 3 or not gemv_planes.is_contiguous():
+            raise TypeError("gemv_planes must be a contiguous float32 tensor [planes, rows, width]")
+        width = 128 * groups if epi == EPI_SCATTER else n_out
+        if gemv_planes.shape[2] != width or gemv_planes.shape[0] < (1 if epi == EPI_SCATTER else gemv_plane_count(groups)):
+            raise ValueError("gemv_planes does not fit this launch")
+        a.split_partial, a.split_rows = gemv_planes.data_ptr(), gemv_planes.shape[1]
+        a.gemv_planes = gemv_planes.shape[0] if epi == EPI_SCATTER else 0
     if tt == ROWS_TT:       # the persistent launch over 128-row work items: its queue words start at zero
         rows_queue = torch.zeros(16, dtype=torch.int32, device=dev)
         a.rows_queue = rows_queue.data_ptr()
@@ -387,7 +405,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                   slice_is_groups, rows_total, out=None, out_stride=None, half_width=0,
                   row_index=None, w_scale_byte=127, row_weight=None, row_slot=None, tt=None, ks=0, nbl=0,
                   tiling=None, dbg_acc=None, post=None, k_split=0, item_tile_rows=0, split_ws=None, nt=0,
-                  roomy=0, spread=0, widths_apart=0, gemv=False):
+                  roomy=0, spread=0, widths_apart=0, gemv=False, gemv_planes=None):
     """One-pool merged dequant GEMM.  ``expert_info`` is an int32 device tensor [E, 4]."""
     _need_cuda(act, w, norms, expert_info)
     _check_bit(bit, (1, 2, 4, 8))
@@ -409,7 +427,7 @@ def matmul_merged(mode, bit, epi, act, act_scale, w, norms, lut, expert_info, *,
                         half_width=half_width, row_weight=row_weight, row_slot=row_slot,
                         dbg_acc=dbg_acc, post=post, k_split=k_split, rows_total=rows_total,
                         item_tile_rows=item_tile_rows, split_ws=split_ws, nt=nt, roomy=roomy, spread=spread, widths_apart=widths_apart,
-                        gemv=gemv)
+                        gemv=gemv, gemv_planes=gemv_planes)
 
 
 def linear_gemm_i8(x_i8: torch.Tensor, x_scale: torch.Tensor, indices_gf: torch.Tensor,

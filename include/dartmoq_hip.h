@@ -330,12 +330,21 @@ typedef struct {
   int k_split_items;
   /* gemv != 0: work items of at most 4 rows each (a decode step of at most 4 tokens: one row per
    * token and expert) run as dot products on the vector ALU instead of MFMA tiles: DMQ_MODE_A16,
-   * 1/2/4-bit pools, epi DMQ_EPI_SILU or DMQ_EPI_SCATTER, tt == 1, groups a multiple of 4 with
-   * groups / 4 in {1, 2, 4, 6, 8}, n_out % 16 == 0; no ks, k_split, mode2, dbg_acc, width_filter or
+   * 1/2/4-bit pools, tt == 1, groups a multiple of 4 with groups / 4 in {1, 2, 4, 6, 8},
+   * n_out % 64 == 0 (16 from 16 groups on); no ks, k_split, mode2, dbg_acc, width_filter or
    * accumulate.  Rows of an item beyond the fourth are not computed.  Same outputs as the MFMA
    * launch up to the order of the fp32 sums (the norm multiplies the fp32 sum of a quarter group
-   * instead of the fp16 operand). */
+   * instead of the fp16 operand).  Epilogues:
+   *  DMQ_EPI_SILU      SiLU * up rows into out;
+   *  DMQ_EPI_SILU_ROT  (n_out % 128 == 0) the rotated SiLU * up rows as partial sums: fp32 planes
+   *                    [split_rows, n_out] in split_partial, 8 planes for groups >= 16, 4 for 8
+   *                    groups, 2 for 4 (out, post_out and split_counter are not used); the rotated
+   *                    row is the sum of the planes in plane order, rounded to fp16;
+   *  DMQ_EPI_SCATTER   as the MFMA launch; with gemv_planes > 0 the input rows are those sums of
+   *                    the first gemv_planes planes [split_rows, 128 * groups] of split_partial
+   *                    instead of the pools' act rows. */
   int gemv;
+  int gemv_planes;
 } dmq_gemm_args;
 
 /* Merged dequant GEMM: one launch for all 1/2/4-bit pools of a layer that share `mode`, one more

@@ -620,3 +620,74 @@ def test_dot_product_launch_rejects_what_it_does_not_cover():
         ops.matmul_merged(A16, bit, SILU, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev,
                           groups=k // 128, slice_is_groups=False, rows_total=1, tt=1, n_out=inter,
                           half_width=inter, gemv=True)
+
+
+@pytest.mark.parametrize("bit", [1, 2, 4])
+@pytest.mark.parametrize("k,inter", [(512, 512), (1024, 1024), (2048, 512), (3072, 128)])
+def test_dot_product_launch_with_the_down_rotation_fused(bit, k, inter):
+    """The dot-product gate_up launch hands the rotated input of the down projection over as fp32
+    planes of partial sums; the dot-product down launch adds them up.  The sum of the planes is the
+    stand-alone rotation of the launch's own SiLU*up rows up to the order of the fp32 sums, the
+    down launch fed with planes equals the down launch fed with that sum rounded to fp16 bit for
+    bit, and a second run gives the same bits."""
+    from dartmoq_hip import ops
+    from dartmoq_hip._lib import EPI_SILU_ROT
+    counts = [2, 0, 4, 1, 3]
+    n_exp = len(counts)
+    starts, rows_total = _expert_rows(counts)
+    g = torch.Generator().manual_seed(300 + bit + k)
+    idx_gf, norms_gf, cb = _pool(bit, 2 * inter * n_exp, k, 17 + bit)
+    x = (torch.randn(rows_total, k, generator=g) * 0.5).half()
+    info = [(starts[e], counts[e], e * 2 * inter, 2 * inter) for e in range(n_exp)]
+    info_dev = torch.tensor(info, dtype=torch.int32).cuda()
+    dinfo = [(starts[e], counts[e], e * (inter // 128), inter // 128) for e in range(n_exp)]
+    dinfo_dev = torch.tensor(dinfo, dtype=torch.int32).cuda()
+    rot = (torch.randn(n_exp * inter // 128, 128, 128, generator=g) / 128 ** 0.5).half().cuda()
+    tiling = ops.build_tiles(info_dev, rows_total, 16)
+    common = dict(groups=k // 128, n_out=inter, half_width=inter, slice_is_groups=False,
+                  rows_total=rows_total, tt=1, tiling=tiling, gemv=True)
+    tens = (x.cuda(), None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev)
+    silu = ops.matmul_merged(A16, bit, SILU, *tens, **common)
+    dn_tiling = ops.build_tiles(dinfo_dev, rows_total, 16)
+    dn_items, ditems, dmax = dn_tiling
+    want, _ = ops.rotate_tiled(A16, silu, rot, dinfo_dev, dn_items, ditems, 16, dmax, rows_total,
+                               rot_per_expert=True, extra_scale=1.0, tt=1)
+    n_planes = ops.gemv_plane_count(k // 128)
+    runs = []
+    for _ in range(2):
+        planes = torch.full((n_planes, rows_total, inter), float("nan"), device="cuda")
+        dummy = torch.empty((rows_total, inter), dtype=torch.float16, device="cuda")
+        ops.matmul_merged(A16, bit, EPI_SILU_ROT, *tens, out=dummy, out_stride=inter,
+                          post=dict(rot=[rot], extra=[1.0], out=dummy, scale=None),
+                          gemv_planes=planes, **common)
+        torch.cuda.synchronize()
+        runs.append(planes.clone())
+    assert torch.equal(runs[0].view(torch.int32), runs[1].view(torch.int32))
+    got = runs[0].sum(0)
+    scale = want.float().abs().max().item()
+    torch.testing.assert_close(got, want.float(), rtol=2e-3, atol=2e-3 * scale)
+
+    # the down launch: planes in, against the same launch fed with the fp16 sum of the planes
+    hidden = 256
+    didx, dnorms, dcb = _pool(bit, hidden, inter * n_exp, 19 + bit)
+    if not ops_gemv_ok(inter // 128):
+        return
+    summed = runs[0][0].clone()
+    for pl in range(1, n_planes):
+        summed += runs[0][pl]
+    slot = torch.randperm(rows_total, generator=g).int().cuda()
+    wts = torch.rand(rows_total, generator=g).cuda()
+    dargs = (A16, bit, SCATTER)
+    dtens = (None, didx.cuda(), dnorms.cuda(), dcb.cuda(), dinfo_dev)
+    dcommon = dict(groups=inter // 128, n_out=hidden, slice_is_groups=True, rows_total=rows_total, tt=1,
+                   out_stride=hidden, row_weight=wts, row_slot=slot, tiling=dn_tiling, gemv=True)
+    a = torch.full((rows_total, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    b = torch.full((rows_total, hidden), float("nan"), dtype=torch.float16, device="cuda")
+    ops.matmul_merged(*dargs, summed.half(), *dtens, out=a, **dcommon)
+    ops.matmul_merged(*dargs, dummy, *dtens, out=b, gemv_planes=runs[0], **dcommon)
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def ops_gemv_ok(groups):
+    return groups % 4 == 0 and groups // 4 in (1, 2, 4, 6, 8)

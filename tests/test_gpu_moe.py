@@ -550,3 +550,63 @@ def test_k_sharing_argument_errors(small_layer):
     mod.ks_override, mod.tt_override = -2, 2   # 16-row tiles only
     with pytest.raises(ValueError):
         mod.forward(x, topk_idx=idx, topk_w=w)
+
+
+@pytest.fixture(scope="module")
+def decode_layer():
+    """16 experts, H=1024 (8 groups), I=512 (4 groups), top-4, mixed 2/1/4-bit pools: group counts
+    the dot-product launches of a decode step cover."""
+    bits = moe.assign_bits(16, {2: 0.75, 1: 0.125, 4: 0.125}, seed=2)
+    return moe.build_layer(1024, 512, 16, 4, bits, seed=8)
+
+
+@pytest.mark.parametrize("tokens", [1, 2])
+@pytest.mark.parametrize("from_logits", [False, True])
+def test_single_token_decode_step_runs_as_dot_products(decode_layer, tokens, from_logits):
+    """wxa16, one token, no tiling named: gate_up and down run on the vector ALU (two tokens: MFMA
+    again).  Same bounds as the MFMA path, and the two agree to fp16 rounding."""
+    from dartmoq_hip.moe import forward_staged
+    layer = decode_layer
+    g = torch.Generator().manual_seed(60 + tokens)
+    x = torch.randn(tokens, layer.hidden, generator=g).half()
+    logits = routing.zipf_logits(tokens, layer.num_experts, 60 + tokens)
+    w, idx = routing.route_topk(logits, layer.top_k)
+    mod = make_module(layer, "wxa16")
+    kw = dict(router_logits=logits.cuda()) if from_logits else dict(topk_idx=idx.cuda().int(), topk_w=w.cuda())
+    out, _stats, aux = forward_staged(mod, x.cuda(), profile=False, **kw)
+    assert aux["tt"] == (0 if tokens == 1 else 1)             # 0: the dot-product launches ran
+    out = out.float().cpu()
+    mfma, _stats, aux_m = forward_staged(mod, x.cuda(), profile=False, tt=1, ks=1, **kw)
+    assert aux_m["tt"] == 1
+    mfma = mfma.float().cpu()
+    ideal = moe.quantized_forward(layer, x, idx, w, "wxa16")
+    ref = moe.reference_forward(layer, x, idx, w)
+    assert relerr(out, ideal) < 3e-3, relerr(out, ideal)
+    assert relerr(out, ref) < MODE_BOUND["wxa16"]
+    assert max_rel(out, ref) < 5e-3 and cosine(out, ref) >= 0.9999
+    assert relerr(out, mfma) < 2e-3, relerr(out, mfma)
+    # the module's own forward takes the same path
+    again = mod.forward(x.cuda(), **kw).float().cpu()
+    assert torch.equal(again, out)
+
+
+def test_decode_dot_products_with_shared_expert(decode_layer):
+    import dataclasses
+    layer = moe.add_shared_expert(dataclasses.replace(decode_layer, shared=None), 512, seed=78)
+    from dartmoq_hip.moe import forward_staged
+    mod = make_module(layer, "wxa16")
+    for tokens, want_tt in ((1, 0), (3, 1)):
+        g = torch.Generator().manual_seed(70 + tokens)
+        x = torch.randn(tokens, layer.hidden, generator=g).half()
+        logits = routing.zipf_logits(tokens, layer.num_experts, 70 + tokens)
+        w, idx = routing.route_topk(logits, layer.top_k)
+        out, _s, aux = forward_staged(mod, x.cuda(), profile=False, router_logits=logits.cuda())
+        assert aux["tt"] == want_tt
+        ideal = moe.quantized_forward(layer, x, idx, w, "wxa16")
+        assert relerr(out.float().cpu(), ideal) < 3e-3
+    # activation-quantized modes keep the MFMA path at any batch size
+    mod8 = make_module(decode_layer, "wxa8")
+    x = torch.randn(1, decode_layer.hidden, generator=torch.Generator().manual_seed(1)).half()
+    logits = routing.zipf_logits(1, decode_layer.num_experts, 1)
+    _o, _s, aux = forward_staged(mod8, x.cuda(), profile=False, router_logits=logits.cuda())
+    assert aux["tt"] == 1

@@ -125,7 +125,7 @@ int dmq_gemm_launch_fp4(const GemmLaunch& L);
 int dmq_gemm_rows_launch(const GemmParams& p, int epi, int* queue, int nbl, hipStream_t stream);
 
 // dot-product launch for work items of at most four rows (csrc/gemv.hip)
-#define DMQ_GEMV_MAX_TOKENS 1
+#define DMQ_GEMV_MAX_TOKENS 2
 bool dmq_gemv_shape_ok(int groups, int n_out, int rotate);
 int dmq_gemv_planes(int groups);
 int dmq_gemv_launch(const GemmParams& p, int silu, int max_items, hipStream_t stream);

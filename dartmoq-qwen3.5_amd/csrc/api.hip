@@ -922,11 +922,15 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
                  ((long)tokens * K + (long)E * DMQ_ROWS_TILE) * 2 * (H > I ? H : I) <= 0xffffffffL;
   for (int i = 0; i < P; ++i)
     rows_ok = rows_ok && layer->pool[i].mode == DMQ_MODE_A16 && layer->pool[i].bit != 8;
-  // A decode step of at most four tokens on an fp16 layer of 1/2/4-bit pools (every expert then has
-  // at most four rows): both GEMMs as dot products on the vector ALU (csrc/gemv.hip) unless the
-  // caller names a tiling.  The down input is rotated by a launch of its own.
+  // A decode step of one or two tokens on an fp16 layer of 1/2/4-bit pools: both GEMMs as dot
+  // products on the vector ALU (csrc/gemv.hip) unless the caller names a tiling -- while the gate_up
+  // launch (one workgroup per routed row and 16 features) is at most two workgroups per CU and its
+  // body keeps two workgroups' registers per CU (H <= 2048).  Measured: H=2048 I=512 top-8 one token
+  // 32.0 -> 25.7 us, two tokens 33.1 -> 32.1, three 35.4 -> 40.5; H=3072 I=1024 with a shared
+  // expert, one token 43.6 -> 52.0 (576 workgroups of 256 registers), so not there.
   bool gemv = tt <= 0 && ks == 0 && tokens <= DMQ_GEMV_MAX_TOKENS && layer->n_widths == 0 &&
-              dmq_gemv_shape_ok(H / DMQ_GS, I, 1) && dmq_gemv_shape_ok(I / DMQ_GS, H, 0);
+              dmq_gemv_shape_ok(H / DMQ_GS, I, 1) && dmq_gemv_shape_ok(I / DMQ_GS, H, 0) &&
+              H <= 2048 && (long)tokens * K * (I / 16) <= 2 * DMQ_GEMV_CUS;
   for (int i = 0; i < P; ++i)
     gemv = gemv && layer->pool[i].mode == DMQ_MODE_A16 && layer->pool[i].bit <= 4;
   if (gemv) { tt = 1; ks = 1; }

@@ -126,6 +126,7 @@ int dmq_gemm_rows_launch(const GemmParams& p, int epi, int* queue, int nbl, hipS
 
 // dot-product launch for work items of at most four rows (csrc/gemv.hip)
 #define DMQ_GEMV_MAX_TOKENS 2
+#define DMQ_GEMV_CUS 256          // compute units of an MI355X
 bool dmq_gemv_shape_ok(int groups, int n_out, int rotate);
 int dmq_gemv_planes(int groups);
 int dmq_gemv_launch(const GemmParams& p, int silu, int max_items, hipStream_t stream);

@@ -31,9 +31,10 @@ static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE
 static inline int pick_ks(int tt, long rows, int groups) {
   if (tt != 1) return 1;
   if (rows <= 16 && groups % 4 == 0) return -4;
-  // (24 groups and more: up to 144 rows, 16 tokens of top-8 plus a shared expert: H = 3072 wxa8
-  // 84.3 -> 81.4 us per forward; from 160 rows on one workgroup per block is ahead by 8 us)
-  if (rows <= (groups >= 24 ? 144 : 128) && groups % 2 == 0) return -2;
+  // (launch-shape tuner, weights from HBM: H = 2048 top-8, 32 / 64 / 128 rows 35.8 / 39.4 / 44.5 us
+  // per forward against 36.8 / 40.4 / 45.0 unshared; H = 3072 wxa8, 72 rows 57.2 against 56.8, 144
+  // rows 61.8 against 59.7, 288 rows 80.1 against 68.2)
+  if (rows <= 128 && groups % 2 == 0) return -2;
   return rows <= 16 ? 4 : 1;
 }
 
@@ -969,30 +970,11 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     ks = 1;
   }
   const int wsplit_eff = sub ? 1 : wsplit;
-  // Few long work items next to many short ones: with 16-row tiles every workgroup of the gate_up
-  // launch is resident from the start, so the launch ends with its slowest item.  The items of a
-  // pool that holds a small share of the experts (the 4-bit and 1-bit pools of a 2 bpw layer: twice
-  // the bytes per step, or a table that takes longer to build) are therefore shared by four
-  // workgroups each while the bulk keeps one per block (configs[3] wxa8 64 tokens: the 4-bit
-  // item ran 47 us, the 1-bit one 40, the median 2-bit one 30).
-  bool rare_pool[DMQ_MAX_POOLS] = {false, false, false, false};
-  int n_rare = 0, wsplit_launch = wsplit_eff;
-  long rare_items = 0;                                   // bound on the work items of those pools
-  if (ks_auto && wsplit_eff == 1 && !sub && tt == 1 && ks == 1 && (long)tokens * K <= DMQ_SPLIT_MAX_ROWS &&
-      tokens <= DMQ_HOIST_ALL_TOKENS) {
-    const int s = (H / DMQ_GS) % 4 == 0 ? 4 : ((H / DMQ_GS) % 2 == 0 ? 2 : 1);
-    for (int i = 0; i < P; ++i) {
-      const long members = layer->pool[i].n_gate_up / (2L * I);
-      rare_pool[i] = members * 8 <= E;
-      if (rare_pool[i]) {
-        ++n_rare;
-        const long by_tokens = members * ((tokens + 15) / 16), by_rows = members + (long)tokens * K / 16;
-        rare_items += by_tokens < by_rows ? by_tokens : by_rows;
-      }
-    }
-    if (s > 1 && n_rare > 0 && n_rare < P) wsplit_launch = s;
-    else { n_rare = 0; for (int i = 0; i < P; ++i) rare_pool[i] = false; }
-  }
+  // (dmq_gemm_args.k_split_items could share only the leading items of the list, say those of the
+  // pools with few, long items; with weights that come from HBM every such rule measured slower than
+  // one workgroup per block: configs[1] 32 tokens 45.9 against 43.5 us, configs[3] wxa8 48 tokens
+  // 82.6 against 72.0.)
+  const int wsplit_launch = wsplit_eff;
   if (tt == DMQ_ROWS_TT ? ks != 1 : !dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   const bool nbl_auto = nbl <= 0;
   if (nbl_auto) nbl = pick_nbl((long)tokens * K, tt > 4 ? 4 : tt);
@@ -1101,11 +1083,8 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   {
     int n = 0;
     for (int i = 0; i < P; ++i) if (!whole_batch[i]) pool_order[n++] = i;
-    // (every pool rotates by token when some pools' items share K, see rare_pool: the prefix then
-    // counts the items of those pools instead)
-    if (n_rare > 0) for (int i = 0; i < P; ++i) if (rare_pool[i]) pool_order[n++] = i;
     lead_pools = n;
-    for (int i = 0; i < P; ++i) if (whole_batch[i] && !rare_pool[i]) pool_order[n++] = i;
+    for (int i = 0; i < P; ++i) if (whole_batch[i]) pool_order[n++] = i;
     // Among the whole-batch pools the ones with the longest work items go first (the order of the
     // list is the order in which workgroups get their slots): 4-bit weights cost twice the look-ups
     // of 2-bit ones, fp16 activations more than quantized ones.  A 4-bit fp16 shared expert at the
@@ -1340,7 +1319,6 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     g.rows_queue = w.rows_queue;
     if (wsplit_launch > 1) {
       g.k_split = wsplit_launch; g.split_rows = w.split_rows;
-      if (n_rare > 0) g.k_split_items = (int)(rare_items < w.max_items ? rare_items : w.max_items);
       g.split_partial = w.split_partial; g.split_counter = w.split_counter;
     }
     if (!sub) {

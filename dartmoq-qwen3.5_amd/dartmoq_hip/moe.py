@@ -131,6 +131,7 @@ class WxA16BitPartitionedGroupMoE:
         self.tt_override = 0        # activation tiles of 16 rows per wave (0 = pick from tokens)
         self.ks_override = 0        # waves splitting K inside a workgroup (0 = pick from tt)
         self.nbl_override = 0       # feature blocks per workgroup of the GEMMs (0 = pick from tokens)
+        self.tile_table = None      # launch shapes by token count (dartmoq_hip.autotune.apply_config_table)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -439,6 +440,17 @@ class WxA16BitPartitionedGroupMoE:
             r.n_shared = self.n_shared
         return r, keep
 
+    def _tiling(self, tokens: int):
+        """(tt, ks, nbl) handed to the library: explicit overrides, else the tuned table's entry for
+        this batch size where the library accepts it, else zeros (the library's own choice)."""
+        if self.tt_override or self.ks_override or self.nbl_override or not self.tile_table:
+            return int(self.tt_override), int(self.ks_override), int(self.nbl_override)
+        from . import autotune
+        cfg = autotune.lookup_config(self.tile_table, tokens)
+        if not autotune.is_config_valid(cfg, tokens, self.top_k + self.n_shared, self.hidden_size):
+            return 0, 0, 0
+        return cfg["tt"], cfg["ks"], cfg["nbl"]
+
     @torch.no_grad()
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor | None = None,
                 topk_idx: torch.Tensor | None = None, topk_w: torch.Tensor | None = None,
@@ -463,7 +475,7 @@ class WxA16BitPartitionedGroupMoE:
         check(load().dmq_moe_ffn_forward_routed(
             ctypes.byref(desc), ctypes.byref(router), x.data_ptr(), tokens,
             None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-            int(self.tt_override), int(self.ks_override), int(self.nbl_override), None, None, stream),
+            *self._tiling(tokens), None, None, stream),
             "moe_ffn_forward_routed")
         del keep
         if orig_dtype != torch.float16:
@@ -549,7 +561,7 @@ class WxA16BitPartitionedGroupMoE:
         check(load().dmq_moe_ffn_forward_prenorm(
             ctypes.byref(desc), ctypes.byref(router), ctypes.byref(pre), h.data_ptr(), tokens,
             None if add is None else add.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(),
-            int(self.tt_override), int(self.ks_override), int(self.nbl_override), None, None, stream),
+            *self._tiling(tokens), None, None, stream),
             "moe_ffn_forward_prenorm")
         if orig_dtype != torch.float16:
             out = out.to(orig_dtype)

@@ -28,13 +28,16 @@ static inline bool valid_mode(int m) { return m >= DMQ_MODE_A16 && m <= DMQ_MODE
 // with at most 16 rows (negative value; the group count must divide).  Measured at H=2048 / 3072:
 // four-way wins up to 16 rows (1 token: 30.6 -> 28.7 us), two-way up to 128, none beyond.
 // Splitting K over the four waves of a workgroup instead only pays when the groups do not divide.
-static inline int pick_ks(int tt, long rows, int groups) {
+static inline int pick_ks(int tt, long rows, int groups, int weights = 0) {
   if (tt != 1) return 1;
   if (rows <= 16 && groups % 4 == 0) return -4;
   // (launch-shape tuner, weights from HBM: H = 2048 top-8, 32 / 64 / 128 rows 35.8 / 39.4 / 44.5 us
   // per forward against 36.8 / 40.4 / 45.0 unshared; H = 3072 wxa8, 72 rows 57.2 against 56.8, 144
   // rows 61.8 against 59.7, 288 rows 80.1 against 68.2)
-  if (rows <= 128 && groups % 2 == 0) return -2;
+  // layers of mostly 4-bit weights (weights != 0: twice the bytes per work item) up to 32 rows only:
+  // 64 rows 49.1 against 47.3 (fp16), 50.9 against 45.7 (FP4), 128 rows 76.4 against 66.3 and 73.6
+  // against 65.6
+  if (rows <= (weights == 0 ? 128 : 32) && groups % 2 == 0) return -2;
   return rows <= 16 ? 4 : 1;
 }
 
@@ -943,7 +946,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   if (tt != 1 && tt != 2 && tt != 4 && tt != DMQ_ROWS_TT) return DMQ_ERR_MODE;
   const bool ks_auto = ks == 0;            // (not for the dot-product launches: no K sharing)
   if (ks == 0) {
-    ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS);
+    ks = pick_ks(tt, (long)tokens * K, H / DMQ_GS, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
     // an 8-bit pool on the fp16 path (a shared expert with a 256-entry table) makes few, long work
     // items: two workgroups per block pay up to 256 routed rows (configs[3] with such a shared
     // expert, wxa16, 16 tokens: 88 -> 75 us; the int8 identity path gains nothing there)

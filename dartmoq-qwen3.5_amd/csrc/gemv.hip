@@ -302,8 +302,8 @@ bool dmq_gemv_shape_ok(int groups, int n_out, int rotate) {
 
 // planes a rotating gate_up launch over `groups` groups writes per block of 128 features
 int dmq_gemv_planes(int groups) {
-  const int nit = groups / 4;
-  return DMQ_GS / (16 * (nit >= 4 ? 1 : 4 / (nit > 0 ? nit : 1)));
+  const int fr = groups >= 16 ? 1 : (groups >= 8 ? 2 : 4);
+  return DMQ_GS / (16 * fr);
 }
 
 template <int NIT>

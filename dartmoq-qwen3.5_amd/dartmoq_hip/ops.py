@@ -377,6 +377,8 @@ def matmul_pools(mode, epi, pools, items, n_items, max_items, *, groups, n_out, 
         width = 128 * groups if epi == EPI_SCATTER else n_out
         if gemv_planes.shape[2] != width or gemv_planes.shape[0] < (1 if epi == EPI_SCATTER else gemv_plane_count(groups)):
             raise ValueError("gemv_planes does not fit this launch")
+        if rows_total is not None and gemv_planes.shape[1] < rows_total:
+            raise ValueError("gemv_planes holds fewer rows than the launch routes")
         a.split_partial, a.split_rows = gemv_planes.data_ptr(), gemv_planes.shape[1]
         a.gemv_planes = gemv_planes.shape[0] if epi == EPI_SCATTER else 0
     if tt == ROWS_TT:       # the persistent launch over 128-row work items: its queue words start at zero

@@ -18,6 +18,10 @@ A16, A8, FP8, FP4 = 0, 1, 2, 3
 STORE, SILU, SCATTER = 0, 1, 2
 
 
+def _gemv_groups_ok(groups):
+    return groups % 4 == 0 and groups // 4 in (1, 2, 4, 6, 8)
+
+
 def _pool(bit, n_rows, k, seed):
     """Random packed pool in group-first layout (indices, prescaled fp16 norms, codebook)."""
     g = torch.Generator().manual_seed(seed)
@@ -670,7 +674,7 @@ def test_dot_product_launch_with_the_down_rotation_fused(bit, k, inter):
     # the down launch: planes in, against the same launch fed with the fp16 sum of the planes
     hidden = 256
     didx, dnorms, dcb = _pool(bit, hidden, inter * n_exp, 19 + bit)
-    if not ops_gemv_ok(inter // 128):
+    if not _gemv_groups_ok(inter // 128):                    # the down launch covers 4, 8, 16, 24, 32 groups
         return
     summed = runs[0][0].clone()
     for pl in range(1, n_planes):
@@ -687,7 +691,3 @@ def test_dot_product_launch_with_the_down_rotation_fused(bit, k, inter):
     ops.matmul_merged(*dargs, dummy, *dtens, out=b, gemv_planes=runs[0], **dcommon)
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
-
-
-def ops_gemv_ok(groups):
-    return groups % 4 == 0 and groups // 4 in (1, 2, 4, 6, 8)

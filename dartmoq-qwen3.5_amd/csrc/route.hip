@@ -856,13 +856,17 @@ void dmq_route_rank_kernel(RouteRankParams p) {
   // slice of the expert in the first pool that holds one: in flight during the scan
   int pool = 0, ss = -1;
   if (valid) {
-    bool found = false;
+    // all pools' table entries are requested at once (one round trip), then the first pool wins
+    int sc[DMQ_MAX_POOLS], st[DMQ_MAX_POOLS];
 #pragma unroll
     for (int q = 0; q < DMQ_MAX_POOLS; ++q) {
-      if (q < p.pools && !found && p.slice_count_rows[q * p.experts + e] > 0) {
-        found = true; pool = q; ss = p.slice_start_rows[q * p.experts + e];
-      }
+      const int qq = q < p.pools ? q : 0;
+      sc[q] = p.slice_count_rows[qq * p.experts + e];
+      st[q] = p.slice_start_rows[qq * p.experts + e];
     }
+#pragma unroll
+    for (int q = DMQ_MAX_POOLS - 1; q >= 0; --q)
+      if (q < p.pools && sc[q] > 0) { pool = q; ss = st[q]; }
   }
   __syncthreads();
   // the list is read four experts at a time (one address for the whole wave: a broadcast)

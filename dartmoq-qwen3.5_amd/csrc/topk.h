@@ -262,13 +262,17 @@ __device__ __forceinline__ void dmq_topk_wg(const TopkParams& tp, int block) {
     // slices of the expert's pool (the first pool that holds a slice of it): requested before the scan
     int pool = 0, ss = -1;
     if (mine && my_e >= 0 && my_e < dp.experts) {      // a caller-made top-k may name no expert
-      bool found = false;
+      // all pools' table entries at once (one round trip), then the first pool wins
+      int sc[DMQ_MAX_POOLS], st[DMQ_MAX_POOLS];
 #pragma unroll
       for (int q = 0; q < DMQ_MAX_POOLS; ++q) {
-        if (q < dp.pools && !found && dp.slice_count_rows[q * dp.experts + my_e] > 0) {
-          found = true; pool = q; ss = dp.slice_start_rows[q * dp.experts + my_e];
-        }
+        const int qq = q < dp.pools ? q : 0;
+        sc[q] = dp.slice_count_rows[qq * dp.experts + my_e];
+        st[q] = dp.slice_start_rows[qq * dp.experts + my_e];
       }
+#pragma unroll
+      for (int q = DMQ_MAX_POOLS - 1; q >= 0; --q)
+        if (q < dp.pools && sc[q] > 0) { pool = q; ss = st[q]; }
     }
     int pos = 0, cnt = 0, before = 0;                 // before: rows of my expert ahead of mine
     for (int q = 0; q < rows4; ++q) {

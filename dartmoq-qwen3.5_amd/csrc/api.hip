@@ -37,13 +37,17 @@ static inline int pick_ks(int tt, long rows, int groups, int weights = 0) {
   // layers of mostly 4-bit weights (weights != 0: twice the bytes per work item) up to 32 rows only:
   // 64 rows 49.1 against 47.3 (fp16), 50.9 against 45.7 (FP4), 128 rows 76.4 against 66.3 and 73.6
   // against 65.6
-  if (rows <= (weights == 0 ? 128 : 32) && groups % 2 == 0) return -2;
+  // (the same search after the routing of 65-1024 rows went to the one-workgroup counting sort:
+  // H = 2048, 96 / 128 rows 41.2 / 41.5 against 40.7 / 40.9 unshared; H = 3072 wxa8, 72 / 108 rows
+  // 57.8 / 60.6 against 55.6 / 58.9: two ways up to 64 rows)
+  if (rows <= (weights == 0 ? 64 : 32) && groups % 2 == 0) return -2;
   return rows <= 16 ? 4 : 1;
 }
 
 // rows up to which the gate_up GEMM may share the K range of a block between workgroups (bounds
 // the fp32 scratch of the partial sums)
 #define DMQ_SPLIT_MAX_ROWS 1024
+#define DMQ_ROUTE_RANK_AUTO_ROWS 64
 // single-block workgroups at the end of every XCD's share of a GEMM launch that otherwise walks
 // several blocks per workgroup: one round of resident workgroups (32 CUs x 3)
 #define DMQ_DOWN_TT4_MIN_AVG 512
@@ -1208,14 +1212,16 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   {
     const int rk = K - n_shared, re = E - n_shared;          // the router's own k and experts
     const SharedGate sg{(const __half*)x, (const __half*)router->shared_gate_row, H, n_shared, pn, nullptr};
-    // up to DMQ_ROUTE_RANK_ROWS (128) routed rows with the top-k at hand: the one-row-per-thread ranking kernel
+    // a few routed rows with the top-k at hand: the one-row-per-thread ranking kernel.  Its scans
+    // grow with the square of the rows (kernel trace: 64 rows 5.7 us, 128 rows 9.1 us; the
+    // one-workgroup counting sort below takes 5.7 us at 256 rows), so it serves up to 64.
     const int* rank_idx = topk_done ? w.topk_idx
                                     : ((!router->logits && n_shared == 0) ? (const int*)router->topk_idx : nullptr);
     const float* rank_w = topk_done ? w.topk_w
                                     : ((!router->logits && n_shared == 0) ? (const float*)router->topk_w : nullptr);
     if (direct_done) {
       rc = DMQ_OK;
-    } else if (!sub && rank_idx && rank_w && R <= DMQ_ROUTE_RANK_ROWS && lead_pools == 0) {
+    } else if (!sub && rank_idx && rank_w && R <= DMQ_ROUTE_RANK_AUTO_ROWS && lead_pools == 0) {
       RouteRankParams rr{};
       rr.in_idx = rank_idx; rr.in_w = rank_w;
       rr.rows = (int)R; rr.k = K; rr.experts = E; rr.pools = P; rr.tile_rows = w.tile_rows;

@@ -624,6 +624,34 @@ def test_dot_product_launch_rejects_what_it_does_not_cover():
         ops.matmul_merged(A16, bit, SILU, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev,
                           groups=k // 128, slice_is_groups=False, rows_total=1, tt=1, n_out=inter,
                           half_width=inter, gemv=True)
+    # 8-bit pools, activation-quantized modes and 32-row tiles keep the MFMA launch
+    k = 512
+    idx_gf, norms_gf, cb = _pool(bit, 2 * inter, k, 3)
+    x = torch.zeros(1, k).half().cuda()
+    common = dict(groups=k // 128, slice_is_groups=False, rows_total=1, n_out=inter, half_width=inter, gemv=True)
+    idx8 = torch.zeros((k // 128, 2 * inter, 128), dtype=torch.uint8)
+    lut8 = (torch.arange(256).float() - 128).mul(3.0 / 128).half()
+    with pytest.raises(ValueError):
+        ops.matmul_merged(A16, 8, SILU, x, None, idx8.cuda(), norms_gf.cuda(), lut8.cuda(), info_dev, tt=1, **common)
+    with pytest.raises(ValueError):
+        ops.matmul_merged(A16, bit, SILU, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev, tt=2, **common)
+    codes = torch.zeros(1, k, dtype=torch.int8).cuda()
+    with pytest.raises(ValueError):
+        ops.matmul_merged(A8, bit, SILU, codes, torch.ones(1, k // 128).half().cuda(), idx_gf.cuda(),
+                          norms_gf.cuda(), torch.zeros(4, dtype=torch.int8).cuda(), info_dev, tt=1, **common)
+    # planes of the wrong width or too few planes
+    from dartmoq_hip._lib import EPI_SILU_ROT
+    rot = torch.zeros(1, 128, 128).half().cuda()
+    dummy = torch.empty((1, inter), dtype=torch.float16, device="cuda")
+    post = dict(rot=[rot], extra=[1.0], out=dummy, scale=None)
+    with pytest.raises(ValueError):
+        ops.matmul_merged(A16, bit, EPI_SILU_ROT, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev,
+                          tt=1, out=dummy, out_stride=inter, post=post,
+                          gemv_planes=torch.zeros(2, 1, 2 * inter, device="cuda"), **common)
+    with pytest.raises(ValueError):
+        ops.matmul_merged(A16, bit, EPI_SILU_ROT, x, None, idx_gf.cuda(), norms_gf.cuda(), cb.cuda(), info_dev,
+                          tt=1, out=dummy, out_stride=inter, post=post,
+                          gemv_planes=torch.zeros(1, 1, inter, device="cuda"), **common)
 
 
 @pytest.mark.parametrize("bit", [1, 2, 4])

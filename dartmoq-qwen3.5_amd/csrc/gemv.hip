@@ -1,5 +1,6 @@
 // Dequant GEMV for a handful of routed rows (fp16 activations, 1/2/4-bit pools): the gate_up and
-// down projections of a decode step of at most four tokens as dot products on the vector ALU.
+// down projections of a decode step of a few tokens (work items of at most four rows) as dot
+// products on the vector ALU.
 //
 // With one to four rows per expert an MFMA tile is 1/16 to 1/4 full and the 16-row GEMM spends
 // about four instructions per weight and lane on a work item that lives a few microseconds; here a
@@ -8,7 +9,8 @@
 // weights = 16 BIT / 4 bytes per lane and group; FR = 4 / 2 / 1 for K = 512 / 1024 / more, so
 // that a lane has at least four loads in flight), every load of the wave is requested before the
 // first is used, a packed byte is expanded through a small table (256 entries of 8 / BIT fp16
-// values, one copy) and multiplied with `v_dot2_f32_f16`, the norm is applied to the fp32 sum of a
+// values, several copies side by side: see GemvGeom) and multiplied with `v_dot2_f32_f16`, the norm
+// is applied to the fp32 sum of a
 // (group, quarter) and the sixteen partial sums of a feature meet in four cross-lane adds.  Same
 // work list, pools and outputs as dmq_gemm_gf_kernel with the SiLU resp. scatter epilogue (results
 // agree to fp32 summation order; the norm is not folded into an fp16 operand here).

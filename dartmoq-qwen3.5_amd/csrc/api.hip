@@ -984,7 +984,13 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   const int wsplit_launch = wsplit_eff;
   if (tt == DMQ_ROWS_TT ? ks != 1 : !dmq_gemm_config_ok(tt, ks)) return DMQ_ERR_MODE;
   const bool nbl_auto = nbl <= 0;
-  if (nbl_auto) nbl = pick_nbl((long)tokens * K, tt > 4 ? 4 : tt);
+  if (nbl_auto) {
+    nbl = pick_nbl((long)tokens * K, tt > 4 ? 4 : tt);
+    // layers of mostly 4-bit look-up weights: two blocks per workgroup from 512 routed rows on
+    // (launch-shape search, 64 / 256 / 1024 tokens of top-8: int8 106.2 / 115.4 / 174.5 us with one
+    // block against 103.6 / 113.1 / 168.9; fp16 64 / 512 tokens 100.6 / 134.6 against 99.3 / 130.0)
+    if (nbl < 2 && 2 * w4 > w_all && (long)tokens * K >= 512) nbl = 2;
+  }
   // a rotation wave covers 16 or 32 rows: 64-row work items are rotated by two waves each
   const int rot_tt = tt > 2 ? 2 : tt;
   MoeWorkspace w = carve(layer, tokens, tt, (uint8_t*)workspace);

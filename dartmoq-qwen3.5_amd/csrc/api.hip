@@ -50,7 +50,7 @@ static inline int pick_ks(int tt, long rows, int groups, int weights = 0) {
 #define DMQ_ROUTE_RANK_AUTO_ROWS 64
 // single-block workgroups at the end of every XCD's share of a GEMM launch that otherwise walks
 // several blocks per workgroup: one round of resident workgroups (32 CUs x 3)
-#define DMQ_DOWN_TT4_MIN_AVG 512
+#define DMQ_DOWN_TT4_MIN_AVG 256
 #define DMQ_TT4_MIN_AVG 112
 #define DMQ_HOIST_ALL_TOKENS 1024
 #define DMQ_TAIL_SLOTS 96
@@ -1385,7 +1385,11 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     // 64-row work items: the down GEMM (K = I, four steps per block) runs them as two 32-row tiles
     // until the experts are big enough for its 64-row kernel to pay
     const long avg_rows = (long)tokens * K / E;
-    const int down_tt = (tt == 4 && avg_rows < DMQ_DOWN_TT4_MIN_AVG) ? 2 : tt;
+    // (re-measured on weights from HBM, 64-row against 2 x 32-row: FP4 1024 / 2048 / 4096 tokens of
+    // the all-4-bit layer 135.9 / 189.5 / 287.4 against 137.9 / 192.7 / 293.1 us; int8 4096 tokens
+    // 409.9 against 414.9; fp16 2 bpw layer 4096 tokens 358.1 against 356.9, 8192 633.0 against 641.2)
+    const long down_min = 2 * wf4 > w_all ? 0 : DMQ_DOWN_TT4_MIN_AVG;
+    const int down_tt = (tt == 4 && avg_rows < down_min) ? 2 : tt;
     d.mode = mode; d.epi = DMQ_EPI_SCATTER; d.tt = down_tt; d.item_tile_rows = w.tile_rows; d.roomy = roomy;
     if (aux_out && mi == 0) ((long*)aux_out)[7] = down_tt;
     d.spread = ((n_modes > 1 && mode != main_mode) || (dual && tt > 1)) ? 1 : 0;

@@ -45,3 +45,32 @@ def test_search_times_the_shapes_and_the_table_drives_the_forward(small_layer, t
         assert torch.equal(out, want)
         ideal = moe.quantized_forward(small_layer, x, idx, w, "wxa16")
         assert relerr(out.float().cpu(), ideal) < 3e-3
+
+
+@pytest.mark.parametrize("tokens", [3, 300])
+def test_validity_filter_agrees_with_the_library(small_layer, tokens):
+    """Every shape of the search space: the library takes it exactly when the tuner's filter says so
+    (H = 256: K cannot be shared four ways; 1200 routed rows: not between workgroups at all)."""
+    from dartmoq_hip import autotune
+    mod = make_module(small_layer, "wxa16")
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(tokens, small_layer.hidden, generator=g).half().cuda()
+    logits = routing.zipf_logits(tokens, small_layer.num_experts, tokens).cuda()
+    want = mod.forward(x, router_logits=logits).float()
+    scale = want.abs().max().item()
+    seen = {True: 0, False: 0}
+    for cfg in autotune.generate_configs():
+        valid = autotune.is_config_valid(cfg, tokens, mod.top_k + mod.n_shared, mod.hidden_size)
+        mod.tt_override, mod.ks_override, mod.nbl_override = cfg["tt"], cfg["ks"], cfg["nbl"]
+        try:
+            out = mod.forward(x, router_logits=logits).float()
+            accepted = True
+        except ValueError:
+            accepted = False
+        finally:
+            mod.tt_override = mod.ks_override = mod.nbl_override = 0
+        assert accepted == valid, cfg
+        seen[valid] += 1
+        if accepted:                                   # any shape computes the same layer
+            torch.testing.assert_close(out, want, rtol=4e-3, atol=4e-3 * scale)
+    assert seen[True] > 10 and seen[False] > 10

@@ -48,6 +48,8 @@ static inline int pick_ks(int tt, long rows, int groups, int weights = 0) {
 // the fp32 scratch of the partial sums)
 #define DMQ_SPLIT_MAX_ROWS 1024
 #define DMQ_ROUTE_RANK_AUTO_ROWS 64
+// routed rows x feature blocks of the gate_up launch up to which 16-row tiles run the two-per-CU instance
+#define DMQ_TWO_PER_CU_MAX 4096
 // single-block workgroups at the end of every XCD's share of a GEMM launch that otherwise walks
 // several blocks per workgroup: one round of resident workgroups (32 CUs x 3)
 #define DMQ_DOWN_TT4_MIN_AVG 256
@@ -775,7 +777,7 @@ static inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // weights: 0 = mostly 1- and 2-bit pools, 1 = mostly 4-bit pools behind the look-up table,
 // 2 = mostly FP4 (e2m1 weights, no table)
-static int pick_tt(int tokens, int top_k, int experts, int weights) {
+static int pick_tt(int tokens, int top_k, int experts, int weights, bool two_per_cu = false) {
   const long avg = (long)tokens * top_k / (experts > 0 ? experts : 1);
   // 64-row work items halve the gate_up GEMM's look-ups per row (two workgroups per CU instead of
   // three) and, where an expert's rows fit one 64-row tile but not one 32-row tile, its tiles.
@@ -793,6 +795,13 @@ static int pick_tt(int tokens, int top_k, int experts, int weights) {
   // 92.8 -> 86.2; H = 3072, I = 1024 with a shared expert, wxa8: 64 tokens 108 -> 102, 128 tokens
   // 133 -> 128, 256 tokens 183 -> 164; at 1 row per expert 16-row tiles are 2-7 % ahead).
   if (weights == 0 ? avg < 2 : avg <= (weights == 1 ? 12 : 8)) return 1;
+  // Narrow pools, 3 rows per expert and more, while the launch is still small enough for the
+  // two-per-CU instance of the 16-row kernel: 32-row items then number a little more than the CUs,
+  // and the CUs that get two of them set the time of the launch.  H = 2048, I = 512, top-8, weights
+  // from HBM, 96 / 112 / 128 tokens: Zipf routing 57.0 / 57.5 / 58.2 us with 32-row items against
+  // 52.7 / 55.9 / 56.8; uniform routing 97.2 / 98.5 / 98.2 against 89.8 / 89.6 / 90.6 (at 64 and 80
+  // tokens Zipf has 32-row items 6 % ahead, uniform 16-row items 6 %: left with 32).
+  if (weights == 0 && two_per_cu && avg >= 3) return 1;
   return avg <= min4 ? 2 : 4;
 }
 
@@ -943,7 +952,8 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
     gemv = gemv && layer->pool[i].mode == DMQ_MODE_A16 && layer->pool[i].bit <= 4;
   if (gemv) { tt = 1; ks = 1; }
   if (tt <= 0) {
-    tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0));
+    tt = pick_tt(tokens, K, E, 2 * wf4 > w_all ? 2 : (2 * w4 > w_all ? 1 : 0),
+                 (long)tokens * K * (I / DMQ_GS) <= DMQ_TWO_PER_CU_MAX);
     if (rows_ok && (long)tokens * K >= DMQ_ROWS_MIN_ROUTED) tt = DMQ_ROWS_TT;
   }
   if (tt == DMQ_ROWS_TT && !rows_ok) tt = 4;
@@ -1058,7 +1068,7 @@ static int forward_routed_impl(const dmq_layer_desc* layer, const dmq_router_arg
   // I=512 up to 128 tokens, H=3072 I=1024 up to 32) and whenever most rows go to 4-bit weights.
   bool roomy = false;
   if (tt == 1) {
-    roomy = (long)tokens * K * (I / DMQ_GS) <= 4096;
+    roomy = (long)tokens * K * (I / DMQ_GS) <= DMQ_TWO_PER_CU_MAX;
     if (2 * w4 > w_all) roomy = true;
   }
 

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """MoE-layer throughput benchmark on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--tokens 2048] [--sweep 1,64] [--mode wxa16]
+    python bench.py --gpus 1 --steps K --warmup W [--tokens 2048] [--sweep 1,16,64,256,4096] [--mode wxa16]
 
 A step is one pass of the hot path (device top-k routing, permutation, rotation, gate_up
 dequant-GEMM + SiLU*up, per-expert rotation, down dequant-GEMM + scatter-add, fp16 store) over
@@ -424,7 +424,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--tokens", type=int, default=2048)
-    ap.add_argument("--sweep", type=str, default="1,64")
+    ap.add_argument("--sweep", type=str, default="1,16,64,256,4096")
     ap.add_argument("--config", type=int, default=1)
     ap.add_argument("--mode", type=str, default="wxa16", choices=list(MFMA_PEAK))
     ap.add_argument("--seed", type=int, default=42)

@@ -218,6 +218,8 @@ def main(argv=None) -> None:
     ap.add_argument("--copies", type=int, default=3)
     ap.add_argument("--repeat", type=int, default=10)
     ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--routing", default="config", choices=["config", "zipf", "uniform"],
+                    help="router logits: the configuration's own, Zipf(1.1)-biased, or unbiased")
     ap.add_argument("--output-dir", default="results/kernel_autotune")
     args = ap.parse_args(argv)
     sp = synthetic.CONFIGS[args.config]
@@ -233,7 +235,8 @@ def main(argv=None) -> None:
             pools, sp["experts"], sp["hidden"], sp["inter"], sp["top_k"], device="cuda", shared_expert=shared)
         mods.append(dartmoq_hip.convert_moe(m, args.mode))
     results = run_full_autotune(mods, [int(t) for t in args.tokens.split(",") if t], args.output_dir,
-                                skew=sp["zipf"], seed=args.seed, n_repeat=args.repeat)
+                                skew=sp["zipf"] if args.routing == "config" else args.routing == "zipf",
+                                seed=args.seed, n_repeat=args.repeat)
     for r in results:
         print_topk(r)
     table = generate_config_table(args.output_dir)
